@@ -1,0 +1,143 @@
+#!/usr/bin/env python3
+"""Benchmark of the k-NN hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--k 32] [--block-size 256]
+                    [--items-per-thread 16] [--sweep]
+
+A step is one bits top-k pass (through the C ABI) over a resident 1024 x 1,048,576 fp32 matrix
+of i.i.d. uniform [0,1) values (4 GiB, generated on the device).  The printed JSON line follows
+the reference's throughput convention: elements/s = rows*cols / mean step time
+(reference scripts/plot-kselection.py:161).  `roofline` prices the top-k kernel against HBM
+bandwidth with its algorithmic bytes (4 B read per matrix element + 8 B written per output pair)
+over the kernel's mean duration measured with events on the launch stream.  `cpu_baseline` times
+the CPU restatement of the reference's parallel top-k (reference src/topk/parallel_knn.cpp:30-65)
+on the host cores, on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "bits-knn-jpdc2024_amd"))
+
+HBM_PEAK_GBS = 8000.0  # MI355X published peak
+
+
+def topk_pass(bitsknn, torch, matrix, k, block, batch, prefetch, out_d, out_l, steps, warmup):
+    for _ in range(warmup):
+        bitsknn.topk_bits(matrix, k, block, batch, prefetch, out_dist=out_d, out_label=out_l)
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        bitsknn.topk_bits(matrix, k, block, batch, prefetch, out_dist=out_d, out_label=out_l)
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kernel_ms = sum(s.elapsed_time(e) for s, e in zip(starts, ends)) / steps
+    return wall / steps, kernel_ms / 1e3
+
+
+def cpu_baseline(rows, cols, k, budget_s=12.0):
+    """Reference CPU path (OpenMP heap per row) restated in oracle/, on config 1's matrix."""
+    import numpy as np
+    from oracle import binding as oracle
+    m = oracle.uniform_matrix(24, rows, cols)
+    threads = min(16, os.cpu_count() or 1)
+    reps, spent = 0, 0.0
+    oracle.topk_parallel(m, k, threads)  # warm
+    while spent < budget_s and reps < 50:
+        t0 = time.perf_counter()
+        _, _, used = oracle.topk_parallel(m, k, threads)
+        spent += time.perf_counter() - t0
+        reps += 1
+    return {"value": rows * cols * reps / spent, "unit": "elements/s", "cores": used, "kind": "port",
+            "sample": f"{reps} passes of parallel_knn::selection restated (OpenMP heap) over a "
+                      f"{rows}x{cols} fp32 uniform matrix, k={k}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--k", type=int, default=32)
+    ap.add_argument("--block-size", type=int, default=256)
+    ap.add_argument("--items-per-thread", type=int, default=16)
+    ap.add_argument("--no-prefetch", action="store_true")
+    ap.add_argument("--rows", type=int, default=1024)
+    ap.add_argument("--cols", type=int, default=1 << 20)
+    ap.add_argument("--sweep", action="store_true", help="also time k x block-size combinations")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (--gpus 1); multi-GPU figures are not "
+              "part of it", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import bitsknn
+    bitsknn.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(24)
+    rows, cols = args.rows, args.cols
+    matrix = torch.rand((rows, cols), device=dev, generator=gen)
+    prefetch = not args.no_prefetch
+
+    def run(k, block, batch, steps, warmup):
+        out_d = torch.empty((rows, k), dtype=torch.float32, device=dev)
+        out_l = torch.empty((rows, k), dtype=torch.int32, device=dev)
+        return topk_pass(bitsknn, torch, matrix, k, block, batch, prefetch, out_d, out_l, steps, warmup)
+
+    step_s, kernel_s = run(args.k, args.block_size, args.items_per_thread, args.steps, args.warmup)
+    bytes_alg = 4.0 * rows * cols + 8.0 * rows * args.k
+    achieved = bytes_alg / kernel_s / 1e9
+
+    result = {
+        "metric": "bits top-k selected-from elements/s (rows*cols / step time)",
+        "value": rows * cols / step_s,
+        "unit": "elements/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": step_s * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"bits top-k, fp32 matrix {rows}x{cols} uniform[0,1) resident in HBM, "
+                               f"k={args.k}, block {args.block_size}, items/thread {args.items_per_thread}, "
+                               f"prefetch {int(prefetch)}"},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel_ms": kernel_s * 1e3, "algorithmic_bytes": bytes_alg},
+    }
+
+    if args.sweep:
+        sweep = []
+        for k in (16, 32, 128, 512, 2048):
+            for block in (128, 256, 512):
+                if k // block > 16:
+                    continue
+                s, ks = run(k, block, args.items_per_thread, max(5, args.steps // 2), 3)
+                sweep.append({"k": k, "block": block, "elements_per_s": rows * cols / s,
+                              "hbm_frac": (4.0 * rows * cols + 8.0 * rows * k) / ks / 1e9 / HBM_PEAK_GBS})
+        result["sweep"] = sweep
+
+    del matrix
+    torch.cuda.empty_cache()
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(1024, 65536, 32)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,152 @@
+"""Thin ctypes binding of libbitsknn.so (the C ABI declared in include/bitsknn.h).
+
+Used by the parity tests and the benchmark to call the HIP kernels on torch-allocated device
+memory.  torch is plumbing here (device buffers, the current stream); every computation goes
+through the C ABI.  There is no CPU fallback: a missing library raises ImportError-like
+RuntimeError on first use, and every non-zero status raises BitsKnnError with the library's
+message.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "libbitsknn.so")
+
+OK, ERR_UNSUPPORTED, ERR_INVALID, ERR_HIP = 0, 1, 2, 3
+DIST_L2, DIST_PARTIAL_L2, DIST_EXPANDED = 0, 1, 2
+
+# every symbol include/bitsknn.h declares
+EXPORTS = (
+    "bitsknn_last_error",
+    "bitsknn_version",
+    "bitsknn_topk_bits_f32",
+    "bitsknn_label_offsets",
+    "bitsknn_fill_f32",
+    "bitsknn_dist_f32",
+    "bitsknn_fused_l2_topk_f32",
+)
+
+
+class BitsKnnError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(message)
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    """Load libbitsknn.so (built in-tree by `make -C bits-knn-jpdc2024_amd lib`)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `make -C {os.path.dirname(_HERE)} lib` "
+                "(there is no fallback path)")
+        L = ctypes.CDLL(LIB_PATH)
+        vp, sz, i32, u32 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int32, ctypes.c_uint32
+        L.bitsknn_last_error.restype = ctypes.c_char_p
+        L.bitsknn_last_error.argtypes = []
+        L.bitsknn_version.restype = ctypes.c_char_p
+        L.bitsknn_version.argtypes = []
+        L.bitsknn_topk_bits_f32.restype = ctypes.c_int
+        L.bitsknn_topk_bits_f32.argtypes = [vp, sz, vp, sz, vp, sz, sz, vp, vp, sz, u32, u32, u32,
+                                            ctypes.c_int, vp]
+        L.bitsknn_label_offsets.restype = ctypes.c_int
+        L.bitsknn_label_offsets.argtypes = [vp, sz, sz, sz, vp]
+        L.bitsknn_fill_f32.restype = ctypes.c_int
+        L.bitsknn_fill_f32.argtypes = [vp, sz, ctypes.c_float, vp]
+        L.bitsknn_dist_f32.restype = ctypes.c_int
+        L.bitsknn_dist_f32.argtypes = [ctypes.c_int, ctypes.c_int, sz, sz, vp, sz, vp, sz, vp, sz, vp]
+        L.bitsknn_fused_l2_topk_f32.restype = ctypes.c_int
+        L.bitsknn_fused_l2_topk_f32.argtypes = [vp, vp, ctypes.c_int, i32, i32, vp, vp, ctypes.c_int,
+                                                ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                ctypes.c_int, ctypes.c_int, vp]
+        _lib = L
+    return _lib
+
+
+def _check(status):
+    if status != OK:
+        raise BitsKnnError(status, lib().bitsknn_last_error().decode())
+
+
+def _stream():
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def version():
+    return lib().bitsknn_version().decode()
+
+
+def topk_bits(dist, k, block_size=256, items_per_thread=16, prefetch=False, in_label=None,
+              label_offsets=None, out_dist=None, out_label=None):
+    """bits top-k of every row of a 2-D float32 device tensor (last dim contiguous).
+    Returns (values, labels), each rows x k."""
+    import torch
+    assert dist.is_cuda and dist.dtype == torch.float32 and dist.dim() == 2 and dist.stride(1) == 1
+    rows, cols = dist.shape
+    if out_dist is None:
+        out_dist = torch.empty((rows, k), dtype=torch.float32, device=dist.device)
+    if out_label is None:
+        out_label = torch.empty((rows, k), dtype=torch.int32, device=dist.device)
+    label_stride = 0
+    if in_label is not None:
+        assert in_label.dtype == torch.int32 and in_label.shape == dist.shape and in_label.stride(1) == 1
+        label_stride = in_label.stride(0)
+    if label_offsets is not None:
+        assert label_offsets.dtype == torch.int32 and label_offsets.numel() == rows
+    _check(lib().bitsknn_topk_bits_f32(_ptr(dist), dist.stride(0) if rows > 1 else max(dist.stride(0), cols),
+                                       _ptr(in_label), label_stride, _ptr(label_offsets), rows, cols,
+                                       _ptr(out_dist), _ptr(out_label), out_dist.stride(0), k,
+                                       block_size, items_per_thread, 1 if prefetch else 0, _stream()))
+    return out_dist, out_label
+
+
+def label_offsets(rows, parts, cols_per_part, device="cuda"):
+    import torch
+    out = torch.empty(rows * parts, dtype=torch.int32, device=device)
+    _check(lib().bitsknn_label_offsets(_ptr(out), rows, parts, cols_per_part, _stream()))
+    return out
+
+
+def fill(t, value):
+    _check(lib().bitsknn_fill_f32(_ptr(t), t.numel(), float(value), _stream()))
+    return t
+
+
+def distances(queries_dm, points_dm, op=DIST_L2, out=None):
+    """Distance matrix q x n from dim-major inputs (d x q and d x n float32 device tensors)."""
+    import torch
+    d, q = queries_dm.shape
+    d2, n = points_dm.shape
+    assert d == d2 and queries_dm.stride(1) == 1 and points_dm.stride(1) == 1
+    if out is None:
+        out = torch.empty((q, n), dtype=torch.float32, device=queries_dm.device)
+    _check(lib().bitsknn_dist_f32(op, d, q, n, _ptr(queries_dm), queries_dm.stride(0),
+                                  _ptr(points_dm), points_dm.stride(0), _ptr(out), out.stride(0),
+                                  _stream()))
+    return out
+
+
+def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1, dim_mult=1,
+                  out_dist=None, out_label=None):
+    """bits-fused: top-k of ||p||^2 - 2 q.p without materialising the distance matrix."""
+    import torch
+    d, q = queries_dm.shape
+    d2, n = points_dm.shape
+    assert d == d2 and queries_dm.is_contiguous() and points_dm.is_contiguous()
+    if out_dist is None:
+        out_dist = torch.empty((q, k), dtype=torch.float32, device=queries_dm.device)
+    if out_label is None:
+        out_label = torch.empty((q, k), dtype=torch.int32, device=queries_dm.device)
+    _check(lib().bitsknn_fused_l2_topk_f32(_ptr(queries_dm), _ptr(points_dm), d, q, n,
+                                           _ptr(out_dist), _ptr(out_label), k, params[0], params[1],
+                                           params[2], block_query_dim, dim_mult, _stream()))
+    return out_dist, out_label

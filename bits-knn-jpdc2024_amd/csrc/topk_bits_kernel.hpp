@@ -1,0 +1,477 @@
+// bits top-k selection for gfx950 (wave64).
+//
+// One workgroup per matrix row.  The row is streamed from HBM in 16-byte loads; a value is kept
+// only if it is below the current k-th smallest value ("radius").  Kept values are appended as
+// 64-bit (value, label) keys to a buffer in LDS (one LDS atomic per wave and value slot, slots
+// assigned by ballot + lane prefix count).  When the buffer is full the whole workgroup sorts it
+// descending with a bitonic network held in registers, takes the element-wise minimum with the
+// ascending top-k list (a bitonic separator), re-sorts the resulting bitonic sequence and
+// publishes the new radius.
+//
+// Same algorithm and phases as the reference kernel
+// (include/bits/topk/singlepass/detail/bits_kernel.cuh:317-408: alloc :117-126, insert :277-302,
+// merge :145-199, radius :30-51), laid out for 64-wide waves: exchange distances below 64 lanes
+// stay inside a wave, only distances of 64 lanes and more go through LDS, and the per-batch
+// overflow vote is one LDS flag read after one barrier that does not wait for global loads.
+
+#ifndef BITSKNN_CSRC_TOPK_BITS_KERNEL_HPP_
+#define BITSKNN_CSRC_TOPK_BITS_KERNEL_HPP_
+
+#include "common.hpp"
+
+namespace bitsknn
+{
+
+typedef float vfloat4 __attribute__((ext_vector_type(4)));
+
+struct topk_args
+{
+    const float* in;
+    size_t in_stride;
+    const std::int32_t* in_label;
+    size_t label_stride;
+    const std::int32_t* label_offsets;
+    u32 cols;
+    float* out_dist;
+    std::int32_t* out_label;
+    size_t out_stride;
+    u32 k;
+};
+
+// Workgroup barrier that orders LDS traffic only, so that global loads issued earlier stay in
+// flight across it.
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+__device__ __forceinline__ u64 lane_xor(u64 x, int mask)
+{
+    const u32 lo = static_cast<u32>(__shfl_xor(static_cast<int>(static_cast<u32>(x)), mask, WAVE));
+    const u32 hi = static_cast<u32>(__shfl_xor(static_cast<int>(static_cast<u32>(x >> 32U)), mask, WAVE));
+    return (static_cast<u64>(hi) << 32U) | lo;
+}
+
+// One compare-exchange layer of a bitonic network over N = BS*IPT keys held IPT per thread in
+// blocked order (thread t owns sorted positions t*IPT .. t*IPT+IPT-1).  K2 is the size of the
+// sequences being merged in this phase, J the exchange distance.  DESC flips the final order.
+template <int BS, int IPT, int K2, int J, bool DESC>
+__device__ __forceinline__ void net_step(u64 (&x)[IPT], u64* scratch, int t)
+{
+    constexpr int N = BS * IPT;
+    if constexpr (J < IPT)
+    {
+        // both elements live in this thread
+#pragma unroll
+        for (int r = 0; r < IPT; ++r)
+        {
+            if ((r & J) == 0)
+            {
+                bool down = DESC;
+                if constexpr (K2 < IPT)
+                {
+                    down = (((r & K2) != 0) != DESC);
+                }
+                else if constexpr (K2 < N)
+                {
+                    down = (((t & (K2 / IPT)) != 0) != DESC);
+                }
+                const u64 a = x[r];
+                const u64 b = x[r | J];
+                const bool sw = (b < a) != down;
+                x[r] = sw ? b : a;
+                x[r | J] = sw ? a : b;
+            }
+        }
+    }
+    else
+    {
+        constexpr int M = J / IPT; // partner thread = t ^ M
+        bool down = DESC;
+        if constexpr (K2 < N)
+        {
+            down = (((t & (K2 / IPT)) != 0) != DESC);
+        }
+        const bool keep_min = (((t & M) == 0) != down);
+        if constexpr (M < WAVE)
+        {
+#pragma unroll
+            for (int r = 0; r < IPT; ++r)
+            {
+                const u64 o = lane_xor(x[r], M);
+                const bool take = (o < x[r]) == keep_min;
+                x[r] = take ? o : x[r];
+            }
+        }
+        else
+        {
+            // partner lives in another wave: exchange through LDS, striped so that neighbouring
+            // lanes touch neighbouring 8-byte slots
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < IPT; ++r)
+            {
+                scratch[r * BS + t] = x[r];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < IPT; ++r)
+            {
+                const u64 o = scratch[r * BS + (t ^ M)];
+                const bool take = (o < x[r]) == keep_min;
+                x[r] = take ? o : x[r];
+            }
+        }
+    }
+}
+
+template <int BS, int IPT, int K2, int J, bool DESC>
+__device__ __forceinline__ void net_phase(u64 (&x)[IPT], u64* scratch, int t)
+{
+    net_step<BS, IPT, K2, J, DESC>(x, scratch, t);
+    if constexpr (J > 1)
+    {
+        net_phase<BS, IPT, K2, J / 2, DESC>(x, scratch, t);
+    }
+}
+
+// full bitonic sort: phases K2 = 2, 4, ..., N
+template <int BS, int IPT, int K2, bool DESC>
+__device__ __forceinline__ void net_sort(u64 (&x)[IPT], u64* scratch, int t)
+{
+    net_phase<BS, IPT, K2, K2 / 2, DESC>(x, scratch, t);
+    if constexpr (K2 < BS * IPT)
+    {
+        net_sort<BS, IPT, K2 * 2, DESC>(x, scratch, t);
+    }
+}
+
+// Merge the first `limit` keys of the LDS buffer into the ascending top-k list.  The buffer
+// memory doubles as exchange scratch once its keys are in registers.
+template <int BS, int IPT>
+__device__ __forceinline__ void merge_buffer(u64 (&topk)[IPT], u64* buffer, int limit, int t)
+{
+    constexpr int N = BS * IPT;
+    u64 tmp[IPT];
+#pragma unroll
+    for (int r = 0; r < IPT; ++r)
+    {
+        const int idx = r * BS + t;
+        tmp[r] = idx < limit ? buffer[idx] : PAD_KEY;
+    }
+    // (the first LDS exchange of the sort starts with a barrier, so the loads above are done)
+    net_sort<BS, IPT, 2, true>(tmp, buffer, t);
+    // ascending list vs descending buffer: element-wise minimum keeps the N smallest of the 2N
+    // keys and leaves them as a bitonic sequence
+#pragma unroll
+    for (int r = 0; r < IPT; ++r)
+    {
+        topk[r] = tmp[r] < topk[r] ? tmp[r] : topk[r];
+    }
+    net_phase<BS, IPT, N, N / 2, false>(topk, buffer, t);
+}
+
+// value of sorted element k-1, broadcast to the whole workgroup (includes a barrier)
+template <int IPT>
+__device__ __forceinline__ float broadcast_radius(const u64 (&topk)[IPT], u32 k, float* slot, int t)
+{
+#pragma unroll
+    for (int r = 0; r < IPT; ++r)
+    {
+        if (static_cast<u32>(t * IPT + r) == k - 1)
+        {
+            *slot = key_value(topk[r]);
+        }
+    }
+    __syncthreads();
+    return *slot;
+}
+
+// BS threads, IPT list entries per thread, L 16-byte (or 4 x 4-byte when !VEC) loads in flight
+// per thread and iteration.
+//
+// The kernel is one loop around a single merge site: the first NL values of the row are written
+// to the buffer and merged into the empty list, every later overflow merges a full buffer, and
+// the end of the row merges whatever is left.
+template <int BS, int IPT, int L, bool VEC>
+__global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
+{
+    constexpr int NL = BS * IPT;     // length of the top-k list and of the buffer
+    constexpr int E = 4 * L;         // values per thread and iteration
+    constexpr u32 CHUNK = BS * E;    // values per workgroup and iteration
+    static_assert(E <= 32, "one pass bit per value in a 32-bit lane mask");
+
+    __shared__ u64 buffer[NL];
+    __shared__ int s_size;
+    __shared__ int s_flag[3];
+    __shared__ float s_radius;
+
+    const int t = static_cast<int>(threadIdx.x);
+    const int lane = t & (WAVE - 1);
+    const size_t row_idx = blockIdx.x;
+    const float* __restrict__ row = a.in + row_idx * a.in_stride;
+    const std::int32_t* __restrict__ lrow =
+        a.in_label != nullptr ? a.in_label + row_idx * a.label_stride : nullptr;
+    const u32 label_offset =
+        a.label_offsets != nullptr ? static_cast<u32>(a.label_offsets[row_idx]) : 0U;
+    const u32 n = a.cols;
+
+    auto label_of = [&](u32 col) -> std::int32_t {
+        const u32 base = lrow != nullptr ? static_cast<u32>(lrow[col]) : col;
+        return static_cast<std::int32_t>(base + label_offset);
+    };
+
+    // column of value j of this thread within a chunk
+    auto column_of = [&](u32 chunk, int j) -> u32 {
+        if constexpr (VEC)
+        {
+            return chunk + static_cast<u32>(((j / 4) * BS + t) * 4 + (j % 4));
+        }
+        else
+        {
+            return chunk + static_cast<u32>(j * BS + t);
+        }
+    };
+
+    u64 topk[IPT];
+#pragma unroll
+    for (int r = 0; r < IPT; ++r)
+    {
+        topk[r] = PAD_KEY;
+    }
+
+    const u32 first = n < static_cast<u32>(NL) ? n : static_cast<u32>(NL);
+    const u32 full_end =
+        n > static_cast<u32>(NL) ? static_cast<u32>(NL) + ((n - static_cast<u32>(NL)) / CHUNK) * CHUNK
+                                 : static_cast<u32>(NL);
+    u32 chunk = NL;
+
+    // the first NL values go straight to the buffer
+#pragma unroll
+    for (int r = 0; r < IPT; ++r)
+    {
+        const u32 col = static_cast<u32>(r * BS + t);
+        if (col < first)
+        {
+            buffer[col] = make_key(row[col], label_of(col));
+        }
+    }
+    if (t == 0)
+    {
+        s_size = static_cast<int>(first);
+        s_flag[0] = 0;
+        s_flag[1] = 0;
+        s_flag[2] = 0;
+    }
+    __syncthreads();
+
+    float radius = __builtin_inff();
+    int phase = 0;
+    bool merge_now = true;   // workgroup-uniform
+    int limit = static_cast<int>(first);
+    bool finished = false;
+    u32 cur_chunk = 0;       // first column of the chunk held in v[]
+
+    float v[E];
+#pragma unroll
+    for (int j = 0; j < E; ++j)
+    {
+        v[j] = 0.0F;
+    }
+
+    // Slot bookkeeping of the current chunk: bit j of my_pass says value j of this lane passed
+    // the filter; the passing lanes of value j were assigned consecutive slots from
+    // slot_base[j] (wave-uniform) in lane order.  slot_base drops by NL with every merge; a value
+    // is written in the round where its slot falls into [0, NL).
+    u32 my_pass = 0;
+    int slot_base[E];
+#pragma unroll
+    for (int j = 0; j < E; ++j)
+    {
+        slot_base[j] = 0;
+    }
+    bool wave_has_values = false;
+
+    auto write_slots = [&]() -> bool {
+        bool later = false;
+#pragma unroll
+        for (int j = 0; j < E; ++j)
+        {
+            const bool mine = ((my_pass >> j) & 1U) != 0;
+            const u64 mask = __builtin_amdgcn_ballot_w64(mine);
+            if (mask != 0)
+            {
+                const int count = __popcll(mask);
+                const int base = slot_base[j];
+                if (base < NL && base + count > 0)
+                {
+                    const int rank = static_cast<int>(__builtin_amdgcn_mbcnt_hi(
+                        static_cast<u32>(mask >> 32U),
+                        __builtin_amdgcn_mbcnt_lo(static_cast<u32>(mask), 0U)));
+                    const int slot = base + rank;
+                    if (mine && slot >= 0 && slot < NL)
+                    {
+                        const u32 col = column_of(cur_chunk, j);
+                        buffer[slot] = make_key(v[j], label_of(col));
+                    }
+                }
+                later |= (base + count > NL);
+            }
+        }
+        return later;
+    };
+
+    // workgroup-wide vote; three rotating flags keep the reset of a flag two barriers away from
+    // its last read
+    auto vote = [&](bool wave_pred) -> bool {
+        const int c = phase;
+        const int nx = c == 2 ? 0 : c + 1;
+        if (t == 0)
+        {
+            s_flag[nx] = 0;
+        }
+        if (wave_pred && lane == 0)
+        {
+            s_flag[c] = 1;
+        }
+        lds_barrier();
+        phase = nx;
+        return s_flag[c] != 0;
+    };
+
+    for (;;)
+    {
+        if (merge_now)
+        {
+            merge_buffer<BS, IPT>(topk, buffer, limit, t);
+            if (t == 0)
+            {
+                s_size -= limit;
+            }
+            radius = broadcast_radius<IPT>(topk, a.k, &s_radius, t);
+            // values of the current chunk that did not fit before
+            bool later = false;
+            if (wave_has_values)
+            {
+#pragma unroll
+                for (int j = 0; j < E; ++j)
+                {
+                    slot_base[j] -= NL;
+                }
+                later = write_slots();
+            }
+            merge_now = vote(later);
+            limit = NL;
+            continue;
+        }
+        if (finished)
+        {
+            break;
+        }
+        if (chunk >= n)
+        {
+            // end of the row: merge what is left in the buffer (the last vote's barrier ordered
+            // every slot write and every update of the size before this read)
+            finished = true;
+            wave_has_values = false;
+            const int left = s_size;
+            if (left > 0)
+            {
+                merge_now = true;
+                limit = left;
+            }
+            continue;
+        }
+
+        // next chunk
+        if (chunk < full_end)
+        {
+            if constexpr (VEC)
+            {
+                const vfloat4* __restrict__ p = reinterpret_cast<const vfloat4*>(row + chunk) + t;
+#pragma unroll
+                for (int l = 0; l < L; ++l)
+                {
+                    const vfloat4 x = __builtin_nontemporal_load(p + l * BS);
+                    v[4 * l + 0] = x.x;
+                    v[4 * l + 1] = x.y;
+                    v[4 * l + 2] = x.z;
+                    v[4 * l + 3] = x.w;
+                }
+            }
+            else
+            {
+                const float* __restrict__ p = row + chunk + t;
+#pragma unroll
+                for (int j = 0; j < E; ++j)
+                {
+                    v[j] = __builtin_nontemporal_load(p + j * BS);
+                }
+            }
+        }
+        else
+        {
+            // ragged tail: bounds-checked 4-byte loads in the same value-to-thread mapping
+#pragma unroll
+            for (int j = 0; j < E; ++j)
+            {
+                const u32 col = column_of(chunk, j);
+                v[j] = col < n ? row[col] : __builtin_inff();
+            }
+        }
+        cur_chunk = chunk;
+        chunk += CHUNK;
+
+        // filter
+        float smallest = v[0];
+#pragma unroll
+        for (int j = 1; j < E; ++j)
+        {
+            smallest = fminf(smallest, v[j]);
+        }
+        wave_has_values = __builtin_amdgcn_ballot_w64(smallest < radius) != 0;
+        bool later = false;
+        if (wave_has_values)
+        {
+            my_pass = 0;
+#pragma unroll
+            for (int j = 0; j < E; ++j)
+            {
+                const bool pass = v[j] < radius;
+                my_pass |= pass ? (1U << j) : 0U;
+                const u64 mask = __builtin_amdgcn_ballot_w64(pass);
+                if (mask != 0)
+                {
+                    int base = 0;
+                    if (lane == 0)
+                    {
+                        base = atomicAdd(&s_size, __popcll(mask));
+                    }
+                    slot_base[j] = __builtin_amdgcn_readfirstlane(base);
+                }
+            }
+            later = write_slots();
+        }
+        merge_now = vote(later);
+    }
+
+    float* __restrict__ out_d = a.out_dist + row_idx * a.out_stride;
+    std::int32_t* __restrict__ out_l = a.out_label + row_idx * a.out_stride;
+#pragma unroll
+    for (int r = 0; r < IPT; ++r)
+    {
+        const u32 e = static_cast<u32>(t * IPT + r);
+        if (e < a.k)
+        {
+            out_d[e] = key_value(topk[r]);
+            out_l[e] = key_label(topk[r]);
+        }
+    }
+}
+
+
+} // namespace bitsknn
+
+#endif // BITSKNN_CSRC_TOPK_BITS_KERNEL_HPP_

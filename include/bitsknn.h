@@ -1,0 +1,124 @@
+/*
+ * bitsknn -- C ABI of the MI355X (gfx950) k-NN hot path.
+ *
+ * Plain C, raw device pointers and sizes.  Every entry point
+ *   - returns 0 (BITSKNN_OK) or a BITSKNN_ERR_* code; the message of the last failure on the
+ *     calling thread is available from bitsknn_last_error();
+ *   - takes device pointers that the caller owns, allocates nothing and frees nothing;
+ *   - enqueues its kernels on `stream` (a hipStream_t passed as void*, NULL = default stream)
+ *     and returns without synchronising -- the caller synchronises, like the reference's host
+ *     wrappers do at the end of every phase (reference src/topk/singlepass/bits_knn.cu:95,
+ *     src/knn.cpp:28).
+ *
+ * Each declaration cites the reference interface it replaces (paths relative to the
+ * reference tree).  Strides are in elements, not bytes.
+ */
+#ifndef BITSKNN_H_
+#define BITSKNN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BITSKNN_OK 0
+#define BITSKNN_ERR_UNSUPPORTED 1 /* parameter outside the compiled lists (reference: runtime_error "Unsupported ...") */
+#define BITSKNN_ERR_INVALID 2     /* null pointer / inconsistent sizes */
+#define BITSKNN_ERR_HIP 3         /* a HIP runtime call failed (reference: CUCH -> runtime_error) */
+
+/* Message of the last error reported on this thread ("" if none). Never NULL. */
+const char* bitsknn_last_error(void);
+
+/* Library version string. */
+const char* bitsknn_version(void);
+
+/*
+ * bits top-k selection: for every row of a rows x cols fp32 matrix, the k smallest values in
+ * ascending order with their labels; equal values are ordered by lower label.
+ *
+ * Replaces run_bits_kernel<float, int32_t, PREFETCH, BLOCK_SIZE, BATCH_SIZE, K>
+ * (include/bits/topk/singlepass/bits_kernel.hpp:22-27,
+ *  include/bits/topk/singlepass/detail/bits_kernel.cuh:317-429) and the runtime dispatch of
+ * struct bits (src/topk/singlepass/bits_knn.cu:29-65).
+ *
+ *  in, in_row_stride       distance matrix, row r starts at in + r*in_row_stride
+ *  in_label                NULL: the label of column c is c; else a rows x cols int32 matrix
+ *  label_row_stride        row stride of in_label (ignored when in_label is NULL)
+ *  label_offsets           NULL or rows int32 values added to every label of that row
+ *  out_dist, out_label     rows x k outputs, row stride out_row_stride (>= k)
+ *  k                       1 <= k <= 2048; rounded up to the next of {16,...,2048} internally
+ *  block_size              threads per row: 128, 256 or 512
+ *  items_per_thread        values each thread has in flight per iteration: 1..16
+ *  prefetch                non-zero (the reference's `bits-prefetch`): twice as many values in
+ *                          flight per thread, i.e. the next batch is requested together with the
+ *                          current one; zero: `bits`
+ *
+ * Errors: "Unsupported block size: N", "Unsupported batch size: N", "Unsupported k value: N"
+ * exactly as the reference throws them (bits_knn.cu:52-62).
+ * When k > cols the tail of a row is filled with (+inf, INT32_MAX).
+ */
+int bitsknn_topk_bits_f32(const float* in, size_t in_row_stride, const int32_t* in_label,
+                          size_t label_row_stride, const int32_t* label_offsets, size_t rows,
+                          size_t cols, float* out_dist, int32_t* out_label, size_t out_row_stride,
+                          uint32_t k, uint32_t block_size, uint32_t items_per_thread, int prefetch,
+                          void* stream);
+
+/*
+ * Label offsets for a row-split single-query problem: offsets[i] = (i % parts) * cols_per_part
+ * for i < rows*parts.  Replaces populate_label_offsets_kernel
+ * (src/topk/singlepass/bits_knn.cu:67-76).
+ */
+int bitsknn_label_offsets(int32_t* offsets, size_t rows, size_t parts, size_t cols_per_part,
+                          void* stream);
+
+/* Fill count floats with value.  Replaces fill_kernel (src/cuda_stream.cu:9-24). */
+int bitsknn_fill_f32(float* dst, size_t count, float value, void* stream);
+
+/*
+ * Distance matrix dist[i*dist_row_stride + j] between query i and point j, inputs dim-major
+ * (component t of vector v at base[t*stride + v]), as the reference uploads them
+ * (src/distance/magma_distance.cu:13-71).
+ *
+ * Replaces run_abstract_gemm<Ops>(K, M, N, A, B, C)
+ * (include/bits/distance/abstract_gemm.cuh:730-755) for
+ *   BITSKNN_DIST_L2          Ops = l2_ops: acc = fmaf(q-p, q-p, acc) over the dimensions in
+ *                            order (abstract_gemm.cuh:59-100); bit-reproducible
+ *   BITSKNN_DIST_PARTIAL_L2  Ops = partial_l2_ops: ||p||^2 - 2 q.p, no ||q||^2
+ *                            (abstract_gemm.cuh:108-170); contraction on fp32 MFMA
+ * and the SGEMM + squared_length_kernel + add_norm_kernel sequence of
+ * cublas_distance::compute (src/distance/cublas_distance.cu:111-186) for
+ *   BITSKNN_DIST_EXPANDED    -2 q.p on fp32 MFMA, then + ||p||^2, written once
+ */
+#define BITSKNN_DIST_L2 0
+#define BITSKNN_DIST_PARTIAL_L2 1
+#define BITSKNN_DIST_EXPANDED 2
+int bitsknn_dist_f32(int op, int dim, size_t q, size_t n, const float* queries_dim_major,
+                     size_t query_stride, const float* points_dim_major, size_t point_stride,
+                     float* dist, size_t dist_row_stride, void* stream);
+
+/*
+ * bits-fused: partial squared L2 distance (||p||^2 - 2 q.p) and top-k in one kernel; the
+ * q x n distance matrix is never written to memory.  Outputs q x k, row stride k, ascending,
+ * equal distances ordered by lower point index.
+ *
+ * Replaces fused_cache::run / launch_fused_cache
+ * (src/topk/singlepass/fused_cache_knn.cu:29-145,
+ *  include/bits/topk/singlepass/detail/fused_cache_kernel.cuh:25-42).
+ * Inputs dim-major with strides q and n (fused_cache_knn.cu:156-194).
+ *  k                          one of 4, 8, 16, 32, 64, 128, 256 ("Unsupported k value: N" otherwise)
+ *  query_reg, db_reg, dim_reg, block_query_dim, dim_mult
+ *                             the reference's tuning parameters; validated against its lists
+ *                             ({2,4,8,16}, {4,8,16}, {1,2,4}, {1,2,4}, {1,2,4}) with its
+ *                             messages; dim must be >= dim_mult*dim_reg as there
+ */
+int bitsknn_fused_l2_topk_f32(const float* queries_dim_major, const float* points_dim_major,
+                              int dim, int32_t q, int32_t n, float* out_dist, int32_t* out_label,
+                              int k, int query_reg, int db_reg, int dim_reg, int block_query_dim,
+                              int dim_mult, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BITSKNN_H_ */

@@ -1,0 +1,214 @@
+"""Parity of the bits top-k HIP kernel (through the C ABI) with the CPU oracle.
+
+Bar: bit-exact values and labels, equal values ordered by lower label.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(bk, dev, matrix, k, block=256, batch=16, prefetch=False, labels=None, offsets=None):
+    import torch
+    d = torch.from_numpy(matrix).to(dev)
+    lab = torch.from_numpy(labels).to(dev) if labels is not None else None
+    off = torch.from_numpy(offsets).to(dev) if offsets is not None else None
+    od, ol = bk.topk_bits(d, k, block, batch, prefetch, in_label=lab, label_offsets=off)
+    torch.cuda.synchronize()
+    return od.cpu().numpy(), ol.cpu().numpy()
+
+
+def _check(bk, dev, oracle, matrix, k, **kw):
+    gd, gl = _run(bk, dev, matrix, k, **kw)
+    ed, el = oracle.topk(matrix, k, labels=kw.get("labels"), label_offsets=kw.get("offsets"))
+    assert np.array_equal(gd.view(np.uint32), ed.view(np.uint32)), "values differ"
+    assert np.array_equal(gl, el), "labels differ"
+
+
+# the reference's own unit-test shapes (tests/topk/bits_knn_test.cpp:7-63): seed 42, d = 10
+@pytest.mark.parametrize("n,k", [(128, 128), (1024, 256)])
+@pytest.mark.parametrize("batch", [1, 7, 16])
+def test_reference_unit_test_shapes(bk, dev, oracle, n, k, batch):
+    p, q = oracle.generate(42, n, 1, 10)
+    dist = oracle.dist(q, p, "l2")
+    _check(bk, dev, oracle, dist, k, block=128, batch=batch)
+
+
+@pytest.mark.parametrize("block", [128, 256, 512])
+@pytest.mark.parametrize("k", [1, 16, 32, 64, 100, 128, 256, 512, 1024, 2048])
+def test_uniform_rows_all_k_and_blocks(bk, dev, oracle, block, k):
+    m = oracle.uniform_matrix(1000 + k + block, 6, 40000)
+    _check(bk, dev, oracle, m, k, block=block, batch=8)
+
+
+@pytest.mark.parametrize("batch,prefetch", [(1, False), (4, False), (5, False), (9, False), (12, False),
+                                            (16, False), (1, True), (8, True), (12, True), (16, True)])
+def test_batch_sizes_and_prefetch(bk, dev, oracle, batch, prefetch):
+    m = oracle.uniform_matrix(77 + batch, 5, 70001)
+    _check(bk, dev, oracle, m, 128, block=256, batch=batch, prefetch=prefetch)
+    _check(bk, dev, oracle, m, 2048, block=256, batch=batch, prefetch=prefetch)
+
+
+@pytest.mark.parametrize("cols", [1, 2, 15, 16, 17, 127, 128, 129, 255, 256, 257, 511, 513, 1000, 4095,
+                                  4096, 4097, 12289, 16385])
+def test_ragged_row_lengths(bk, dev, oracle, cols):
+    m = oracle.uniform_matrix(cols, 3, cols)
+    for k in (1, 16, 32, 300):
+        _check(bk, dev, oracle, m, k, block=128, batch=7)
+        _check(bk, dev, oracle, m, k, block=512, batch=16)
+
+
+def test_rows_not_16_byte_aligned(bk, dev, oracle):
+    import torch
+    # a row stride that is not a multiple of 4 floats, and a base offset of one float
+    big = oracle.uniform_matrix(5, 9, 30011)
+    t = torch.from_numpy(big).to(dev)
+    for view, ref in ((t[:, 1:20000], big[:, 1:20000]), (t[:, 3:30011], big[:, 3:30011]), (t[:, :30008], big[:, :30008])):
+        od, ol = bk.topk_bits(view, 64, 256, 16)
+        torch.cuda.synchronize()
+        ed, el = oracle.topk(ref, 64)
+        assert np.array_equal(od.cpu().numpy(), ed) and np.array_equal(ol.cpu().numpy(), el)
+
+
+@pytest.mark.parametrize("kind", ["ascending", "descending", "256-values", "constant", "two-values"])
+@pytest.mark.parametrize("k", [32, 256, 2048])
+def test_hard_inputs(bk, dev, oracle, kind, k):
+    rows, cols = 4, 65536
+    base = oracle.uniform_matrix(99, rows, cols)
+    if kind == "ascending":
+        m = np.sort(base, axis=1)
+    elif kind == "descending":
+        m = np.sort(base, axis=1)[:, ::-1].copy()
+    elif kind == "256-values":
+        m = (np.floor(base * 256) / 256).astype(np.float32)
+    elif kind == "constant":
+        m = np.full((rows, cols), 0.25, dtype=np.float32)
+    else:
+        m = (base > 0.5).astype(np.float32)
+    for block in (128, 256, 512):
+        if k // block > 16:
+            continue
+        _check(bk, dev, oracle, m, k, block=block, batch=16)
+
+
+def test_negative_values_and_infinities(bk, dev, oracle):
+    m = oracle.uniform_matrix(3, 4, 20000, -5.0, 5.0)
+    m[0, 17] = -np.inf
+    m[1, 5] = np.inf
+    m[2, :] = np.inf
+    m[2, 100] = 1.0
+    _check(bk, dev, oracle, m, 64, block=256, batch=16)
+    _check(bk, dev, oracle, m, 1024, block=128, batch=3)
+
+
+def test_negative_zero_is_returned_as_positive_zero(bk, dev, oracle):
+    # documented deviation: -0.0 ties with +0.0 (as for the oracle) but is written back as +0.0
+    m = oracle.uniform_matrix(4, 1, 5000, 1.0, 2.0)
+    m[0, 10] = -0.0
+    m[0, 4000] = 0.0
+    gd, gl = _run(bk, dev, m, 16)
+    assert list(gl[0, :2]) == [10, 4000]
+    assert gd[0, 0] == 0.0 and gd[0, 1] == 0.0 and not np.signbit(gd[0, 0])
+
+
+def test_k_larger_than_row(bk, dev, oracle):
+    m = oracle.uniform_matrix(8, 3, 20)
+    _check(bk, dev, oracle, m, 32, block=128, batch=1)
+
+
+def test_explicit_labels_and_offsets(bk, dev, oracle):
+    rng = np.random.default_rng(1)
+    m = (np.floor(oracle.uniform_matrix(12, 6, 9000) * 64) / 64).astype(np.float32)
+    labels = np.stack([rng.permutation(9000) for _ in range(6)]).astype(np.int32)
+    offsets = (np.arange(6) * 9000).astype(np.int32)
+    _check(bk, dev, oracle, m, 200, block=256, batch=16, labels=labels)
+    _check(bk, dev, oracle, m, 200, block=256, batch=16, offsets=offsets)
+    _check(bk, dev, oracle, m, 200, block=128, batch=5, labels=labels, offsets=offsets)
+
+
+def test_row_split_like_bits_sq(bk, dev, oracle):
+    """One long row split into parts, then merged with explicit labels
+    (reference src/topk/singlepass/bits_knn.cu:132-186)."""
+    import torch
+    n, deg, k = 1 << 18, 8, 64
+    row = oracle.uniform_matrix(21, 1, n)
+    t = torch.from_numpy(row).to(dev)
+    cols = n // deg
+    offs = bk.label_offsets(1, deg, cols, dev)
+    assert offs.cpu().tolist() == [i * cols for i in range(deg)]
+    pd, pl = bk.topk_bits(t.view(deg, cols), k, 256, 16, True, label_offsets=offs)
+    fd, fl = bk.topk_bits(pd.view(1, deg * k), k, 256, 16, True, in_label=pl.view(1, deg * k))
+    torch.cuda.synchronize()
+    ed, el = oracle.topk(row, k)
+    assert np.array_equal(fd.cpu().numpy(), ed) and np.array_equal(fl.cpu().numpy(), el)
+
+
+def test_strided_output(bk, dev, oracle):
+    import torch
+    m = oracle.uniform_matrix(31, 5, 10000)
+    od = torch.full((5, 100), -1.0, device=dev)
+    ol = torch.full((5, 100), -1, dtype=torch.int32, device=dev)
+    bk.topk_bits(torch.from_numpy(m).to(dev), 40, 256, 16, out_dist=od, out_label=ol)
+    torch.cuda.synchronize()
+    ed, el = oracle.topk(m, 40)
+    assert np.array_equal(od[:, :40].cpu().numpy(), ed) and np.array_equal(ol[:, :40].cpu().numpy(), el)
+    assert (od[:, 40:] == -1).all() and (ol[:, 40:] == -1).all()
+
+
+def test_fill_and_errors_on_device(bk, dev):
+    import torch
+    t = torch.zeros(100003, device=dev)
+    bk.fill(t, 2.5)
+    torch.cuda.synchronize()
+    assert (t == 2.5).all()
+    with pytest.raises(bk.BitsKnnError, match="Unsupported block size: 64"):
+        bk.topk_bits(torch.zeros((2, 100), device=dev), 16, 64, 1)
+
+
+# reference-held checksums of query 0 (data/kselection-*.err), distances by the oracle
+@pytest.mark.parametrize("n,q", [(1 << 20, 1024), (1 << 18, 4096)])
+def test_golden_kselection_checksums(bk, dev, oracle, golden, n, q):
+    p, qq = oracle.generate(24, n, q, 1)
+    dist = oracle.dist(qq[:4], p, "l2")
+    checked = 0
+    for rec in golden:
+        if rec["family"] != "kselection" or rec["n"] != n or rec["q"] != q:
+            continue
+        for block in (128, 256, 512):
+            if rec["k"] // block > 16:
+                continue
+            gd, gl = _run(bk, dev, dist, rec["k"], block=block, batch=16)
+            assert str(oracle.checksum(gl[0])) in rec["checksums"], (rec, block)
+            ed, el = oracle.topk(dist, rec["k"])
+            assert np.array_equal(gd, ed) and np.array_equal(gl, el)
+            checked += 1
+    assert checked >= 7
+
+
+def test_full_size_properties(bk, dev):
+    """1024 x 2^20 uniform rows (4 GiB): size-independent properties against torch.topk values."""
+    import torch
+    g = torch.Generator(device=dev)
+    g.manual_seed(24)
+    rows, cols = 1024, 1 << 20
+    m = torch.rand((rows, cols), device=dev, generator=g)
+    for k, block in ((32, 256), (512, 512), (2048, 256)):
+        od, ol = bk.topk_bits(m, k, block, 16, True)
+        torch.cuda.synchronize()
+        # ascending
+        assert bool((od[:, 1:] >= od[:, :-1]).all())
+        # every value is the matrix entry its label points to
+        assert torch.equal(torch.gather(m, 1, ol.long()), od)
+        # equal values come out by ascending label, labels are distinct
+        same = od[:, 1:] == od[:, :-1]
+        assert bool((ol[:, 1:][same] > ol[:, :-1][same]).all())
+        assert bool((torch.sort(ol, dim=1).values[:, 1:] != torch.sort(ol, dim=1).values[:, :-1]).all())
+        # the k smallest: bit-equal to torch's sorted top-k values on a sample of rows
+        sample = torch.arange(0, rows, 37, device=dev)
+        tv = torch.topk(m[sample], k, dim=1, largest=False, sorted=True).values
+        assert torch.equal(tv, od[sample])
+        # nothing smaller was left behind
+        kth = od[:, -1:]
+        assert bool(((m < kth).sum(dim=1) <= k - 1).all())
+    del m
+    torch.cuda.empty_cache()
