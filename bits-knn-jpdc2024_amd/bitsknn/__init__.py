@@ -44,6 +44,10 @@ def lib():
             raise RuntimeError(
                 f"{LIB_PATH} is missing: build it with `make -C {os.path.dirname(_HERE)} lib` "
                 "(there is no fallback path)")
+        # torch bundles its own HIP runtime under the same soname as the system one; it has to be
+        # loaded first so that this library binds to the runtime that owns torch's device memory
+        # and streams instead of bringing up a second runtime in the process
+        import torch  # noqa: F401
         L = ctypes.CDLL(LIB_PATH)
         vp, sz, i32, u32 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int32, ctypes.c_uint32
         L.bitsknn_last_error.restype = ctypes.c_char_p

@@ -173,16 +173,16 @@ __device__ __forceinline__ void merge_buffer(u64 (&topk)[IPT], u64* buffer, int 
     net_phase<BS, IPT, N, N / 2, false>(topk, buffer, t);
 }
 
-// value of sorted element k-1, broadcast to the whole workgroup (includes a barrier)
+// key of sorted element k-1, broadcast to the whole workgroup (includes a barrier)
 template <int IPT>
-__device__ __forceinline__ float broadcast_radius(const u64 (&topk)[IPT], u32 k, float* slot, int t)
+__device__ __forceinline__ u64 broadcast_radius(const u64 (&topk)[IPT], u32 k, u64* slot, int t)
 {
 #pragma unroll
     for (int r = 0; r < IPT; ++r)
     {
         if (static_cast<u32>(t * IPT + r) == k - 1)
         {
-            *slot = key_value(topk[r]);
+            *slot = topk[r];
         }
     }
     __syncthreads();
@@ -206,7 +206,7 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     __shared__ u64 buffer[NL];
     __shared__ int s_size;
     __shared__ int s_flag[3];
-    __shared__ float s_radius;
+    __shared__ u64 s_radius;
 
     const int t = static_cast<int>(threadIdx.x);
     const int lane = t & (WAVE - 1);
@@ -267,7 +267,12 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     }
     __syncthreads();
 
+    // Filter threshold: the k-th smallest key so far.  With implicit labels every later column
+    // has a larger label than anything merged before, so `value < radius` loses nothing; with
+    // explicit labels an equal value can still win on its label and is compared on the full key.
     float radius = __builtin_inff();
+    u64 radius_key = PAD_KEY;
+    const bool explicit_labels = lrow != nullptr;
     int phase = 0;
     bool merge_now = true;   // workgroup-uniform
     int limit = static_cast<int>(first);
@@ -350,7 +355,8 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
             {
                 s_size -= limit;
             }
-            radius = broadcast_radius<IPT>(topk, a.k, &s_radius, t);
+            radius_key = broadcast_radius<IPT>(topk, a.k, &s_radius, t);
+            radius = key_value(radius_key);
             // values of the current chunk that did not fit before
             bool later = false;
             if (wave_has_values)
@@ -431,7 +437,8 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
         {
             smallest = fminf(smallest, v[j]);
         }
-        wave_has_values = __builtin_amdgcn_ballot_w64(smallest < radius) != 0;
+        wave_has_values =
+            __builtin_amdgcn_ballot_w64(explicit_labels ? smallest <= radius : smallest < radius) != 0;
         bool later = false;
         if (wave_has_values)
         {
@@ -439,7 +446,12 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
 #pragma unroll
             for (int j = 0; j < E; ++j)
             {
-                const bool pass = v[j] < radius;
+                bool pass = v[j] < radius;
+                if (explicit_labels && v[j] == radius)
+                {
+                    const u32 col = column_of(cur_chunk, j);
+                    pass = col < n && make_key(v[j], label_of(col)) < radius_key;
+                }
                 my_pass |= pass ? (1U << j) : 0U;
                 const u64 mask = __builtin_amdgcn_ballot_w64(pass);
                 if (mask != 0)
