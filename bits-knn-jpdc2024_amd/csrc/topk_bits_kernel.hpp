@@ -287,45 +287,30 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     }
 
     // Slot bookkeeping of the current chunk: bit j of my_pass says value j of this lane passed
-    // the filter; the passing lanes of value j were assigned consecutive slots from
-    // slot_base[j] (wave-uniform) in lane order.  slot_base drops by NL with every merge; a value
-    // is written in the round where its slot falls into [0, NL).
+    // the filter.  The wave reserves one contiguous range of slots [.., wave_end) with a single
+    // LDS atomic; inside it every lane owns consecutive slots from my_slot (lane order, by a
+    // wave prefix sum of the per-lane counts).  Both drop by NL with every merge; a value is
+    // written in the round where its slot falls into [0, NL).
     u32 my_pass = 0;
-    int slot_base[E];
-#pragma unroll
-    for (int j = 0; j < E; ++j)
-    {
-        slot_base[j] = 0;
-    }
+    int my_slot = 0;
+    int wave_end = 0;
     bool wave_has_values = false;
 
-    auto write_slots = [&]() -> bool {
-        bool later = false;
+    auto write_slots = [&]() {
+        int slot = my_slot;
 #pragma unroll
         for (int j = 0; j < E; ++j)
         {
-            const bool mine = ((my_pass >> j) & 1U) != 0;
-            const u64 mask = __builtin_amdgcn_ballot_w64(mine);
-            if (mask != 0)
+            if (((my_pass >> j) & 1U) != 0)
             {
-                const int count = __popcll(mask);
-                const int base = slot_base[j];
-                if (base < NL && base + count > 0)
+                if (slot >= 0 && slot < NL)
                 {
-                    const int rank = static_cast<int>(__builtin_amdgcn_mbcnt_hi(
-                        static_cast<u32>(mask >> 32U),
-                        __builtin_amdgcn_mbcnt_lo(static_cast<u32>(mask), 0U)));
-                    const int slot = base + rank;
-                    if (mine && slot >= 0 && slot < NL)
-                    {
-                        const u32 col = column_of(cur_chunk, j);
-                        buffer[slot] = make_key(v[j], label_of(col));
-                    }
+                    const u32 col = column_of(cur_chunk, j);
+                    buffer[slot] = make_key(v[j], label_of(col));
                 }
-                later |= (base + count > NL);
+                ++slot;
             }
         }
-        return later;
     };
 
     // workgroup-wide vote; three rotating flags keep the reset of a flag two barriers away from
@@ -361,12 +346,10 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
             bool later = false;
             if (wave_has_values)
             {
-#pragma unroll
-                for (int j = 0; j < E; ++j)
-                {
-                    slot_base[j] -= NL;
-                }
-                later = write_slots();
+                my_slot -= NL;
+                wave_end -= NL;
+                write_slots();
+                later = wave_end > NL;
             }
             merge_now = vote(later);
             limit = NL;
@@ -453,18 +436,31 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
                     pass = col < n && make_key(v[j], label_of(col)) < radius_key;
                 }
                 my_pass |= pass ? (1U << j) : 0U;
-                const u64 mask = __builtin_amdgcn_ballot_w64(pass);
-                if (mask != 0)
-                {
-                    int base = 0;
-                    if (lane == 0)
-                    {
-                        base = atomicAdd(&s_size, __popcll(mask));
-                    }
-                    slot_base[j] = __builtin_amdgcn_readfirstlane(base);
-                }
             }
-            later = write_slots();
+            // exclusive prefix sum of the per-lane counts over the wave, one ballot per count bit
+            const int count = __popc(my_pass);
+            int prefix = 0;
+            int total = 0;
+#pragma unroll
+            for (int b = 0; (1 << b) <= E; ++b)
+            {
+                const u64 bit_mask = __builtin_amdgcn_ballot_w64(((count >> b) & 1) != 0);
+                const int below = static_cast<int>(__builtin_amdgcn_mbcnt_hi(
+                    static_cast<u32>(bit_mask >> 32U),
+                    __builtin_amdgcn_mbcnt_lo(static_cast<u32>(bit_mask), 0U)));
+                prefix += below << b;
+                total += __popcll(bit_mask) << b;
+            }
+            int base = 0;
+            if (lane == 0)
+            {
+                base = atomicAdd(&s_size, total);
+            }
+            base = __builtin_amdgcn_readfirstlane(base);
+            my_slot = base + prefix;
+            wave_end = base + total;
+            write_slots();
+            later = wave_end > NL;
         }
         merge_now = vote(later);
     }
