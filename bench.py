@@ -68,8 +68,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--k", type=int, default=32)
     ap.add_argument("--block-size", type=int, default=256)
-    ap.add_argument("--items-per-thread", type=int, default=16)
-    ap.add_argument("--no-prefetch", action="store_true")
+    ap.add_argument("--items-per-thread", type=int, default=8)
+    ap.add_argument("--prefetch", action="store_true", help="the bits-prefetch variant")
     ap.add_argument("--rows", type=int, default=1024)
     ap.add_argument("--cols", type=int, default=1 << 20)
     ap.add_argument("--sweep", action="store_true", help="also time k x block-size combinations")
@@ -89,7 +89,7 @@ def main():
     gen.manual_seed(24)
     rows, cols = args.rows, args.cols
     matrix = torch.rand((rows, cols), device=dev, generator=gen)
-    prefetch = not args.no_prefetch
+    prefetch = args.prefetch
 
     def run(k, block, batch, steps, warmup):
         out_d = torch.empty((rows, k), dtype=torch.float32, device=dev)

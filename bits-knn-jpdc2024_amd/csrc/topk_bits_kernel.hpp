@@ -1,18 +1,24 @@
 // bits top-k selection for gfx950 (wave64).
 //
 // One workgroup per matrix row.  The row is streamed from HBM in 16-byte loads; a value is kept
-// only if it is below the current k-th smallest value ("radius").  Kept values are appended as
-// 64-bit (value, label) keys to a buffer in LDS (one LDS atomic per wave and value slot, slots
-// assigned by ballot + lane prefix count).  When the buffer is full the whole workgroup sorts it
-// descending with a bitonic network held in registers, takes the element-wise minimum with the
-// ascending top-k list (a bitonic separator), re-sorts the resulting bitonic sequence and
-// publishes the new radius.
+// only if its (value, label) key is below the current k-th smallest key ("radius").  Kept values
+// are appended as 64-bit keys to a buffer in LDS.  When the buffer is full the whole workgroup
+// sorts it descending with a bitonic network held in registers, takes the element-wise minimum
+// with the ascending top-k list (a bitonic separator), re-sorts the resulting bitonic sequence
+// and publishes the new radius.
 //
 // Same algorithm and phases as the reference kernel
 // (include/bits/topk/singlepass/detail/bits_kernel.cuh:317-408: alloc :117-126, insert :277-302,
-// merge :145-199, radius :30-51), laid out for 64-wide waves: exchange distances below 64 lanes
-// stay inside a wave, only distances of 64 lanes and more go through LDS, and the per-batch
-// overflow vote is one LDS flag read after one barrier that does not wait for global loads.
+// merge :145-199, radius :30-51), laid out for 64-wide waves:
+//  * every wave owns a private slice of the buffer, so appending needs no atomics: slots come
+//    from a ballot-based prefix sum over the wave and a wave-uniform fill counter;
+//  * the waves of a row do not synchronise per batch.  A wave whose slice is full raises a flag
+//    in LDS and waits at a barrier; the others poll the flag once per batch and join.  The only
+//    barriers are those of a merge;
+//  * exchange distances below 64 lanes stay inside a wave, only distances of 64 lanes and more
+//    go through LDS.
+// Because waves drift apart, the filter compares full keys when a value equals the radius, so
+// that "equal values by lower label" holds no matter which wave saw which value first.
 
 #ifndef BITSKNN_CSRC_TOPK_BITS_KERNEL_HPP_
 #define BITSKNN_CSRC_TOPK_BITS_KERNEL_HPP_
@@ -148,18 +154,20 @@ __device__ __forceinline__ void net_sort(u64 (&x)[IPT], u64* scratch, int t)
     }
 }
 
-// Merge the first `limit` keys of the LDS buffer into the ascending top-k list.  The buffer
-// memory doubles as exchange scratch once its keys are in registers.
+// Merge the filled part of every wave's buffer slice into the ascending top-k list.  Slice w
+// holds fill[w] keys from buffer[w*CAP].  The buffer memory doubles as exchange scratch once its
+// keys are in registers.
 template <int BS, int IPT>
-__device__ __forceinline__ void merge_buffer(u64 (&topk)[IPT], u64* buffer, int limit, int t)
+__device__ __forceinline__ void merge_buffer(u64 (&topk)[IPT], u64* buffer, const int* fill, int t)
 {
     constexpr int N = BS * IPT;
+    constexpr int CAP = WAVE * IPT;
     u64 tmp[IPT];
 #pragma unroll
     for (int r = 0; r < IPT; ++r)
     {
         const int idx = r * BS + t;
-        tmp[r] = idx < limit ? buffer[idx] : PAD_KEY;
+        tmp[r] = (idx % CAP) < fill[idx / CAP] ? buffer[idx] : PAD_KEY;
     }
     // (the first LDS exchange of the sort starts with a barrier, so the loads above are done)
     net_sort<BS, IPT, 2, true>(tmp, buffer, t);
@@ -191,25 +199,25 @@ __device__ __forceinline__ u64 broadcast_radius(const u64 (&topk)[IPT], u32 k, u
 
 // BS threads, IPT list entries per thread, L 16-byte (or 4 x 4-byte when !VEC) loads in flight
 // per thread and iteration.
-//
-// The kernel is one loop around a single merge site: the first NL values of the row are written
-// to the buffer and merged into the empty list, every later overflow merges a full buffer, and
-// the end of the row merges whatever is left.
 template <int BS, int IPT, int L, bool VEC>
 __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
 {
-    constexpr int NL = BS * IPT;     // length of the top-k list and of the buffer
+    constexpr int NL = BS * IPT;     // length of the top-k list and of the whole buffer
+    constexpr int W = BS / WAVE;     // waves per row
+    constexpr int CAP = WAVE * IPT;  // buffer slots owned by one wave (NL / W)
     constexpr int E = 4 * L;         // values per thread and iteration
     constexpr u32 CHUNK = BS * E;    // values per workgroup and iteration
     static_assert(E <= 32, "one pass bit per value in a 32-bit lane mask");
 
     __shared__ u64 buffer[NL];
-    __shared__ int s_size;
-    __shared__ int s_flag[3];
     __shared__ u64 s_radius;
+    __shared__ int s_fill[W];
+    __shared__ int s_flag;  // some wave wants a merge
+    __shared__ int s_more;  // some wave still has values to process after this merge
 
     const int t = static_cast<int>(threadIdx.x);
     const int lane = t & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(t / WAVE);
     const size_t row_idx = blockIdx.x;
     const float* __restrict__ row = a.in + row_idx * a.in_stride;
     const std::int32_t* __restrict__ lrow =
@@ -217,6 +225,7 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     const u32 label_offset =
         a.label_offsets != nullptr ? static_cast<u32>(a.label_offsets[row_idx]) : 0U;
     const u32 n = a.cols;
+    u64* const slice = buffer + wave * CAP;
 
     auto label_of = [&](u32 col) -> std::int32_t {
         const u32 base = lrow != nullptr ? static_cast<u32>(lrow[col]) : col;
@@ -248,7 +257,7 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
                                  : static_cast<u32>(NL);
     u32 chunk = NL;
 
-    // the first NL values go straight to the buffer
+    // the first NL values go straight to the buffer: column c into slot c
 #pragma unroll
     for (int r = 0; r < IPT; ++r)
     {
@@ -260,24 +269,14 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     }
     if (t == 0)
     {
-        s_size = static_cast<int>(first);
-        s_flag[0] = 0;
-        s_flag[1] = 0;
-        s_flag[2] = 0;
+        s_flag = 0;
+        s_more = 0;
     }
     __syncthreads();
 
-    // Filter threshold: the k-th smallest key so far.  With implicit labels every later column
-    // has a larger label than anything merged before, so `value < radius` loses nothing; with
-    // explicit labels an equal value can still win on its label and is compared on the full key.
     float radius = __builtin_inff();
     u64 radius_key = PAD_KEY;
-    const bool explicit_labels = lrow != nullptr;
-    int phase = 0;
-    bool merge_now = true;   // workgroup-uniform
-    int limit = static_cast<int>(first);
-    bool finished = false;
-    u32 cur_chunk = 0;       // first column of the chunk held in v[]
+    u32 cur_chunk = 0; // first column of the chunk held in v[]
 
     float v[E];
 #pragma unroll
@@ -286,183 +285,216 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
         v[j] = 0.0F;
     }
 
-    // Slot bookkeeping of the current chunk: bit j of my_pass says value j of this lane passed
-    // the filter.  The wave reserves one contiguous range of slots [.., wave_end) with a single
-    // LDS atomic; inside it every lane owns consecutive slots from my_slot (lane order, by a
-    // wave prefix sum of the per-lane counts).  Both drop by NL with every merge; a value is
-    // written in the round where its slot falls into [0, NL).
+    // Fill of this wave's slice (wave-uniform).  Passing values take slots in the order
+    // (value index j, lane): value j of the lanes in its pass mask gets consecutive slots after
+    // those of the values before it.
+    //
+    // Only when a chunk does not fit into the slice is per-lane state kept for it: bit j of
+    // my_pass says value j of this lane passed the filter (decided with the radius of that
+    // moment), slot_base is the slot of the chunk's first passing value.  A merge empties every
+    // slice, so slot_base drops by CAP; a value is written in the round where its slot falls
+    // into [0, CAP).
+    int fill = static_cast<int>(first) - wave * CAP;
+    fill = fill < 0 ? 0 : (fill > CAP ? CAP : fill);
     u32 my_pass = 0;
-    int my_slot = 0;
-    int wave_end = 0;
-    bool wave_has_values = false;
+    int slot_base = 0;
+    bool pending = false; // values of the chunk in v[] still wait for a slot
 
-    auto write_slots = [&]() {
-        int slot = my_slot;
+    auto lane_rank = [&](u64 mask) -> int {
+        return static_cast<int>(__builtin_amdgcn_mbcnt_hi(
+            static_cast<u32>(mask >> 32U), __builtin_amdgcn_mbcnt_lo(static_cast<u32>(mask), 0U)));
+    };
+
+    // exact filter: below the radius key (an equal value is decided by its label; the +inf
+    // padding of a ragged tail never passes)
+    auto passes = [&](float value, int j) -> bool {
+        bool pass = value < radius;
+        if (value == radius)
+        {
+            const u32 col = column_of(cur_chunk, j);
+            pass = col < n && make_key(value, label_of(col)) < radius_key;
+        }
+        return pass;
+    };
+
+    // writes the pending values whose slot is inside the slice; returns the end of the
+    // chunk's reservation
+    auto write_pending = [&]() -> int {
+        int running = slot_base;
 #pragma unroll
         for (int j = 0; j < E; ++j)
         {
-            if (((my_pass >> j) & 1U) != 0)
+            const bool mine = ((my_pass >> j) & 1U) != 0;
+            const u64 mask = __builtin_amdgcn_ballot_w64(mine);
+            if (mask != 0)
             {
-                if (slot >= 0 && slot < NL)
+                const int slot = running + lane_rank(mask);
+                if (mine && slot >= 0 && slot < CAP)
                 {
                     const u32 col = column_of(cur_chunk, j);
-                    buffer[slot] = make_key(v[j], label_of(col));
+                    slice[slot] = make_key(v[j], label_of(col));
                 }
-                ++slot;
+                running += __popcll(mask);
             }
         }
-    };
-
-    // workgroup-wide vote; three rotating flags keep the reset of a flag two barriers away from
-    // its last read
-    auto vote = [&](bool wave_pred) -> bool {
-        const int c = phase;
-        const int nx = c == 2 ? 0 : c + 1;
-        if (t == 0)
-        {
-            s_flag[nx] = 0;
-        }
-        if (wave_pred && lane == 0)
-        {
-            s_flag[c] = 1;
-        }
-        lds_barrier();
-        phase = nx;
-        return s_flag[c] != 0;
+        return running;
     };
 
     for (;;)
     {
-        if (merge_now)
+        // ---- rendezvous: every wave arrives here when it needs a merge, saw the flag, or ran
+        // out of values
+        const bool more_work = pending || chunk < n;
+        if (lane == 0)
         {
-            merge_buffer<BS, IPT>(topk, buffer, limit, t);
-            if (t == 0)
+            s_fill[wave] = fill;
+            if (more_work)
             {
-                s_size -= limit;
+                s_more = 1;
             }
+        }
+        __syncthreads();
+        int total = 0;
+#pragma unroll
+        for (int w = 0; w < W; ++w)
+        {
+            total += s_fill[w];
+        }
+        const bool more = s_more != 0;
+        if (total > 0)
+        {
+            merge_buffer<BS, IPT>(topk, buffer, s_fill, t);
             radius_key = broadcast_radius<IPT>(topk, a.k, &s_radius, t);
             radius = key_value(radius_key);
-            // values of the current chunk that did not fit before
-            bool later = false;
-            if (wave_has_values)
-            {
-                my_slot -= NL;
-                wave_end -= NL;
-                write_slots();
-                later = wave_end > NL;
-            }
-            merge_now = vote(later);
-            limit = NL;
-            continue;
         }
-        if (finished)
+        else
+        {
+            __syncthreads(); // orders the reads above before the reset below
+        }
+        if (t == 0)
+        {
+            s_flag = 0;
+            s_more = 0;
+        }
+        __syncthreads();
+        if (!more)
         {
             break;
         }
-        if (chunk >= n)
+        fill = 0;
+        if (pending)
         {
-            // end of the row: merge what is left in the buffer (the last vote's barrier ordered
-            // every slot write and every update of the size before this read)
-            finished = true;
-            wave_has_values = false;
-            const int left = s_size;
-            if (left > 0)
+            slot_base -= CAP;
+            const int end = write_pending();
+            if (end > CAP)
             {
-                merge_now = true;
-                limit = left;
+                fill = CAP;
+                if (lane == 0)
+                {
+                    s_flag = 1;
+                }
+                continue;
             }
-            continue;
+            fill = end;
+            pending = false;
         }
 
-        // next chunk
-        if (chunk < full_end)
+        // ---- streaming: no synchronisation with the other waves except polling the flag
+        while (chunk < n)
         {
-            if constexpr (VEC)
+            if (chunk < full_end)
             {
-                const vfloat4* __restrict__ p = reinterpret_cast<const vfloat4*>(row + chunk) + t;
-#pragma unroll
-                for (int l = 0; l < L; ++l)
+                if constexpr (VEC)
                 {
-                    const vfloat4 x = __builtin_nontemporal_load(p + l * BS);
-                    v[4 * l + 0] = x.x;
-                    v[4 * l + 1] = x.y;
-                    v[4 * l + 2] = x.z;
-                    v[4 * l + 3] = x.w;
+                    const vfloat4* __restrict__ p = reinterpret_cast<const vfloat4*>(row + chunk) + t;
+#pragma unroll
+                    for (int l = 0; l < L; ++l)
+                    {
+                        const vfloat4 x = __builtin_nontemporal_load(p + l * BS);
+                        v[4 * l + 0] = x.x;
+                        v[4 * l + 1] = x.y;
+                        v[4 * l + 2] = x.z;
+                        v[4 * l + 3] = x.w;
+                    }
+                }
+                else
+                {
+                    const float* __restrict__ p = row + chunk + t;
+#pragma unroll
+                    for (int j = 0; j < E; ++j)
+                    {
+                        v[j] = __builtin_nontemporal_load(p + j * BS);
+                    }
                 }
             }
             else
             {
-                const float* __restrict__ p = row + chunk + t;
+                // ragged tail: bounds-checked 4-byte loads in the same value-to-thread mapping
 #pragma unroll
                 for (int j = 0; j < E; ++j)
                 {
-                    v[j] = __builtin_nontemporal_load(p + j * BS);
+                    const u32 col = column_of(chunk, j);
+                    v[j] = col < n ? row[col] : __builtin_inff();
                 }
             }
-        }
-        else
-        {
-            // ragged tail: bounds-checked 4-byte loads in the same value-to-thread mapping
-#pragma unroll
-            for (int j = 0; j < E; ++j)
-            {
-                const u32 col = column_of(chunk, j);
-                v[j] = col < n ? row[col] : __builtin_inff();
-            }
-        }
-        cur_chunk = chunk;
-        chunk += CHUNK;
+            const int flag = *static_cast<volatile int*>(&s_flag);
+            cur_chunk = chunk;
+            chunk += CHUNK;
 
-        // filter
-        float smallest = v[0];
+            float smallest = v[0];
 #pragma unroll
-        for (int j = 1; j < E; ++j)
-        {
-            smallest = fminf(smallest, v[j]);
-        }
-        wave_has_values =
-            __builtin_amdgcn_ballot_w64(explicit_labels ? smallest <= radius : smallest < radius) != 0;
-        bool later = false;
-        if (wave_has_values)
-        {
-            my_pass = 0;
-#pragma unroll
-            for (int j = 0; j < E; ++j)
+            for (int j = 1; j < E; ++j)
             {
-                bool pass = v[j] < radius;
-                if (explicit_labels && v[j] == radius)
+                smallest = fminf(smallest, v[j]);
+            }
+            if (__builtin_amdgcn_ballot_w64(smallest <= radius) != 0)
+            {
+                int running = fill;
+#pragma unroll
+                for (int j = 0; j < E; ++j)
                 {
-                    const u32 col = column_of(cur_chunk, j);
-                    pass = col < n && make_key(v[j], label_of(col)) < radius_key;
+                    if (__builtin_amdgcn_ballot_w64(v[j] <= radius) != 0)
+                    {
+                        const bool pass = passes(v[j], j);
+                        const u64 mask = __builtin_amdgcn_ballot_w64(pass);
+                        if (mask != 0)
+                        {
+                            const int slot = running + lane_rank(mask);
+                            if (pass && slot < CAP)
+                            {
+                                const u32 col = column_of(cur_chunk, j);
+                                slice[slot] = make_key(v[j], label_of(col));
+                            }
+                            running += __popcll(mask);
+                        }
+                    }
                 }
-                my_pass |= pass ? (1U << j) : 0U;
-            }
-            // exclusive prefix sum of the per-lane counts over the wave, one ballot per count bit
-            const int count = __popc(my_pass);
-            int prefix = 0;
-            int total = 0;
+                if (running > CAP)
+                {
+                    // the slice is full: remember which values passed (the radius changes with
+                    // the merge) and ask for a merge
+                    my_pass = 0;
 #pragma unroll
-            for (int b = 0; (1 << b) <= E; ++b)
-            {
-                const u64 bit_mask = __builtin_amdgcn_ballot_w64(((count >> b) & 1) != 0);
-                const int below = static_cast<int>(__builtin_amdgcn_mbcnt_hi(
-                    static_cast<u32>(bit_mask >> 32U),
-                    __builtin_amdgcn_mbcnt_lo(static_cast<u32>(bit_mask), 0U)));
-                prefix += below << b;
-                total += __popcll(bit_mask) << b;
+                    for (int j = 0; j < E; ++j)
+                    {
+                        my_pass |= passes(v[j], j) ? (1U << j) : 0U;
+                    }
+                    slot_base = fill;
+                    pending = true;
+                    fill = CAP;
+                    if (lane == 0)
+                    {
+                        s_flag = 1;
+                    }
+                    break;
+                }
+                fill = running;
             }
-            int base = 0;
-            if (lane == 0)
+            if (__builtin_amdgcn_readfirstlane(flag) != 0)
             {
-                base = atomicAdd(&s_size, total);
+                break;
             }
-            base = __builtin_amdgcn_readfirstlane(base);
-            my_slot = base + prefix;
-            wave_end = base + total;
-            write_slots();
-            later = wave_end > NL;
         }
-        merge_now = vote(later);
     }
 
     float* __restrict__ out_d = a.out_dist + row_idx * a.out_stride;
