@@ -85,6 +85,12 @@ def _ptr(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else None
 
 
+def _row_stride(t):
+    # torch reports arbitrary strides for dimensions of extent 1
+    rows, cols = t.shape
+    return max(t.stride(0), cols) if rows > 1 else cols
+
+
 def version():
     return lib().bitsknn_version().decode()
 
@@ -94,7 +100,8 @@ def topk_bits(dist, k, block_size=256, items_per_thread=16, prefetch=False, in_l
     """bits top-k of every row of a 2-D float32 device tensor (last dim contiguous).
     Returns (values, labels), each rows x k."""
     import torch
-    assert dist.is_cuda and dist.dtype == torch.float32 and dist.dim() == 2 and dist.stride(1) == 1
+    assert dist.is_cuda and dist.dtype == torch.float32 and dist.dim() == 2
+    assert dist.shape[1] == 1 or dist.stride(1) == 1
     rows, cols = dist.shape
     if out_dist is None:
         out_dist = torch.empty((rows, k), dtype=torch.float32, device=dist.device)
@@ -102,13 +109,13 @@ def topk_bits(dist, k, block_size=256, items_per_thread=16, prefetch=False, in_l
         out_label = torch.empty((rows, k), dtype=torch.int32, device=dist.device)
     label_stride = 0
     if in_label is not None:
-        assert in_label.dtype == torch.int32 and in_label.shape == dist.shape and in_label.stride(1) == 1
-        label_stride = in_label.stride(0)
+        assert in_label.dtype == torch.int32 and in_label.shape == dist.shape and (cols == 1 or in_label.stride(1) == 1)
+        label_stride = _row_stride(in_label)
     if label_offsets is not None:
         assert label_offsets.dtype == torch.int32 and label_offsets.numel() == rows
-    _check(lib().bitsknn_topk_bits_f32(_ptr(dist), dist.stride(0) if rows > 1 else max(dist.stride(0), cols),
+    _check(lib().bitsknn_topk_bits_f32(_ptr(dist), _row_stride(dist),
                                        _ptr(in_label), label_stride, _ptr(label_offsets), rows, cols,
-                                       _ptr(out_dist), _ptr(out_label), out_dist.stride(0), k,
+                                       _ptr(out_dist), _ptr(out_label), _row_stride(out_dist), k,
                                        block_size, items_per_thread, 1 if prefetch else 0, _stream()))
     return out_dist, out_label
 
@@ -130,12 +137,12 @@ def distances(queries_dm, points_dm, op=DIST_L2, out=None):
     import torch
     d, q = queries_dm.shape
     d2, n = points_dm.shape
-    assert d == d2 and queries_dm.stride(1) == 1 and points_dm.stride(1) == 1
+    assert d == d2 and (q == 1 or queries_dm.stride(1) == 1) and (n == 1 or points_dm.stride(1) == 1)
     if out is None:
         out = torch.empty((q, n), dtype=torch.float32, device=queries_dm.device)
-    _check(lib().bitsknn_dist_f32(op, d, q, n, _ptr(queries_dm), queries_dm.stride(0),
-                                  _ptr(points_dm), points_dm.stride(0), _ptr(out), out.stride(0),
-                                  _stream()))
+    _check(lib().bitsknn_dist_f32(op, d, q, n, _ptr(queries_dm), _row_stride(queries_dm),
+                                  _ptr(points_dm), _row_stride(points_dm), _ptr(out),
+                                  _row_stride(out), _stream()))
     return out
 
 

@@ -1,0 +1,131 @@
+"""Parity of the distance kernels (through the C ABI) with the CPU oracle.
+
+Bars: BITSKNN_DIST_L2 bit-exact (sequential fused multiply-add, the reference's default
+distance); the MFMA kernels within 1e-5 relative of the oracle's partial distance measured
+against the magnitude of the terms (||p||^2 and 2|q.p| cancel), and the completed distance
+within the reference test's own tolerances (tests/distance/dist_test.hpp:93-115, 164-186).
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _dm(a, dev):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a.T)).to(dev)
+
+
+def _gpu_dist(bk, dev, queries, points, op):
+    import torch
+    out = bk.distances(_dm(queries, dev), _dm(points, dev), op)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+# shapes of the reference's distance tests (tests/distance/magma_dist_test.cpp:7-96,
+# cublas_dist_test.cpp:6-64): (points, queries, dim)
+REF_SHAPES = [(32, 32, 16), (128, 1, 16), (32, 32, 9), (1024, 32, 32), (23 * 1024, 1, 17), (64, 32, 2)]
+OUR_SHAPES = [(1000, 37, 1), (4097, 130, 3), (257, 129, 64), (5000, 200, 33), (300, 260, 100), (129, 5, 8)]
+
+
+@pytest.mark.parametrize("n,q,d", REF_SHAPES + OUR_SHAPES)
+def test_l2_is_bit_exact(bk, dev, oracle, n, q, d):
+    p, s = oracle.generate(42, n, q, d)
+    got = _gpu_dist(bk, dev, s, p, bk.DIST_L2)
+    exp = oracle.dist(s, p, "l2")
+    assert np.array_equal(got.view(np.uint32), exp.view(np.uint32))
+
+
+def test_l2_unaligned_strides(bk, dev, oracle):
+    import torch
+    p, s = oracle.generate(7, 1003, 45, 5)
+    pd = torch.zeros((5, 1009), device=dev)
+    qd = torch.zeros((5, 47), device=dev)
+    pd[:, 1:1004] = torch.from_numpy(np.ascontiguousarray(p.T)).to(dev)
+    qd[:, 2:47] = torch.from_numpy(np.ascontiguousarray(s.T)).to(dev)
+    out = torch.full((45, 1005), -1.0, device=dev)
+    bk.distances(qd[:, 2:47], pd[:, 1:1004], bk.DIST_L2, out=out[:, 1:1004])
+    torch.cuda.synchronize()
+    exp = oracle.dist(s, p, "l2")
+    assert np.array_equal(out[:, 1:1004].cpu().numpy(), exp)
+    assert (out[:, 0] == -1).all() and (out[:, 1004] == -1).all()
+
+
+@pytest.mark.parametrize("op", ["partial", "expanded"])
+@pytest.mark.parametrize("n,q,d", REF_SHAPES + OUR_SHAPES)
+def test_mfma_distances(bk, dev, oracle, n, q, d, op):
+    p, s = oracle.generate(42, n, q, d)
+    got = _gpu_dist(bk, dev, s, p, bk.DIST_PARTIAL_L2 if op == "partial" else bk.DIST_EXPANDED)
+    exp = oracle.dist(s, p, "partial")
+    truth = oracle.dist(s, p, "f64-partial")
+    # scale of the cancelling terms: ||p||^2 + 2|q.p| <= ||p||^2 + ||q||^2 + ||p||^2
+    scale = (p.astype(np.float64) ** 2).sum(1)[None, :] * 2 + (s.astype(np.float64) ** 2).sum(1)[:, None]
+    assert np.max(np.abs(got - exp) / scale) < 1e-5
+    assert np.max(np.abs(got - truth) / scale) < 1e-5
+    # the reference's own check: add ||q||^2 on the CPU, compare with the plain triple loop at 1e-3
+    full = got.astype(np.float64) + (s.astype(np.float64) ** 2).sum(1)[:, None]
+    ref_full = oracle.dist(s, p, "f64")
+    assert np.allclose(full, ref_full, rtol=1e-3, atol=1e-5)
+
+
+def test_mfma_operand_orientation(bk, dev, oracle):
+    # one-hot vectors make every entry of q.p identify its (query, point, dimension): a transposed
+    # or mis-tiled operand cannot pass
+    n, q, d = 300, 200, 40
+    rng = np.random.default_rng(0)
+    p = np.zeros((n, d), dtype=np.float32)
+    s = np.zeros((q, d), dtype=np.float32)
+    p[np.arange(n), rng.integers(0, d, n)] = np.arange(1, n + 1, dtype=np.float32)
+    s[np.arange(q), rng.integers(0, d, q)] = np.arange(1, q + 1, dtype=np.float32) / 4
+    got = _gpu_dist(bk, dev, s, p, bk.DIST_PARTIAL_L2)
+    assert np.array_equal(got, oracle.dist(s, p, "partial"))  # all products exact in fp32
+
+
+def test_knn_through_both_distances_meets_the_recall_bar(bk, dev, oracle):
+    """GEMM distance + bits top-k (k = 64, d = 64): k-th neighbour distance within 1e-5 relative,
+    recall@k >= 0.999 against the reference arithmetic."""
+    import torch
+    n, q, d, k = 1 << 16, 256, 64, 64
+    p, s = oracle.generate(24, n, q, d)
+    dist = bk.distances(_dm(s, dev), _dm(p, dev), bk.DIST_PARTIAL_L2)
+    gd, gl = bk.topk_bits(dist, k, 256, 8)
+    torch.cuda.synchronize()
+    ed, el = oracle.topk(oracle.dist(s, p, "partial"), k)
+    gd, gl = gd.cpu().numpy(), gl.cpu().numpy()
+    recall = np.mean([len(set(a) & set(b)) / k for a, b in zip(gl, el)])
+    assert recall >= 0.999, recall
+    qn = (s.astype(np.float64) ** 2).sum(1)
+    full_g = gd[:, -1].astype(np.float64) + qn
+    full_e = ed[:, -1].astype(np.float64) + qn
+    assert np.max(np.abs(full_g - full_e) / full_e) < 1e-5
+    # and the top-k of the device matrix itself is bit-exact
+    od, ol = oracle.topk(dist.cpu().numpy(), k)
+    assert np.array_equal(gd, od) and np.array_equal(gl, ol)
+
+
+def test_golden_fused_run_checksums_via_two_phase(bk, dev, oracle, golden):
+    """Reference-held checksums of the fused runs (data/fused-*.err) reproduced by the two-phase
+    path on the device: exact L2 distances + bits top-k, query 0."""
+    import torch
+    checked = 0
+    for n, q, d in ((131072, 8192, 4), (131072, 8192, 8), (131072, 8192, 16), (262144, 4096, 16)):
+        p, s = oracle.generate(24, n, q, d)
+        dist = bk.distances(_dm(s[:8], dev), _dm(p, dev), bk.DIST_L2)
+        part = bk.distances(_dm(s[:8], dev), _dm(p, dev), bk.DIST_PARTIAL_L2)
+        for rec in golden:
+            if rec["family"] != "fused" or (rec["n"], rec["q"], rec["d"]) != (n, q, d):
+                continue
+            for m in (dist, part):
+                _, gl = bk.topk_bits(m, rec["k"], 256, 8)
+                torch.cuda.synchronize()
+                assert str(oracle.checksum(gl[0].cpu().numpy())) in rec["checksums"], rec
+            checked += 1
+    assert checked >= 24
+
+
+def test_dist_errors(bk, dev):
+    import torch
+    a = torch.zeros((4, 10), device=dev)
+    with pytest.raises(bk.BitsKnnError, match="Unsupported distance"):
+        bk.distances(a, a, 7)
