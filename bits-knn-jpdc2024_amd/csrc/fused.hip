@@ -1,8 +1,450 @@
-// Fused distance + top-k kernel (placeholder until implemented).
+// bits-fused for gfx950: partial squared L2 distance (||p||^2 - 2 q.p) and top-k in one kernel.
+// The q x n distance matrix never leaves the registers of the wave that computes it.
+//
+// Replaces the reference's fused_cache_kernel
+// (include/bits/topk/singlepass/fused_cache_kernel_structs.cuh:663-800: distance tiles :315-632,
+// per-query buffers and merges :25-305).  Same phases -- distance tile, filter against the k-th
+// distance of each query, append to a per-query buffer, merge buffers into sorted top-k lists --
+// laid out for the matrix cores and 64-wide waves:
+//
+//  * A workgroup of 4 waves owns 128 queries (32 per wave) and walks over all points in stages of
+//    PT points.  A stage is written to LDS once as the MFMA A operand: rows 0..d-1 hold -2*p,
+//    one more row holds ||p||^2 (accumulated in dimension order), so that
+//    v_mfma_f32_32x32x2_f32 against the query fragment (q_0..q_{d-1}, 1) yields
+//    ||p||^2 - 2 q.p directly, with the dot product accumulated first and the norm added last.
+//  * The query fragment stays in registers for the whole kernel.  In the 32 x 32 result tile a
+//    lane holds 16 distances of ONE query (column), so the filter is a min-tree over 16
+//    registers and one compare against that query's radius.
+//  * Every query has a 32-slot buffer in LDS.  Slots are handed out without atomics: the two
+//    lanes that share a query exchange their pass counts, and the fill is kept in a register.
+//    Before a tile would overflow any buffer of the wave, the wave merges all its buffers.
+//  * The sorted top-k lists live in the output arrays themselves between merges (they are read
+//    and rewritten through L2 a few hundred times per query while 2^20 distances are computed).
+//    A merge sorts the buffers of 32 (or 16, 8 for large k) queries at once with a segmented
+//    bitonic network in registers, 2 (4, 8) lanes per query.
+//
+// Equal distances are ordered by lower point index: points are visited in index order, so a
+// value equal to a query's radius can never displace what is already merged.
+
+#include "bitonic_net.hpp"
 #include "common.hpp"
 
-extern "C" int bitsknn_fused_l2_topk_f32(const float*, const float*, int, int32_t, int32_t, float*,
-                                         int32_t*, int, int, int, int, int, int, void*)
+namespace bitsknn
 {
-    return bitsknn::fail(BITSKNN_ERR_UNSUPPORTED, "bitsknn_fused_l2_topk_f32: not implemented");
+namespace
+{
+
+typedef float vfloat16 __attribute__((ext_vector_type(16)));
+
+constexpr int FQ_WAVES = 4;                   // waves per workgroup
+constexpr int FQ_THREADS = FQ_WAVES * WAVE;   // 256
+constexpr int FQ_QW = 32;                     // queries per wave (one MFMA column tile)
+constexpr int FQ_QB = FQ_QW * FQ_WAVES;       // queries per workgroup
+constexpr int FQ_CAP = 32;                    // buffer slots per query (= points per MFMA tile)
+
+struct fused_args
+{
+    const float* queries; // dim-major, stride q
+    const float* points;  // dim-major, stride n
+    int dim;
+    int q;
+    int n;
+    float* out_dist;
+    std::int32_t* out_label;
+};
+
+// K: list length.  PT: points per stage; the 256 threads stage PT points x dim dimensions, so a
+// thread carries dim / (256 / PT) <= 32 values between its global loads and its LDS stores.
+template <int K, int PT>
+__global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
+{
+    constexpr int TPP = FQ_THREADS / PT;      // threads per point when staging
+    constexpr int MAX_DIM = 32 * TPP;         // largest supported dimension
+    constexpr int MAX_STEPS = MAX_DIM / 2 + 1; // MFMA steps of 2 dimensions, incl. the norm row
+    constexpr int MT = PT / 32;               // MFMA row tiles per stage
+    // merge layout: S keys per query spread over LPQ lanes, R keys per lane
+    constexpr int S = K > FQ_CAP ? K : FQ_CAP;
+    constexpr int LPQ = S / 32 > 2 ? S / 32 : 2;
+    constexpr int R = S / LPQ;
+    constexpr int QPP = WAVE / LPQ;           // queries per merge pass
+    constexpr int PASSES = FQ_QW / QPP;
+
+    extern __shared__ float lds[];
+    const int dim = a.dim;
+    const int rows = dim + 2 - (dim & 1);     // -2p rows, norm row, zero row when dim is even
+    const int steps = rows / 2;
+    float* const stage = lds;                                       // [rows][PT]
+    u64* const buffers = reinterpret_cast<u64*>(lds + static_cast<size_t>(rows) * PT);         // [waves][32][CAP]
+    float* const xchg = reinterpret_cast<float*>(buffers + FQ_WAVES * FQ_QW * FQ_CAP);        // [waves][64]
+
+    const int t = static_cast<int>(threadIdx.x);
+    const int lane = t & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(t / WAVE);
+    const int half = lane / 32;               // which of the two dimensions of an MFMA step
+    const int ql = lane & 31;                 // query of this lane inside the wave
+    const int wave_q0 = static_cast<int>(blockIdx.x) * FQ_QB + wave * FQ_QW;
+    const int my_q = wave_q0 + ql;
+    u64* const wbuf = buffers + static_cast<size_t>(wave) * FQ_QW * FQ_CAP;
+    float* const wx = xchg + wave * WAVE;     // 32 radii, then 32 fills (as int bits)
+    const int n = a.n;
+
+    // query fragment: step s of this lane is dimension 2s + half; dimension `dim` is the constant 1
+    float qf[MAX_STEPS];
+#pragma unroll
+    for (int s = 0; s < MAX_STEPS; ++s)
+    {
+        const int dd = 2 * s + half;
+        float val = 0.0F;
+        if (s < steps)
+        {
+            if (dd < dim)
+            {
+                val = my_q < a.q ? a.queries[static_cast<size_t>(dd) * a.q + my_q] : 0.0F;
+            }
+            else if (dd == dim)
+            {
+                val = 1.0F;
+            }
+        }
+        qf[s] = val;
+    }
+
+    float radius = __builtin_inff(); // k-th smallest distance of my query so far
+    int fill = 0;                    // used slots of my query's buffer (same in both lanes of a query)
+    bool have_list = false;          // wave-uniform: the lists in the output arrays are valid
+
+    // ---- merge of all buffers of this wave into the lists --------------------------------------
+    auto merge_event = [&]() {
+        reinterpret_cast<int*>(wx)[32 + ql] = fill;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll 1
+        for (int pass = 0; pass < PASSES; ++pass)
+        {
+            const int qm = pass * QPP + lane / LPQ; // query (inside the wave) of this lane group
+            const int sub = lane % LPQ;
+            const int gq = wave_q0 + qm;
+            const int used = reinterpret_cast<const int*>(wx)[32 + qm];
+            u64 buf[R];
+            u64 list[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+            {
+                const int i = sub * R + r;
+                buf[r] = i < used ? wbuf[qm * FQ_CAP + (i < FQ_CAP ? i : 0)] : PAD_KEY;
+                list[r] = PAD_KEY;
+                if (have_list && i < K && gq < a.q)
+                {
+                    const size_t at = static_cast<size_t>(gq) * K + i;
+                    const float dv = __hip_atomic_load(a.out_dist + at, __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT);
+                    const std::int32_t lv = __hip_atomic_load(a.out_label + at, __ATOMIC_RELAXED,
+                                                              __HIP_MEMORY_SCOPE_AGENT);
+                    list[r] = make_key(dv, lv);
+                }
+            }
+            // buffer descending, element-wise minimum with the ascending list, re-sort
+            net_sort<LPQ, R, 2, true>(buf, nullptr, sub);
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+            {
+                list[r] = buf[r] < list[r] ? buf[r] : list[r];
+            }
+            net_phase<LPQ, R, S, S / 2, false>(list, nullptr, sub);
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+            {
+                const int i = sub * R + r;
+                if (i < K && gq < a.q)
+                {
+                    const size_t at = static_cast<size_t>(gq) * K + i;
+                    __hip_atomic_store(a.out_dist + at, key_value(list[r]), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(a.out_label + at, key_label(list[r]), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                }
+                if (i == K - 1)
+                {
+                    wx[qm] = key_value(list[r]);
+                }
+            }
+        }
+        // the next merge of this wave reads the lists back with other lanes
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        radius = wx[ql];
+        fill = 0;
+        have_list = true;
+    };
+
+    // ---- staging: global -> registers -> LDS ---------------------------------------------------
+    // thread t carries dimensions (t / PT) + TPP*i of point t % PT
+    const int sp = t % PT;
+    const int sd0 = t / PT;
+    float pre[32];
+    auto fetch = [&](int base) {
+        const int j = base + sp;
+#pragma unroll
+        for (int i = 0; i < 32; ++i)
+        {
+            const int dd = sd0 + TPP * i;
+            pre[i] = 0.0F;
+            if (dd < dim && j < n)
+            {
+                pre[i] = a.points[static_cast<size_t>(dd) * n + j];
+            }
+        }
+    };
+    auto deposit = [&]() {
+#pragma unroll
+        for (int i = 0; i < 32; ++i)
+        {
+            const int dd = sd0 + TPP * i;
+            if (dd < dim)
+            {
+                stage[dd * PT + sp] = -2.0F * pre[i];
+            }
+        }
+    };
+    // ||p||^2 in dimension order from the staged -2p values (exact scaling by 4), by PT threads
+    auto norms = [&](int base) {
+        if (t < PT)
+        {
+            float acc4 = 0.0F;
+            for (int dd = 0; dd < dim; ++dd)
+            {
+                const float m2p = stage[dd * PT + t];
+                acc4 = __builtin_fmaf(m2p, m2p, acc4);
+            }
+            // points beyond the end get an infinite distance and never pass the filter
+            stage[dim * PT + t] = base + t < n ? 0.25F * acc4 : __builtin_inff();
+            if ((dim & 1) == 0)
+            {
+                stage[(dim + 1) * PT + t] = 0.0F;
+            }
+        }
+    };
+
+    fetch(0);
+    for (int base = 0; base < n; base += PT)
+    {
+        __syncthreads(); // everyone is done reading the previous stage
+        deposit();
+        __syncthreads();
+        norms(base);
+        if (base + PT < n)
+        {
+            fetch(base + PT); // in flight while this stage is multiplied
+        }
+        __syncthreads();
+
+#pragma unroll 1
+        for (int mt = 0; mt < MT; ++mt)
+        {
+            vfloat16 acc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+            {
+                acc[r] = 0.0F;
+            }
+            const float* arow = stage + half * PT + mt * 32 + ql;
+#pragma unroll
+            for (int s = 0; s < MAX_STEPS; ++s)
+            {
+                if (s < steps)
+                {
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(arow[2 * s * PT], qf[s], acc, 0, 0, 0);
+                }
+            }
+
+            // filter: lane holds 16 distances of query ql (rows 8*(r/4) + 4*half + r%4)
+            float smallest = acc[0];
+#pragma unroll
+            for (int r = 1; r < 16; ++r)
+            {
+                smallest = fminf(smallest, acc[r]);
+            }
+            if (__builtin_amdgcn_ballot_w64(smallest < radius) != 0)
+            {
+                int mine = 0;
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                {
+                    mine += acc[r] < radius ? 1 : 0;
+                }
+                int other = __shfl_xor(mine, 32, WAVE);
+                if (__builtin_amdgcn_ballot_w64(fill + mine + other > FQ_CAP) != 0)
+                {
+                    merge_event();
+                    mine = 0;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                    {
+                        mine += acc[r] < radius ? 1 : 0;
+                    }
+                    other = __shfl_xor(mine, 32, WAVE);
+                }
+                int slot = fill + (half != 0 ? other : 0);
+                const int first_point = base + mt * 32 + 4 * half;
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                {
+                    if (acc[r] < radius)
+                    {
+                        wbuf[ql * FQ_CAP + slot] = make_key(acc[r], first_point + 8 * (r / 4) + (r % 4));
+                        ++slot;
+                    }
+                }
+                fill += mine + other;
+            }
+        }
+    }
+
+    // whatever is left in the buffers; also writes the lists of queries that never merged
+    merge_event();
+}
+
+template <int K, int PT>
+hipError_t launch_fused(const fused_args& a, hipStream_t stream)
+{
+    const int rows = a.dim + 2 - (a.dim & 1);
+    const size_t lds_bytes = static_cast<size_t>(rows) * PT * sizeof(float) +
+                             static_cast<size_t>(FQ_WAVES) * FQ_QW * FQ_CAP * sizeof(u64) +
+                             static_cast<size_t>(FQ_WAVES) * WAVE * sizeof(float);
+    if (lds_bytes > 48 * 1024)
+    {
+        const hipError_t status =
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<K, PT>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+        if (status != hipSuccess)
+        {
+            return status;
+        }
+    }
+    const unsigned grid = static_cast<unsigned>((a.q + FQ_QB - 1) / FQ_QB);
+    hipLaunchKernelGGL((fused_kernel<K, PT>), dim3(grid), dim3(FQ_THREADS), lds_bytes, stream, a);
+    return hipGetLastError();
+}
+
+// points per stage by dimension: the stage ((dim + 2) x PT floats) stays near 25 KB of LDS
+template <int K>
+hipError_t launch_fused_k(const fused_args& a, hipStream_t stream)
+{
+    if (a.dim <= 16)
+    {
+        return launch_fused<K, 256>(a, stream);
+    }
+    if (a.dim <= 48)
+    {
+        return launch_fused<K, 128>(a, stream);
+    }
+    if (a.dim <= 112)
+    {
+        return launch_fused<K, 64>(a, stream);
+    }
+    return launch_fused<K, 32>(a, stream);
+}
+
+bool in_list(int v, std::initializer_list<int> values)
+{
+    for (const int x : values)
+    {
+        if (x == v)
+        {
+            return true;
+        }
+    }
+    return false;
+}
+
+} // namespace
+} // namespace bitsknn
+
+extern "C" int bitsknn_fused_l2_topk_f32(const float* queries_dim_major,
+                                         const float* points_dim_major, int dim, int32_t q,
+                                         int32_t n, float* out_dist, int32_t* out_label, int k,
+                                         int query_reg, int db_reg, int dim_reg, int block_query_dim,
+                                         int dim_mult, void* stream)
+{
+    using namespace bitsknn;
+    clear_error();
+    // the reference's nested dispatch, outermost first (fused_cache_knn.cu:72-144); the tuning
+    // parameters are validated like there although the MFMA tiling does not depend on them
+    if (!in_list(query_reg, {2, 4, 8, 16}))
+    {
+        return fail(BITSKNN_ERR_UNSUPPORTED, "Unsupported queries_reg value: %d", query_reg);
+    }
+    if (!in_list(db_reg, {4, 8, 16}))
+    {
+        return fail(BITSKNN_ERR_UNSUPPORTED, "Unsupported db_reg value: %d", db_reg);
+    }
+    if (!in_list(dim_reg, {1, 2, 4}))
+    {
+        return fail(BITSKNN_ERR_UNSUPPORTED, "Unsupported dim_reg value: %d", dim_reg);
+    }
+    if (!in_list(block_query_dim, {1, 2, 4}))
+    {
+        return fail(BITSKNN_ERR_UNSUPPORTED, "Unsupported query_block_size value: %d", block_query_dim);
+    }
+    if (!in_list(dim_mult, {1, 2, 4}))
+    {
+        return fail(BITSKNN_ERR_UNSUPPORTED, "Unsupported dim_mult value: %d", dim_mult);
+    }
+    if (!in_list(k, {4, 8, 16, 32, 64, 128, 256}))
+    {
+        return fail(BITSKNN_ERR_UNSUPPORTED, "Unsupported k value: %d", k);
+    }
+    if (dim < dim_mult * dim_reg)
+    {
+        return fail(BITSKNN_ERR_UNSUPPORTED, "Dimension of vectors must not be lower than %d, but is %d",
+                    dim_mult * dim_reg, dim);
+    }
+    if (dim > 256)
+    {
+        return fail(BITSKNN_ERR_UNSUPPORTED, "Unsupported dimension: %d (at most 256)", dim);
+    }
+    if (q <= 0)
+    {
+        return BITSKNN_OK;
+    }
+    if (n <= 0)
+    {
+        return fail(BITSKNN_ERR_INVALID, "bitsknn_fused_l2_topk_f32: no points");
+    }
+    if (queries_dim_major == nullptr || points_dim_major == nullptr || out_dist == nullptr ||
+        out_label == nullptr)
+    {
+        return fail(BITSKNN_ERR_INVALID, "bitsknn_fused_l2_topk_f32: null pointer");
+    }
+    const fused_args a{queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label};
+    auto* hip_stream = static_cast<hipStream_t>(stream);
+    hipError_t status = hipSuccess;
+    switch (k)
+    {
+    case 4:
+        status = launch_fused_k<4>(a, hip_stream);
+        break;
+    case 8:
+        status = launch_fused_k<8>(a, hip_stream);
+        break;
+    case 16:
+        status = launch_fused_k<16>(a, hip_stream);
+        break;
+    case 32:
+        status = launch_fused_k<32>(a, hip_stream);
+        break;
+    case 64:
+        status = launch_fused_k<64>(a, hip_stream);
+        break;
+    case 128:
+        status = launch_fused_k<128>(a, hip_stream);
+        break;
+    default:
+        status = launch_fused_k<256>(a, hip_stream);
+        break;
+    }
+    BITSKNN_HIP_CHECK(status);
+    return BITSKNN_OK;
 }

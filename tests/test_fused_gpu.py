@@ -1,0 +1,147 @@
+"""Parity of bits-fused (distance + top-k in one kernel, through the C ABI) with the CPU oracle.
+
+The distances come from fp32 MFMA, so they are not bit-identical to the reference's sequential
+fused multiply-adds.  Bar (the stated tolerance of this path): the k-th neighbour distance within
+1e-5 relative -- measured on the partial distance ||p||^2 - 2 q.p that the reference outputs,
+relative to the magnitude of the quantities it is the difference of (|value| + ||q||^2) -- and
+recall@k >= 0.999 against the oracle's neighbour sets.  Structure is checked exactly: ascending
+order, distinct in-range labels, and every reported distance equal (to the same tolerance) to the
+oracle's distance of the reported label.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+REL = 1e-5
+
+
+def _dm(a, dev):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a.T)).contiguous().to(dev)
+
+
+def _fused(bk, dev, points, queries, k, params=(8, 4, 2), bqd=1, dim_mult=1):
+    import torch
+    pd = _dm(points, dev).reshape(points.shape[1], points.shape[0])
+    qd = _dm(queries, dev).reshape(queries.shape[1], queries.shape[0])
+    od, ol = bk.fused_l2_topk(qd, pd, k, params, bqd, dim_mult)
+    torch.cuda.synchronize()
+    return od.cpu().numpy(), ol.cpu().numpy()
+
+
+def _check(oracle, points, queries, k, gd, gl, min_recall=0.999):
+    n = points.shape[0]
+    part = oracle.dist(queries, points, "partial")
+    ed, el = oracle.topk(part, k)
+    qn = (queries.astype(np.float64) ** 2).sum(1)[:, None]
+    kk = min(k, n)
+    # structure
+    assert np.all(gd[:, 1:kk] >= gd[:, :kk - 1]), "not ascending"
+    assert gl[:, :kk].min() >= 0 and gl[:, :kk].max() < n
+    for row in gl[:, :kk]:
+        assert len(set(row.tolist())) == kk, "duplicate labels"
+    # every reported distance is the distance of the reported label
+    ref_at = np.take_along_axis(part, gl[:, :kk].astype(np.int64), axis=1)
+    scale = np.abs(ref_at) + qn
+    assert np.max(np.abs(gd[:, :kk] - ref_at) / scale) <= REL
+    # k-th neighbour distance and recall
+    scale_k = np.abs(ed[:, kk - 1]) + qn[:, 0]
+    assert np.max(np.abs(gd[:, kk - 1] - ed[:, kk - 1]) / scale_k) <= REL
+    recall = np.mean([len(set(a[:kk]) & set(b[:kk])) / kk for a, b in zip(gl, el)])
+    assert recall >= min_recall, recall
+    # where the oracle's neighbour gaps are far above the rounding noise the sets must be identical
+    if n > kk:
+        nxt = np.sort(part, axis=1)[:, kk]
+        clear = (nxt - ed[:, kk - 1]) > 1e-4 * (np.abs(nxt) + qn[:, 0])
+        for r in np.nonzero(clear)[0]:
+            assert set(gl[r, :kk]) == set(el[r, :kk])
+    if k > n:
+        assert np.all(np.isinf(gd[:, n:]))
+    return recall
+
+
+# the reference's own fused-cache test cases (tests/topk/fused_cache_kernel_test.cu:12-82):
+# (dim, k, points, queries) with items {8,4,2}, block 4, deg 2
+@pytest.mark.parametrize("d,k,n,q", [(8, 32, 1024, 32), (16, 32, 1024, 1), (37, 32, 997, 43), (9, 16, 25, 7)])
+def test_reference_unit_test_shapes(bk, dev, oracle, d, k, n, q):
+    p, s = oracle.generate(42, n, q, d)
+    gd, gl = _fused(bk, dev, p, s, k, (8, 4, 2), 4, 2)
+    _check(oracle, p, s, k, gd, gl)
+
+
+@pytest.mark.parametrize("k", [4, 8, 16, 32, 64, 128, 256])
+@pytest.mark.parametrize("d", [4, 8, 16, 32])
+def test_all_k_values(bk, dev, oracle, k, d):
+    p, s = oracle.generate(100 + k + d, 20000, 150, d)
+    gd, gl = _fused(bk, dev, p, s, k)
+    _check(oracle, p, s, k, gd, gl)
+
+
+@pytest.mark.parametrize("d", [1, 2, 3, 5, 17, 33, 48, 49, 64, 100, 113, 200, 256])
+def test_dimensions(bk, dev, oracle, d):
+    p, s = oracle.generate(d, 3000, 70, d)
+    gd, gl = _fused(bk, dev, p, s, 16, (2, 4, 1), 1, 1)
+    _check(oracle, p, s, 16, gd, gl)
+
+
+@pytest.mark.parametrize("n,q", [(1, 1), (31, 5), (32, 33), (33, 127), (255, 128), (257, 129), (1000, 300), (5001, 1)])
+def test_ragged_counts(bk, dev, oracle, n, q):
+    p, s = oracle.generate(n + q, n, q, 8)
+    for k in (4, 32):
+        gd, gl = _fused(bk, dev, p, s, k)
+        _check(oracle, p, s, k, gd, gl)
+
+
+def test_duplicate_points_are_ordered_by_index(bk, dev, oracle):
+    # every point appears 4 times: equal distances must come out by ascending index
+    base, s = oracle.generate(5, 500, 64, 8)
+    p = np.concatenate([base, base, base, base])
+    gd, gl = _fused(bk, dev, p, s, 32)
+    part = oracle.dist(s, p, "partial")
+    ed, el = oracle.topk(part, 32)
+    assert np.array_equal(gl, el)
+
+
+def test_exact_arithmetic_is_bit_exact(bk, dev, oracle):
+    # small integers: every product and sum is exact in fp32, so the fused result must equal the
+    # oracle bit for bit, labels included (heavy ties)
+    rng = np.random.default_rng(3)
+    p = rng.integers(-8, 9, size=(4000, 12)).astype(np.float32)
+    s = rng.integers(-8, 9, size=(100, 12)).astype(np.float32)
+    gd, gl = _fused(bk, dev, p, s, 64)
+    ed, el = oracle.topk(oracle.dist(s, p, "partial"), 64)
+    assert np.array_equal(gd, ed) and np.array_equal(gl, el)
+
+
+# reference-held checksums of the fused runs (data/fused-*.err), query 0
+@pytest.mark.parametrize("n,q", [(131072, 8192), (262144, 4096)])
+def test_golden_fused_checksums(bk, dev, oracle, golden, n, q):
+    checked = 0
+    for d in (4, 8, 16):
+        p, s = oracle.generate(24, n, q, d)
+        part0 = oracle.dist(s[:64], p, "partial")
+        for rec in golden:
+            if rec["family"] != "fused" or (rec["n"], rec["q"], rec["d"]) != (n, q, d):
+                continue
+            k = rec["k"]
+            gd, gl = _fused(bk, dev, p, s, k)
+            assert str(oracle.checksum(gl[0])) in rec["checksums"], (rec, oracle.checksum(gl[0]))
+            _check(oracle, p, s[:64], k, gd[:64], gl[:64])
+            checked += 1
+    assert checked >= 18
+
+
+def test_parameter_validation(bk, dev):
+    import torch
+    qd = torch.zeros((8, 4), device=dev)
+    pd = torch.zeros((8, 100), device=dev)
+    for args, msg in (((qd, pd, 5), "Unsupported k value: 5"),
+                      ((qd, pd, 32, (3, 4, 2)), "Unsupported queries_reg value: 3"),
+                      ((qd, pd, 32, (8, 5, 2)), "Unsupported db_reg value: 5"),
+                      ((qd, pd, 32, (8, 4, 3)), "Unsupported dim_reg value: 3"),
+                      ((qd, pd, 32, (8, 4, 2), 3), "Unsupported query_block_size value: 3"),
+                      ((qd, pd, 32, (8, 4, 2), 1, 3), "Unsupported dim_mult value: 3"),
+                      ((qd, pd, 32, (8, 4, 4), 1, 4), "Dimension of vectors must not be lower than 16, but is 8")):
+        with pytest.raises(bk.BitsKnnError, match=msg):
+            bk.fused_l2_topk(*args)
