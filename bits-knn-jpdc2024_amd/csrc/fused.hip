@@ -53,60 +53,78 @@ struct fused_args
     std::int32_t* out_label;
 };
 
-// K: list length.  PT: points per stage; the 256 threads stage PT points x dim dimensions, so a
-// thread carries dim / (256 / PT) <= 32 values between its global loads and its LDS stores.
-template <int K, int PT>
+// stage geometry by padded dimension DP: PT points per stage, so that the stage
+// ((DP + 2) x PT floats) stays below 20 KB for DP <= 128
+template <int DP>
+struct fused_geometry
+{
+    static constexpr int PT = DP <= 16 ? 256 : (DP <= 32 ? 128 : (DP <= 64 ? 64 : 32));
+    static constexpr int ROWS = DP + 2;       // -2p rows (zero beyond dim), ||p||^2 row, zero row
+    static constexpr int STEPS = ROWS / 2;    // MFMA steps of 2 rows
+    static constexpr int TPP = FQ_THREADS / PT; // threads per point when staging
+    static constexpr int VPT = DP / TPP;      // values a thread carries from global memory to LDS
+    static constexpr int MT = PT / 32;        // MFMA row tiles per stage
+    static constexpr size_t lds_bytes()
+    {
+        return static_cast<size_t>(ROWS) * PT * sizeof(float) +
+               static_cast<size_t>(FQ_WAVES) * FQ_QW * FQ_CAP * sizeof(u64) +
+               static_cast<size_t>(FQ_WAVES) * WAVE * sizeof(float);
+    }
+};
+
+// K: list length.  DP: dimension padded to 8, 16, 32, 64, 128 or 256 (padding rows are zero on
+// both sides of the product).
+template <int K, int DP>
 __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 {
-    constexpr int TPP = FQ_THREADS / PT;      // threads per point when staging
-    constexpr int MAX_DIM = 32 * TPP;         // largest supported dimension
-    constexpr int MAX_STEPS = MAX_DIM / 2 + 1; // MFMA steps of 2 dimensions, incl. the norm row
-    constexpr int MT = PT / 32;               // MFMA row tiles per stage
+    using G = fused_geometry<DP>;
+    constexpr int PT = G::PT;
+    constexpr int STEPS = G::STEPS;
+    constexpr int TPP = G::TPP;
+    constexpr int VPT = G::VPT;
+    constexpr int MT = G::MT;
     // merge layout: S keys per query spread over LPQ lanes, R keys per lane
     constexpr int S = K > FQ_CAP ? K : FQ_CAP;
-    constexpr int LPQ = S / 32 > 2 ? S / 32 : 2;
-    constexpr int R = S / LPQ;
+    constexpr int R = 4;
+    constexpr int LPQ = S / R;
     constexpr int QPP = WAVE / LPQ;           // queries per merge pass
     constexpr int PASSES = FQ_QW / QPP;
 
     extern __shared__ float lds[];
-    const int dim = a.dim;
-    const int rows = dim + 2 - (dim & 1);     // -2p rows, norm row, zero row when dim is even
-    const int steps = rows / 2;
-    float* const stage = lds;                                       // [rows][PT]
-    u64* const buffers = reinterpret_cast<u64*>(lds + static_cast<size_t>(rows) * PT);         // [waves][32][CAP]
-    float* const xchg = reinterpret_cast<float*>(buffers + FQ_WAVES * FQ_QW * FQ_CAP);        // [waves][64]
+    float* const stage = lds;                                                           // [ROWS][PT]
+    u64* const buffers = reinterpret_cast<u64*>(lds + static_cast<size_t>(G::ROWS) * PT); // [waves][32][CAP]
+    float* const xchg = reinterpret_cast<float*>(buffers + FQ_WAVES * FQ_QW * FQ_CAP);  // [waves][64]
 
+    const int dim = a.dim;
+    const int n = a.n;
     const int t = static_cast<int>(threadIdx.x);
     const int lane = t & (WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(t / WAVE);
-    const int half = lane / 32;               // which of the two dimensions of an MFMA step
+    const int half = lane / 32;               // which of the two rows of an MFMA step
     const int ql = lane & 31;                 // query of this lane inside the wave
     const int wave_q0 = static_cast<int>(blockIdx.x) * FQ_QB + wave * FQ_QW;
     const int my_q = wave_q0 + ql;
     u64* const wbuf = buffers + static_cast<size_t>(wave) * FQ_QW * FQ_CAP;
     float* const wx = xchg + wave * WAVE;     // 32 radii, then 32 fills (as int bits)
-    const int n = a.n;
 
-    // query fragment: step s of this lane is dimension 2s + half; dimension `dim` is the constant 1
-    float qf[MAX_STEPS];
+    // query fragment: step s of this lane is row 2s + half; row DP multiplies the norm by 1
+    float qf[STEPS];
 #pragma unroll
-    for (int s = 0; s < MAX_STEPS; ++s)
+    for (int s = 0; s < STEPS; ++s)
     {
         const int dd = 2 * s + half;
-        float val = 0.0F;
-        if (s < steps)
+        float val = dd == DP ? 1.0F : 0.0F;
+        if (dd < dim && my_q < a.q)
         {
-            if (dd < dim)
-            {
-                val = my_q < a.q ? a.queries[static_cast<size_t>(dd) * a.q + my_q] : 0.0F;
-            }
-            else if (dd == dim)
-            {
-                val = 1.0F;
-            }
+            val = a.queries[static_cast<size_t>(dd) * a.q + my_q];
         }
         qf[s] = val;
+    }
+
+    // rows that never change: padding dimensions and the last row
+    for (int i = t; i < (G::ROWS - dim) * PT; i += FQ_THREADS)
+    {
+        stage[dim * PT + i] = 0.0F;
     }
 
     float radius = __builtin_inff(); // k-th smallest distance of my query so far
@@ -179,15 +197,59 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         have_list = true;
     };
 
+    // ---- filter one 32 x 32 tile held in `acc` and append what passes ---------------------------
+    // lane holds 16 distances of query ql: rows 8*(r/4) + 4*half + r%4 of the tile
+    auto filter_tile = [&](const vfloat16& acc, int tile_base) {
+        float smallest = acc[0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r)
+        {
+            smallest = fminf(smallest, acc[r]);
+        }
+        if (__builtin_amdgcn_ballot_w64(smallest < radius) != 0)
+        {
+            int mine = 0;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+            {
+                mine += acc[r] < radius ? 1 : 0;
+            }
+            int other = __shfl_xor(mine, 32, WAVE);
+            if (__builtin_amdgcn_ballot_w64(fill + mine + other > FQ_CAP) != 0)
+            {
+                merge_event();
+                mine = 0;
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                {
+                    mine += acc[r] < radius ? 1 : 0;
+                }
+                other = __shfl_xor(mine, 32, WAVE);
+            }
+            int slot = fill + (half != 0 ? other : 0);
+            const int first_point = tile_base + 4 * half;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+            {
+                if (acc[r] < radius)
+                {
+                    wbuf[ql * FQ_CAP + slot] = make_key(acc[r], first_point + 8 * (r / 4) + (r % 4));
+                    ++slot;
+                }
+            }
+            fill += mine + other;
+        }
+    };
+
     // ---- staging: global -> registers -> LDS ---------------------------------------------------
     // thread t carries dimensions (t / PT) + TPP*i of point t % PT
     const int sp = t % PT;
     const int sd0 = t / PT;
-    float pre[32];
+    float pre[VPT];
     auto fetch = [&](int base) {
         const int j = base + sp;
 #pragma unroll
-        for (int i = 0; i < 32; ++i)
+        for (int i = 0; i < VPT; ++i)
         {
             const int dd = sd0 + TPP * i;
             pre[i] = 0.0F;
@@ -199,7 +261,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     };
     auto deposit = [&]() {
 #pragma unroll
-        for (int i = 0; i < 32; ++i)
+        for (int i = 0; i < VPT; ++i)
         {
             const int dd = sd0 + TPP * i;
             if (dd < dim)
@@ -219,15 +281,13 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 acc4 = __builtin_fmaf(m2p, m2p, acc4);
             }
             // points beyond the end get an infinite distance and never pass the filter
-            stage[dim * PT + t] = base + t < n ? 0.25F * acc4 : __builtin_inff();
-            if ((dim & 1) == 0)
-            {
-                stage[(dim + 1) * PT + t] = 0.0F;
-            }
+            stage[DP * PT + t] = base + t < n ? 0.25F * acc4 : __builtin_inff();
         }
     };
 
     fetch(0);
+    // the query fragment and the first stage have arrived (nothing else is in flight yet)
+    __builtin_amdgcn_s_waitcnt(0x0F70);
     for (int base = 0; base < n; base += PT)
     {
         __syncthreads(); // everyone is done reading the previous stage
@@ -240,65 +300,47 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         }
         __syncthreads();
 
-#pragma unroll 1
-        for (int mt = 0; mt < MT; ++mt)
+        if constexpr (MT >= 2)
         {
-            vfloat16 acc;
+            // two row tiles at a time: two independent accumulator chains keep the matrix core
+            // issuing back to back
+#pragma unroll 1
+            for (int mt = 0; mt < MT; mt += 2)
+            {
+                vfloat16 acc0;
+                vfloat16 acc1;
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                {
+                    acc0[r] = 0.0F;
+                    acc1[r] = 0.0F;
+                }
+                const float* arow = stage + half * PT + mt * 32 + ql;
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s)
+                {
+                    acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(arow[2 * s * PT], qf[s], acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(arow[2 * s * PT + 32], qf[s], acc1, 0, 0, 0);
+                }
+                filter_tile(acc0, base + mt * 32);
+                filter_tile(acc1, base + mt * 32 + 32);
+            }
+        }
+        else
+        {
+            vfloat16 acc0;
 #pragma unroll
             for (int r = 0; r < 16; ++r)
             {
-                acc[r] = 0.0F;
+                acc0[r] = 0.0F;
             }
-            const float* arow = stage + half * PT + mt * 32 + ql;
+            const float* arow = stage + half * PT + ql;
 #pragma unroll
-            for (int s = 0; s < MAX_STEPS; ++s)
+            for (int s = 0; s < STEPS; ++s)
             {
-                if (s < steps)
-                {
-                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(arow[2 * s * PT], qf[s], acc, 0, 0, 0);
-                }
+                acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(arow[2 * s * PT], qf[s], acc0, 0, 0, 0);
             }
-
-            // filter: lane holds 16 distances of query ql (rows 8*(r/4) + 4*half + r%4)
-            float smallest = acc[0];
-#pragma unroll
-            for (int r = 1; r < 16; ++r)
-            {
-                smallest = fminf(smallest, acc[r]);
-            }
-            if (__builtin_amdgcn_ballot_w64(smallest < radius) != 0)
-            {
-                int mine = 0;
-#pragma unroll
-                for (int r = 0; r < 16; ++r)
-                {
-                    mine += acc[r] < radius ? 1 : 0;
-                }
-                int other = __shfl_xor(mine, 32, WAVE);
-                if (__builtin_amdgcn_ballot_w64(fill + mine + other > FQ_CAP) != 0)
-                {
-                    merge_event();
-                    mine = 0;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                    {
-                        mine += acc[r] < radius ? 1 : 0;
-                    }
-                    other = __shfl_xor(mine, 32, WAVE);
-                }
-                int slot = fill + (half != 0 ? other : 0);
-                const int first_point = base + mt * 32 + 4 * half;
-#pragma unroll
-                for (int r = 0; r < 16; ++r)
-                {
-                    if (acc[r] < radius)
-                    {
-                        wbuf[ql * FQ_CAP + slot] = make_key(acc[r], first_point + 8 * (r / 4) + (r % 4));
-                        ++slot;
-                    }
-                }
-                fill += mine + other;
-            }
+            filter_tile(acc0, base);
         }
     }
 
@@ -306,17 +348,14 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     merge_event();
 }
 
-template <int K, int PT>
+template <int K, int DP>
 hipError_t launch_fused(const fused_args& a, hipStream_t stream)
 {
-    const int rows = a.dim + 2 - (a.dim & 1);
-    const size_t lds_bytes = static_cast<size_t>(rows) * PT * sizeof(float) +
-                             static_cast<size_t>(FQ_WAVES) * FQ_QW * FQ_CAP * sizeof(u64) +
-                             static_cast<size_t>(FQ_WAVES) * WAVE * sizeof(float);
+    constexpr size_t lds_bytes = fused_geometry<DP>::lds_bytes();
     if (lds_bytes > 48 * 1024)
     {
         const hipError_t status =
-            hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<K, PT>),
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<K, DP>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
         if (status != hipSuccess)
         {
@@ -324,27 +363,34 @@ hipError_t launch_fused(const fused_args& a, hipStream_t stream)
         }
     }
     const unsigned grid = static_cast<unsigned>((a.q + FQ_QB - 1) / FQ_QB);
-    hipLaunchKernelGGL((fused_kernel<K, PT>), dim3(grid), dim3(FQ_THREADS), lds_bytes, stream, a);
+    hipLaunchKernelGGL((fused_kernel<K, DP>), dim3(grid), dim3(FQ_THREADS), lds_bytes, stream, a);
     return hipGetLastError();
 }
 
-// points per stage by dimension: the stage ((dim + 2) x PT floats) stays near 25 KB of LDS
 template <int K>
 hipError_t launch_fused_k(const fused_args& a, hipStream_t stream)
 {
+    if (a.dim <= 8)
+    {
+        return launch_fused<K, 8>(a, stream);
+    }
     if (a.dim <= 16)
     {
-        return launch_fused<K, 256>(a, stream);
+        return launch_fused<K, 16>(a, stream);
     }
-    if (a.dim <= 48)
+    if (a.dim <= 32)
     {
-        return launch_fused<K, 128>(a, stream);
+        return launch_fused<K, 32>(a, stream);
     }
-    if (a.dim <= 112)
+    if (a.dim <= 64)
     {
         return launch_fused<K, 64>(a, stream);
     }
-    return launch_fused<K, 32>(a, stream);
+    if (a.dim <= 128)
+    {
+        return launch_fused<K, 128>(a, stream);
+    }
+    return launch_fused<K, 256>(a, stream);
 }
 
 bool in_list(int v, std::initializer_list<int> values)
