@@ -1,0 +1,468 @@
+// Algorithms registered in the `knn` driver.  Each one mirrors the phases of its reference
+// counterpart (cited per class); all device work goes through the C ABI in bitsknn.h.
+#include "knn.hpp"
+
+#include <algorithm>
+#include <stdexcept>
+#include <utility>
+
+namespace
+{
+
+using knn_host::device_buffer;
+using knn_host::sync_default_stream;
+
+// dim-major copy (component t of vector v at [t*count + v]) of a matrix given in `layout`
+std::vector<float> to_dim_major(const float* data, std::size_t count, std::size_t dim,
+                                matrix_layout layout)
+{
+    std::vector<float> out(count * dim);
+    if (layout == matrix_layout::column_major)
+    {
+        std::copy(data, data + count * dim, out.begin());
+        return out;
+    }
+    for (std::size_t v = 0; v < count; ++v)
+    {
+        for (std::size_t t = 0; t < dim; ++t)
+        {
+            out[t * count + v] = data[v * dim + t];
+        }
+    }
+    return out;
+}
+
+float component(const float* data, std::size_t count, std::size_t dim, matrix_layout layout,
+                std::size_t v, std::size_t t)
+{
+    return layout == matrix_layout::row_major ? data[v * dim + t] : data[t * count + v];
+}
+
+} // namespace
+
+// ---------------------------------------------------------------------------------------------
+// distances (reference: src/distance/magma_distance.cu:13-103, cublas_distance.cu:104-186)
+// ---------------------------------------------------------------------------------------------
+
+void device_distance::prepare(const knn_args& args)
+{
+    args_ = args;
+    if (args_.dist_layout != matrix_layout::row_major)
+    {
+        throw std::runtime_error{"Only the row-major layout of the distance matrix is supported."};
+    }
+    const auto points = to_dim_major(args_.points, args_.point_count, args_.dim, args_.points_layout);
+    const auto queries = to_dim_major(args_.queries, args_.query_count, args_.dim, args_.queries_layout);
+    points_ = device_buffer<float>{args_.dim * args_.point_count};
+    queries_ = device_buffer<float>{args_.dim * args_.query_count};
+    dist_ = device_buffer<float>{args_.query_count * args_.point_count};
+    transfer_.start();
+    points_.upload(points.data(), points.size());
+    queries_.upload(queries.data(), queries.size());
+    sync_default_stream();
+    transfer_.stop();
+}
+
+void device_distance::compute()
+{
+    BITSKNN_CHECK(bitsknn_dist_f32(op_, static_cast<int>(args_.dim), args_.query_count,
+                                   args_.point_count, queries_.data(), args_.query_count,
+                                   points_.data(), args_.point_count, dist_.data(), args_.point_count,
+                                   nullptr));
+}
+
+const std::vector<float>& device_distance::matrix_cpu()
+{
+    dist_host_.resize(dist_.size());
+    dist_.download(dist_host_.data(), dist_host_.size());
+    sync_default_stream();
+    return dist_host_;
+}
+
+std::unique_ptr<device_distance> make_l2_distance()
+{
+    return std::make_unique<device_distance>(BITSKNN_DIST_L2, "magma-dist");
+}
+
+std::unique_ptr<device_distance> make_partial_l2_distance()
+{
+    return std::make_unique<device_distance>(BITSKNN_DIST_PARTIAL_L2, "magma-part-dist");
+}
+
+std::unique_ptr<device_distance> make_expanded_distance()
+{
+    return std::make_unique<device_distance>(BITSKNN_DIST_EXPANDED, "cublas-dist");
+}
+
+// ---------------------------------------------------------------------------------------------
+// base classes (reference: src/knn.cpp:11-31, src/cuda_knn.cpp:12-63)
+// ---------------------------------------------------------------------------------------------
+
+void knn::initialize(const knn_args& args)
+{
+    args_ = args;
+    args_.dist_layout = matrix_layout::row_major;
+    if (dist_impl_ == nullptr)
+    {
+        dist_impl_ = make_l2_distance(); // the default distance of every algorithm
+    }
+    dist_impl_->prepare(args_);
+}
+
+void knn::distances()
+{
+    dist_impl_->compute();
+    sync_default_stream();
+}
+
+void device_knn::allocate_outputs()
+{
+    out_dist_ = device_buffer<float>{query_count() * k()};
+    out_label_ = device_buffer<std::int32_t>{query_count() * k()};
+}
+
+void device_knn::initialize(const knn_args& args)
+{
+    knn::initialize(args);
+    allocate_outputs();
+}
+
+std::vector<distance_pair> device_knn::finish()
+{
+    if (no_output_)
+    {
+        transfer_out_.start();
+        transfer_out_.stop();
+        return {};
+    }
+    const std::size_t total = query_count() * k();
+    std::vector<float> dist(total);
+    std::vector<std::int32_t> label(total);
+    transfer_out_.start();
+    out_dist_.download(dist.data(), total);
+    out_label_.download(label.data(), total);
+    sync_default_stream();
+    transfer_out_.stop();
+    std::vector<distance_pair> result(total);
+    for (std::size_t i = 0; i < total; ++i)
+    {
+        result[i] = distance_pair{dist[i], label[i]};
+    }
+    return result;
+}
+
+namespace
+{
+
+// ---------------------------------------------------------------------------------------------
+// CPU reference algorithms (reference: src/topk/serial_knn.cpp:10-54, parallel_knn.cpp:12-67)
+// ---------------------------------------------------------------------------------------------
+
+// Full sort of every row of the device-computed distance matrix, by distance only.
+class serial_knn : public knn
+{
+public:
+    std::string id() const override { return "serial"; }
+
+    void prepare() override
+    {
+        rows_.clear();
+        rows_.reserve(point_count() * query_count());
+    }
+
+    void distances() override
+    {
+        knn::distances();
+        const auto& matrix = dist_impl_->matrix_cpu();
+        rows_.clear();
+        for (std::size_t i = 0; i < query_count(); ++i)
+        {
+            for (std::size_t j = 0; j < point_count(); ++j)
+            {
+                rows_.push_back(distance_pair{matrix[i * point_count() + j], static_cast<std::int32_t>(j)});
+            }
+        }
+    }
+
+    void selection() override
+    {
+        for (std::size_t i = 0; i < query_count(); ++i)
+        {
+            const auto first = rows_.begin() + static_cast<std::ptrdiff_t>(i * point_count());
+            std::sort(first, first + static_cast<std::ptrdiff_t>(point_count()),
+                      [](const distance_pair& a, const distance_pair& b) { return a.distance < b.distance; });
+        }
+    }
+
+    std::vector<distance_pair> finish() override
+    {
+        std::vector<distance_pair> result(query_count() * k());
+        for (std::size_t i = 0; i < query_count(); ++i)
+        {
+            std::copy_n(rows_.begin() + static_cast<std::ptrdiff_t>(i * point_count()), k(),
+                        result.begin() + static_cast<std::ptrdiff_t>(i * k()));
+        }
+        return result;
+    }
+
+private:
+    std::vector<distance_pair> rows_;
+};
+
+// OpenMP over the queries: size-k max-heap with strict admission, then a final sort.  The
+// distances (||p||^2 - 2 q.p, the quantity the reference's CPU distance computes with Eigen) are
+// computed on the host as well.
+class parallel_knn : public knn
+{
+public:
+    std::string id() const override { return "parallel"; }
+
+    void initialize(const knn_args& args) override
+    {
+        args_ = args;
+        args_.dist_layout = matrix_layout::row_major;
+    }
+
+    void prepare() override
+    {
+        result_.clear();
+        result_.resize(query_count() * k());
+    }
+
+    void distances() override
+    {
+        const std::size_t n = point_count();
+        const std::size_t q = query_count();
+        const std::size_t d = dim();
+        matrix_.resize(q * n);
+        std::vector<float> norm(n, 0.0F);
+        for (std::size_t j = 0; j < n; ++j)
+        {
+            for (std::size_t t = 0; t < d; ++t)
+            {
+                const float p = component(args_.points, n, d, args_.points_layout, j, t);
+                norm[j] += p * p;
+            }
+        }
+#pragma omp parallel for
+        for (std::size_t i = 0; i < q; ++i)
+        {
+            for (std::size_t j = 0; j < n; ++j)
+            {
+                float dot = 0;
+                for (std::size_t t = 0; t < d; ++t)
+                {
+                    dot += component(args_.queries, q, d, args_.queries_layout, i, t) *
+                           component(args_.points, n, d, args_.points_layout, j, t);
+                }
+                matrix_[i * n + j] = norm[j] - 2 * dot;
+            }
+        }
+    }
+
+    void selection() override
+    {
+        const auto less = [](const distance_pair& a, const distance_pair& b) { return a.distance < b.distance; };
+        const std::size_t n = point_count();
+        const std::size_t kk = k();
+#pragma omp parallel for
+        for (std::size_t i = 0; i < query_count(); ++i)
+        {
+            const float* row = matrix_.data() + i * n;
+            const auto heap_begin = result_.begin() + static_cast<std::ptrdiff_t>(i * kk);
+            const auto heap_end = heap_begin + static_cast<std::ptrdiff_t>(kk);
+            for (std::size_t j = 0; j < kk; ++j)
+            {
+                heap_begin[static_cast<std::ptrdiff_t>(j)] = distance_pair{row[j], static_cast<std::int32_t>(j)};
+            }
+            std::make_heap(heap_begin, heap_end, less);
+            for (std::size_t j = kk; j < n; ++j)
+            {
+                if (heap_begin->distance > row[j])
+                {
+                    std::pop_heap(heap_begin, heap_end, less);
+                    *(heap_end - 1) = distance_pair{row[j], static_cast<std::int32_t>(j)};
+                    std::push_heap(heap_begin, heap_end, less);
+                }
+            }
+            std::sort(heap_begin, heap_end, less);
+        }
+    }
+
+    std::vector<distance_pair> finish() override { return result_; }
+
+private:
+    std::vector<float> matrix_;
+    std::vector<distance_pair> result_;
+};
+
+// ---------------------------------------------------------------------------------------------
+// bits (reference: src/topk/singlepass/bits_knn.cu:29-186)
+// ---------------------------------------------------------------------------------------------
+
+class bits_knn : public device_knn
+{
+public:
+    explicit bits_knn(bool prefetch) : prefetch_(prefetch) {}
+    std::string id() const override { return prefetch_ ? "bits-prefetch" : "bits"; }
+
+    void selection() override
+    {
+        BITSKNN_CHECK(bitsknn_topk_bits_f32(
+            in_dist_gpu(), point_count(), nullptr, 0, nullptr, query_count(), point_count(),
+            out_dist_.data(), out_label_.data(), k(), static_cast<std::uint32_t>(k()),
+            static_cast<std::uint32_t>(args_.selection_block_size),
+            static_cast<std::uint32_t>(args_.items_per_thread[0]), prefetch_ ? 1 : 0, nullptr));
+        sync_default_stream();
+    }
+
+private:
+    bool prefetch_;
+};
+
+// `bits-sq`: every row is cut into --deg parts that are selected independently (labels shifted
+// by the part offset), then the deg*k partial results of a row are selected again with their
+// labels.
+class single_query_bits : public device_knn
+{
+public:
+    std::string id() const override { return "bits-sq"; }
+
+    void initialize(const knn_args& args) override
+    {
+        device_knn::initialize(args);
+        if (args_.deg > 1)
+        {
+            if (point_count() % args_.deg != 0)
+            {
+                throw std::runtime_error("bits-sq: the number of objects must be a multiple of --deg");
+            }
+            const std::size_t parts = query_count() * args_.deg;
+            tmp_dist_ = device_buffer<float>{parts * k()};
+            tmp_label_ = device_buffer<std::int32_t>{parts * k()};
+            offsets_ = device_buffer<std::int32_t>{parts};
+            BITSKNN_CHECK(bitsknn_label_offsets(offsets_.data(), query_count(), args_.deg,
+                                                point_count() / args_.deg, nullptr));
+        }
+    }
+
+    void selection() override
+    {
+        const auto block = static_cast<std::uint32_t>(args_.selection_block_size);
+        const auto batch = static_cast<std::uint32_t>(args_.items_per_thread[0]);
+        const auto kk = static_cast<std::uint32_t>(k());
+        if (args_.deg <= 1)
+        {
+            BITSKNN_CHECK(bitsknn_topk_bits_f32(in_dist_gpu(), point_count(), nullptr, 0, nullptr,
+                                                query_count(), point_count(), out_dist_.data(),
+                                                out_label_.data(), k(), kk, block, batch, 1, nullptr));
+        }
+        else
+        {
+            const std::size_t cols = point_count() / args_.deg;
+            const std::size_t parts = query_count() * args_.deg;
+            BITSKNN_CHECK(bitsknn_topk_bits_f32(in_dist_gpu(), cols, nullptr, 0, offsets_.data(), parts,
+                                                cols, tmp_dist_.data(), tmp_label_.data(), k(), kk,
+                                                block, batch, 1, nullptr));
+            const std::size_t merged = k() * args_.deg;
+            BITSKNN_CHECK(bitsknn_topk_bits_f32(tmp_dist_.data(), merged, tmp_label_.data(), merged,
+                                                nullptr, query_count(), merged, out_dist_.data(),
+                                                out_label_.data(), k(), kk, block, batch, 1, nullptr));
+        }
+        sync_default_stream();
+    }
+
+private:
+    device_buffer<float> tmp_dist_;
+    device_buffer<std::int32_t> tmp_label_;
+    device_buffer<std::int32_t> offsets_;
+};
+
+// ---------------------------------------------------------------------------------------------
+// bits-fused (reference: src/topk/singlepass/fused_cache_knn.cu:149-216)
+// ---------------------------------------------------------------------------------------------
+
+class fused_cache_knn : public device_knn
+{
+public:
+    std::string id() const override { return "fused-cache"; }
+
+    void initialize(const knn_args& args) override
+    {
+        // no distance matrix is allocated: the kernel never materialises it
+        args_ = args;
+        args_.dist_layout = matrix_layout::row_major;
+        allocate_outputs();
+        const auto points = to_dim_major(args_.points, point_count(), dim(), args_.points_layout);
+        const auto queries = to_dim_major(args_.queries, query_count(), dim(), args_.queries_layout);
+        points_ = device_buffer<float>{points.size()};
+        queries_ = device_buffer<float>{queries.size()};
+        transfer_in_.start();
+        points_.upload(points.data(), points.size());
+        queries_.upload(queries.data(), queries.size());
+        sync_default_stream();
+        transfer_in_.stop();
+    }
+
+    void distances() override {}
+
+    void selection() override
+    {
+        BITSKNN_CHECK(bitsknn_fused_l2_topk_f32(
+            queries_.data(), points_.data(), static_cast<int>(dim()), static_cast<std::int32_t>(query_count()),
+            static_cast<std::int32_t>(point_count()), out_dist_.data(), out_label_.data(),
+            static_cast<int>(k()), static_cast<int>(args_.items_per_thread[0]),
+            static_cast<int>(args_.items_per_thread[1]), static_cast<int>(args_.items_per_thread[2]),
+            static_cast<int>(args_.selection_block_size), static_cast<int>(args_.deg), nullptr));
+        sync_default_stream();
+    }
+
+    float transfer_in_seconds() const override { return transfer_in_.seconds(); }
+
+private:
+    device_buffer<float> points_;
+    device_buffer<float> queries_;
+    knn_host::transfer_timer transfer_in_;
+};
+
+// ---------------------------------------------------------------------------------------------
+// distance-only runs (reference: include/bits/distance/dist_runner.hpp:8-15)
+// ---------------------------------------------------------------------------------------------
+
+class dist_runner : public device_knn
+{
+public:
+    using factory = std::unique_ptr<device_distance> (*)();
+    dist_runner(std::string id, factory make) : id_(std::move(id)), make_(make) {}
+    std::string id() const override { return id_; }
+
+    void initialize(const knn_args& args) override
+    {
+        set_dist_impl(make_());
+        device_knn::initialize(args);
+        BITSKNN_CHECK(bitsknn_fill_f32(out_dist_.data(), out_dist_.size(), 0.0F, nullptr));
+        HIP_CHECK(hipMemsetAsync(out_label_.data(), 0, out_label_.size() * sizeof(std::int32_t), nullptr));
+        sync_default_stream();
+    }
+
+private:
+    std::string id_;
+    factory make_;
+};
+
+} // namespace
+
+std::vector<std::unique_ptr<knn>> make_algorithms()
+{
+    std::vector<std::unique_ptr<knn>> algorithms;
+    algorithms.push_back(std::make_unique<serial_knn>());
+    algorithms.push_back(std::make_unique<parallel_knn>());
+    algorithms.push_back(std::make_unique<bits_knn>(false));
+    algorithms.push_back(std::make_unique<bits_knn>(true));
+    algorithms.push_back(std::make_unique<single_query_bits>());
+    algorithms.push_back(std::make_unique<fused_cache_knn>());
+    algorithms.push_back(std::make_unique<dist_runner>("cublas-dist", &make_expanded_distance));
+    algorithms.push_back(std::make_unique<dist_runner>("magma-dist", &make_l2_distance));
+    algorithms.push_back(std::make_unique<dist_runner>("magma-part-dist", &make_partial_l2_distance));
+    return algorithms;
+}
