@@ -2,7 +2,8 @@
 """Benchmark of the k-NN hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--k 32] [--block-size 256]
-                    [--items-per-thread 16] [--sweep]
+                    [--items-per-thread 8] [--sweep] [--no-fused] [--no-cpu-baseline]
+                    [--copy-calibration]
 
 A step is one bits top-k pass (through the C ABI) over a resident 1024 x 1,048,576 fp32 matrix
 of i.i.d. uniform [0,1) values (4 GiB, generated on the device).  The printed JSON line follows
@@ -11,7 +12,9 @@ the reference's throughput convention: elements/s = rows*cols / mean step time
 bandwidth with its algorithmic bytes (4 B read per matrix element + 8 B written per output pair)
 over the kernel's mean duration measured with events on the launch stream.  `cpu_baseline` times
 the CPU restatement of the reference's parallel top-k (reference src/topk/parallel_knn.cpp:30-65)
-on the host cores, on a bounded sample.
+on the host cores, on a bounded sample.  `fused` reports the second headline figure, bits-fused
+queries/s at n = 2^20 points, q = 65,536 queries, d = 32, k = 32, priced against the fp32 MFMA peak
+with 2*q*n*d flops.
 """
 import argparse
 import json
@@ -23,7 +26,49 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "bits-knn-jpdc2024_amd"))
 
-HBM_PEAK_GBS = 8000.0  # MI355X published peak
+HBM_PEAK_GBS = 8000.0       # MI355X published peak
+MFMA_F32_PEAK_TFLOPS = 157.3  # dense fp32 matrix peak
+
+
+# HBM bytes per launch of the top-k kernel from two counter passes (FETCH_SIZE, WRITE_SIZE, each
+# scaled by what the counter reads for a plain 1 GiB copy), keyed by (rows, cols, k).  Measured
+# under a profiler, so it cannot be taken live; other workloads report null.
+MEASURED_TRAFFIC_BYTES = {(1024, 1 << 20, 32): 4295268223}
+
+
+def fused_headline(bitsknn, torch, dev, q=65536, n=1 << 20, d=32, k=32, runs=3):
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(24)
+    points = torch.rand((d, n), device=dev, generator=gen)
+    queries = torch.rand((d, q), device=dev, generator=gen)
+    out_d = torch.empty((q, k), dtype=torch.float32, device=dev)
+    out_l = torch.empty((q, k), dtype=torch.int32, device=dev)
+    bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l)
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(runs):
+        bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l)
+    end.record()
+    torch.cuda.synchronize()
+    seconds = start.elapsed_time(end) / 1e3 / runs
+    tflops = 2.0 * q * n * d / seconds / 1e12
+    return {"workload": f"bits-fused, {n} points x {q} queries, d={d}, k={k}, fp32 uniform[0,1)",
+            "queries_per_s": q / seconds, "ms": seconds * 1e3, "pairs_per_s": q * n / seconds,
+            "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_F32_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": tflops / MFMA_F32_PEAK_TFLOPS}}
+
+
+def copy_calibration(torch, dev, gib=1, reps=3):
+    """A plain device-to-device copy of known size, so that byte counters read under a profiler
+    can be scaled (bytes read = bytes written = gib GiB per copy)."""
+    src = torch.empty(gib << 28, dtype=torch.float32, device=dev).fill_(1.0)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    for _ in range(reps):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    return {"bytes_read_per_copy": gib << 30, "bytes_written_per_copy": gib << 30, "copies": reps}
 
 
 def topk_pass(bitsknn, torch, matrix, k, block, batch, prefetch, out_d, out_l, steps, warmup):
@@ -74,6 +119,9 @@ def main():
     ap.add_argument("--cols", type=int, default=1 << 20)
     ap.add_argument("--sweep", action="store_true", help="also time k x block-size combinations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-fused", action="store_true", help="skip the bits-fused headline figure")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run plain 1 GiB device copies (reference traffic for byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (--gpus 1); multi-GPU figures are not "
@@ -117,7 +165,8 @@ def main():
                                f"k={args.k}, block {args.block_size}, items/thread {args.items_per_thread}, "
                                f"prefetch {int(prefetch)}"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((rows, cols, args.k)),
                      "kernel_ms": kernel_s * 1e3, "algorithmic_bytes": bytes_alg},
     }
 
@@ -134,6 +183,10 @@ def main():
 
     del matrix
     torch.cuda.empty_cache()
+    if args.copy_calibration:
+        result["copy_calibration"] = copy_calibration(torch, dev)
+    if not args.no_fused:
+        result["fused"] = fused_headline(bitsknn, torch, dev)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(1024, 65536, 32)
     print(json.dumps(result))
