@@ -17,10 +17,50 @@
 namespace bitsknn
 {
 
-__device__ __forceinline__ u64 lane_xor(u64 x, int mask)
+// Value of `x` held by lane (lane ^ MASK), MASK a power of two below 64.  Distances 1, 2, 4 and 8
+// are data-parallel-primitive moves inside a row of 16 lanes (full VALU rate, no LDS); 16 and 32
+// use the row / half-wave swap instructions of gfx950.
+template <int MASK>
+__device__ __forceinline__ u32 lane_xor32(u32 x)
 {
-    const u32 lo = static_cast<u32>(__shfl_xor(static_cast<int>(static_cast<u32>(x)), mask, WAVE));
-    const u32 hi = static_cast<u32>(__shfl_xor(static_cast<int>(static_cast<u32>(x >> 32U)), mask, WAVE));
+    static_assert(MASK == 1 || MASK == 2 || MASK == 4 || MASK == 8 || MASK == 16 || MASK == 32);
+    const int v = static_cast<int>(x);
+    if constexpr (MASK == 1)
+    {
+        return static_cast<u32>(__builtin_amdgcn_mov_dpp(v, 0xB1, 0xF, 0xF, false)); // quad_perm [1,0,3,2]
+    }
+    else if constexpr (MASK == 2)
+    {
+        return static_cast<u32>(__builtin_amdgcn_mov_dpp(v, 0x4E, 0xF, 0xF, false)); // quad_perm [2,3,0,1]
+    }
+    else if constexpr (MASK == 4)
+    {
+        // lanes 0-3 and 8-11 of a row read 4 lanes up (row_shl:4), the others 4 lanes down
+        const int up = __builtin_amdgcn_update_dpp(v, v, 0x104, 0xF, 0x5, false);
+        return static_cast<u32>(__builtin_amdgcn_update_dpp(up, v, 0x114, 0xF, 0xA, false));
+    }
+    else if constexpr (MASK == 8)
+    {
+        return static_cast<u32>(__builtin_amdgcn_mov_dpp(v, 0x128, 0xF, 0xF, false)); // row_ror:8
+    }
+    else if constexpr (MASK == 16)
+    {
+        // swaps the odd 16-lane rows of the first copy with the even rows of the second
+        const auto swapped = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+        return (threadIdx.x & 16U) != 0 ? swapped[0] : swapped[1];
+    }
+    else
+    {
+        const auto swapped = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+        return (threadIdx.x & 32U) != 0 ? swapped[0] : swapped[1];
+    }
+}
+
+template <int MASK>
+__device__ __forceinline__ u64 lane_xor(u64 x)
+{
+    const u32 lo = lane_xor32<MASK>(static_cast<u32>(x));
+    const u32 hi = lane_xor32<MASK>(static_cast<u32>(x >> 32U));
     return (static_cast<u64>(hi) << 32U) | lo;
 }
 
@@ -70,7 +110,7 @@ __device__ __forceinline__ void net_step(u64 (&x)[IPT], u64* scratch, int t)
 #pragma unroll
             for (int r = 0; r < IPT; ++r)
             {
-                const u64 o = lane_xor(x[r], M);
+                const u64 o = lane_xor<M>(x[r]);
                 const bool take = (o < x[r]) == keep_min;
                 x[r] = take ? o : x[r];
             }
