@@ -59,6 +59,39 @@ def fused_headline(bitsknn, torch, dev, q=65536, n=1 << 20, d=32, k=32, runs=3):
                          "unit": "TFLOP/s", "frac": tflops / MFMA_F32_PEAK_TFLOPS}}
 
 
+def gemm_knn(bitsknn, torch, dev, q=4096, n=1 << 20, d=64, k=64, runs=3):
+    """Config 4: ||p||^2 - 2 q.p on MFMA into a q x n matrix (16 GiB), then bits top-k on it."""
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(24)
+    points = torch.rand((d, n), device=dev, generator=gen)
+    queries = torch.rand((d, q), device=dev, generator=gen)
+    dist = torch.empty((q, n), dtype=torch.float32, device=dev)
+    out_d = torch.empty((q, k), dtype=torch.float32, device=dev)
+    out_l = torch.empty((q, k), dtype=torch.int32, device=dev)
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(runs):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) / 1e3 / runs
+
+    t_dist = timed(lambda: bitsknn.distances(queries, points, bitsknn.DIST_PARTIAL_L2, out=dist))
+    t_topk = timed(lambda: bitsknn.topk_bits(dist, k, 256, 8, out_dist=out_d, out_label=out_l))
+    tflops = 2.0 * q * n * d / t_dist / 1e12
+    return {"workload": f"GEMM distance + bits, {n} points x {q} queries, d={d}, k={k}",
+            "distance_ms": t_dist * 1e3, "pairs_per_s": q * n / t_dist,
+            "distance_roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_F32_PEAK_TFLOPS,
+                                  "unit": "TFLOP/s", "frac": tflops / MFMA_F32_PEAK_TFLOPS,
+                                  "store_GBps": 4.0 * q * n / t_dist / 1e9},
+            "selection_ms": t_topk * 1e3, "selection_elements_per_s": q * n / t_topk,
+            "selection_hbm_frac": (4.0 * q * n + 8.0 * q * k) / t_topk / 1e9 / HBM_PEAK_GBS}
+
+
 def copy_calibration(torch, dev, gib=1, reps=3):
     """A plain device-to-device copy of known size, so that byte counters read under a profiler
     can be scaled (bytes read = bytes written = gib GiB per copy)."""
@@ -120,6 +153,9 @@ def main():
     ap.add_argument("--sweep", action="store_true", help="also time k x block-size combinations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fused", action="store_true", help="skip the bits-fused headline figure")
+    ap.add_argument("--no-topk", action="store_true", help="skip the top-k leg (profiling other kernels)")
+    ap.add_argument("--gemm-knn", action="store_true",
+                    help="also time config 4: MFMA distance matrix (16 GiB) + bits top-k")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run plain 1 GiB device copies (reference traffic for byte counters)")
     args = ap.parse_args()
@@ -133,11 +169,20 @@ def main():
     bitsknn.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    rows, cols = args.rows, args.cols
+    prefetch = args.prefetch
+    if args.no_topk:
+        result = {"metric": "bits top-k selected-from elements/s (rows*cols / step time)", "value": None,
+                  "unit": "elements/s", "n_gpus": 1, "config": {"workload": "top-k leg skipped"}}
+        if not args.no_fused:
+            result["fused"] = fused_headline(bitsknn, torch, dev, runs=max(1, args.steps))
+        if args.gemm_knn:
+            result["gemm_knn"] = gemm_knn(bitsknn, torch, dev)
+        print(json.dumps(result))
+        return
     gen = torch.Generator(device=dev)
     gen.manual_seed(24)
-    rows, cols = args.rows, args.cols
     matrix = torch.rand((rows, cols), device=dev, generator=gen)
-    prefetch = args.prefetch
 
     def run(k, block, batch, steps, warmup):
         out_d = torch.empty((rows, k), dtype=torch.float32, device=dev)
@@ -187,6 +232,8 @@ def main():
         result["copy_calibration"] = copy_calibration(torch, dev)
     if not args.no_fused:
         result["fused"] = fused_headline(bitsknn, torch, dev)
+    if args.gemm_knn:
+        result["gemm_knn"] = gemm_knn(bitsknn, torch, dev)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(1024, 65536, 32)
     print(json.dumps(result))

@@ -59,14 +59,18 @@ template <int DP>
 struct fused_geometry
 {
     static constexpr int PT = DP <= 16 ? 256 : (DP <= 32 ? 128 : (DP <= 64 ? 64 : 32));
-    static constexpr int ROWS = DP + 2;       // -2p rows (zero beyond dim), ||p||^2 row, zero row
-    static constexpr int STEPS = ROWS / 2;    // MFMA steps of 2 rows
     static constexpr int TPP = FQ_THREADS / PT; // threads per point when staging
+    // -2p rows (zero beyond dim), then one row per staging thread of a point with its share of
+    // ||p||^2 (at least two rows, so that the row count is even)
+    static constexpr int NORM_ROWS = TPP > 2 ? TPP : 2;
+    static constexpr int ROWS = DP + NORM_ROWS;
+    static constexpr int STEPS = ROWS / 2;    // MFMA steps of 2 rows
     static constexpr int VPT = DP / TPP;      // values a thread carries from global memory to LDS
     static constexpr int MT = PT / 32;        // MFMA row tiles per stage
     static constexpr size_t lds_bytes()
     {
-        return static_cast<size_t>(ROWS) * PT * sizeof(float) +
+        // two stages (one being multiplied, one being filled), the query buffers, exchange slots
+        return 2 * static_cast<size_t>(ROWS) * PT * sizeof(float) +
                static_cast<size_t>(FQ_WAVES) * FQ_QW * FQ_CAP * sizeof(u64) +
                static_cast<size_t>(FQ_WAVES) * WAVE * sizeof(float);
     }
@@ -91,8 +95,9 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     constexpr int PASSES = FQ_QW / QPP;
 
     extern __shared__ float lds[];
-    float* const stage = lds;                                                           // [ROWS][PT]
-    u64* const buffers = reinterpret_cast<u64*>(lds + static_cast<size_t>(G::ROWS) * PT); // [waves][32][CAP]
+    constexpr int STAGE_FLOATS = G::ROWS * PT;
+    float* const stages = lds;                                                    // [2][ROWS][PT]
+    u64* const buffers = reinterpret_cast<u64*>(lds + 2 * STAGE_FLOATS);          // [waves][32][CAP]
     float* const xchg = reinterpret_cast<float*>(buffers + FQ_WAVES * FQ_QW * FQ_CAP);  // [waves][64]
 
     const int dim = a.dim;
@@ -107,13 +112,13 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     u64* const wbuf = buffers + static_cast<size_t>(wave) * FQ_QW * FQ_CAP;
     float* const wx = xchg + wave * WAVE;     // 32 radii, then 32 fills (as int bits)
 
-    // query fragment: step s of this lane is row 2s + half; row DP multiplies the norm by 1
+    // query fragment: step s of this lane is row 2s + half; the norm rows are multiplied by 1
     float qf[STEPS];
 #pragma unroll
     for (int s = 0; s < STEPS; ++s)
     {
         const int dd = 2 * s + half;
-        float val = dd == DP ? 1.0F : 0.0F;
+        float val = dd >= DP ? 1.0F : 0.0F;
         if (dd < dim && my_q < a.q)
         {
             val = a.queries[static_cast<size_t>(dd) * a.q + my_q];
@@ -121,11 +126,12 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         qf[s] = val;
     }
 
-    // rows that never change: padding dimensions and the last row
-    for (int i = t; i < (G::ROWS - dim) * PT; i += FQ_THREADS)
+    // rows that never change in either stage: padding dimensions, unused norm rows
+    for (int i = t; i < 2 * STAGE_FLOATS; i += FQ_THREADS)
     {
-        stage[dim * PT + i] = 0.0F;
+        lds[i] = 0.0F;
     }
+    __syncthreads();
 
     float radius = __builtin_inff(); // k-th smallest distance of my query so far
     int fill = 0;                    // used slots of my query's buffer (same in both lanes of a query)
@@ -199,6 +205,38 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 
     // ---- filter one 32 x 32 tile held in `acc` and append what passes ---------------------------
     // lane holds 16 distances of query ql: rows 8*(r/4) + 4*half + r%4 of the tile
+    auto append_tile = [&](const vfloat16& acc, int tile_base) {
+        int mine = 0;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+        {
+            mine += acc[r] < radius ? 1 : 0;
+        }
+        int other = __shfl_xor(mine, 32, WAVE);
+        if (__builtin_amdgcn_ballot_w64(fill + mine + other > FQ_CAP) != 0)
+        {
+            merge_event();
+            mine = 0;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+            {
+                mine += acc[r] < radius ? 1 : 0;
+            }
+            other = __shfl_xor(mine, 32, WAVE);
+        }
+        int slot = fill + (half != 0 ? other : 0);
+        const int first_point = tile_base + 4 * half;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+        {
+            if (acc[r] < radius)
+            {
+                wbuf[ql * FQ_CAP + slot] = make_key(acc[r], first_point + 8 * (r / 4) + (r % 4));
+                ++slot;
+            }
+        }
+        fill += mine + other;
+    };
     auto filter_tile = [&](const vfloat16& acc, int tile_base) {
         float smallest = acc[0];
 #pragma unroll
@@ -208,98 +246,60 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         }
         if (__builtin_amdgcn_ballot_w64(smallest < radius) != 0)
         {
-            int mine = 0;
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-            {
-                mine += acc[r] < radius ? 1 : 0;
-            }
-            int other = __shfl_xor(mine, 32, WAVE);
-            if (__builtin_amdgcn_ballot_w64(fill + mine + other > FQ_CAP) != 0)
-            {
-                merge_event();
-                mine = 0;
-#pragma unroll
-                for (int r = 0; r < 16; ++r)
-                {
-                    mine += acc[r] < radius ? 1 : 0;
-                }
-                other = __shfl_xor(mine, 32, WAVE);
-            }
-            int slot = fill + (half != 0 ? other : 0);
-            const int first_point = tile_base + 4 * half;
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-            {
-                if (acc[r] < radius)
-                {
-                    wbuf[ql * FQ_CAP + slot] = make_key(acc[r], first_point + 8 * (r / 4) + (r % 4));
-                    ++slot;
-                }
-            }
-            fill += mine + other;
+            append_tile(acc, tile_base);
         }
     };
 
     // ---- staging: global -> registers -> LDS ---------------------------------------------------
-    // thread t carries dimensions (t / PT) + TPP*i of point t % PT
+    // thread t carries dimensions (t / PT) + TPP*i of point t % PT, turns them into -2p rows and
+    // adds up its share of ||p||^2 (the shares of a point meet inside the MFMA)
     const int sp = t % PT;
     const int sd0 = t / PT;
+    const bool whole_dim = dim == DP;
     float pre[VPT];
     auto fetch = [&](int base) {
-        const int j = base + sp;
-#pragma unroll
-        for (int i = 0; i < VPT; ++i)
+        if (whole_dim && base + PT <= n)
         {
-            const int dd = sd0 + TPP * i;
-            pre[i] = 0.0F;
-            if (dd < dim && j < n)
+            const float* __restrict__ src = a.points + static_cast<size_t>(sd0) * n + base + sp;
+#pragma unroll
+            for (int i = 0; i < VPT; ++i)
             {
-                pre[i] = a.points[static_cast<size_t>(dd) * n + j];
+                pre[i] = src[static_cast<size_t>(TPP * i) * n];
+            }
+        }
+        else
+        {
+            const int j = base + sp;
+#pragma unroll
+            for (int i = 0; i < VPT; ++i)
+            {
+                const int dd = sd0 + TPP * i;
+                pre[i] = 0.0F;
+                if (dd < dim && j < n)
+                {
+                    pre[i] = a.points[static_cast<size_t>(dd) * n + j];
+                }
             }
         }
     };
-    auto deposit = [&]() {
+    auto deposit = [&](float* stage, int base) {
+        float share = 0.0F;
 #pragma unroll
         for (int i = 0; i < VPT; ++i)
         {
             const int dd = sd0 + TPP * i;
-            if (dd < dim)
+            share = __builtin_fmaf(pre[i], pre[i], share);
+            if (whole_dim || dd < dim)
             {
                 stage[dd * PT + sp] = -2.0F * pre[i];
             }
         }
-    };
-    // ||p||^2 in dimension order from the staged -2p values (exact scaling by 4), by PT threads
-    auto norms = [&](int base) {
-        if (t < PT)
-        {
-            float acc4 = 0.0F;
-            for (int dd = 0; dd < dim; ++dd)
-            {
-                const float m2p = stage[dd * PT + t];
-                acc4 = __builtin_fmaf(m2p, m2p, acc4);
-            }
-            // points beyond the end get an infinite distance and never pass the filter
-            stage[DP * PT + t] = base + t < n ? 0.25F * acc4 : __builtin_inff();
-        }
+        // points beyond the end get an infinite distance and never pass the filter
+        stage[(DP + sd0) * PT + sp] = base + sp < n ? share : __builtin_inff();
     };
 
-    fetch(0);
-    // the query fragment and the first stage have arrived (nothing else is in flight yet)
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    for (int base = 0; base < n; base += PT)
-    {
-        __syncthreads(); // everyone is done reading the previous stage
-        deposit();
-        __syncthreads();
-        norms(base);
-        if (base + PT < n)
-        {
-            fetch(base + PT); // in flight while this stage is multiplied
-        }
-        __syncthreads();
-
+    // all row tiles of a stage: distances, filter, append
+    auto multiply = [&](const float* stage, int base) {
         if constexpr (MT >= 2)
         {
             // two row tiles at a time: two independent accumulator chains keep the matrix core
@@ -342,6 +342,35 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             }
             filter_tile(acc0, base);
         }
+    };
+
+    // Stage s is multiplied while stage s+1 sits in registers and is written to the other LDS
+    // buffer afterwards; stage s+2 is requested from memory right after that.  One barrier per
+    // stage: it separates the last read of a buffer from its next fill and the fill from its
+    // first read.
+    fetch(0);
+    // the query fragment and the first stage have arrived (nothing else is in flight yet)
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    deposit(stages, 0);
+    if (PT < n)
+    {
+        fetch(PT);
+    }
+    __syncthreads();
+    int parity = 0;
+    for (int base = 0; base < n; base += PT)
+    {
+        multiply(stages + parity * STAGE_FLOATS, base);
+        parity ^= 1;
+        if (base + PT < n)
+        {
+            deposit(stages + parity * STAGE_FLOATS, base + PT);
+            if (base + 2 * PT < n)
+            {
+                fetch(base + 2 * PT);
+            }
+        }
+        __syncthreads();
     }
 
     // whatever is left in the buffers; also writes the lists of queries that never merged
