@@ -24,6 +24,8 @@ EXPORTS = (
     "bitsknn_fill_f32",
     "bitsknn_dist_f32",
     "bitsknn_fused_l2_topk_f32",
+    "bitsknn_fused_workspace_bytes",
+    "bitsknn_fused_l2_topk_f32_ws",
 )
 
 
@@ -67,6 +69,12 @@ def lib():
         L.bitsknn_fused_l2_topk_f32.argtypes = [vp, vp, ctypes.c_int, i32, i32, vp, vp, ctypes.c_int,
                                                 ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                 ctypes.c_int, ctypes.c_int, vp]
+        L.bitsknn_fused_workspace_bytes.restype = ctypes.c_size_t
+        L.bitsknn_fused_workspace_bytes.argtypes = [i32, i32, ctypes.c_int]
+        L.bitsknn_fused_l2_topk_f32_ws.restype = ctypes.c_int
+        L.bitsknn_fused_l2_topk_f32_ws.argtypes = [vp, vp, ctypes.c_int, i32, i32, vp, vp, ctypes.c_int,
+                                                   ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                   ctypes.c_int, ctypes.c_int, vp, sz, vp]
         _lib = L
     return _lib
 
@@ -147,8 +155,10 @@ def distances(queries_dm, points_dm, op=DIST_L2, out=None):
 
 
 def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1, dim_mult=1,
-                  out_dist=None, out_label=None):
-    """bits-fused: top-k of ||p||^2 - 2 q.p without materialising the distance matrix."""
+                  out_dist=None, out_label=None, workspace=None):
+    """bits-fused: top-k of ||p||^2 - 2 q.p without materialising the distance matrix.
+    workspace: None -> the plain entry point; "auto" -> allocate what
+    bitsknn_fused_workspace_bytes asks for; or a uint8 device tensor."""
     import torch
     d, q = queries_dm.shape
     d2, n = points_dm.shape
@@ -157,7 +167,21 @@ def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1,
         out_dist = torch.empty((q, k), dtype=torch.float32, device=queries_dm.device)
     if out_label is None:
         out_label = torch.empty((q, k), dtype=torch.int32, device=queries_dm.device)
-    _check(lib().bitsknn_fused_l2_topk_f32(_ptr(queries_dm), _ptr(points_dm), d, q, n,
-                                           _ptr(out_dist), _ptr(out_label), k, params[0], params[1],
-                                           params[2], block_query_dim, dim_mult, _stream()))
+    if workspace is None:
+        _check(lib().bitsknn_fused_l2_topk_f32(_ptr(queries_dm), _ptr(points_dm), d, q, n,
+                                               _ptr(out_dist), _ptr(out_label), k, params[0],
+                                               params[1], params[2], block_query_dim, dim_mult,
+                                               _stream()))
+        return out_dist, out_label
+    if isinstance(workspace, str):
+        workspace = torch.empty(max(1, fused_workspace_bytes(q, n, k)), dtype=torch.uint8,
+                                device=queries_dm.device)
+    _check(lib().bitsknn_fused_l2_topk_f32_ws(_ptr(queries_dm), _ptr(points_dm), d, q, n,
+                                              _ptr(out_dist), _ptr(out_label), k, params[0],
+                                              params[1], params[2], block_query_dim, dim_mult,
+                                              _ptr(workspace), workspace.numel(), _stream()))
     return out_dist, out_label
+
+
+def fused_workspace_bytes(q, n, k):
+    return int(lib().bitsknn_fused_workspace_bytes(q, n, k))

@@ -49,8 +49,10 @@ struct fused_args
     int dim;
     int q;
     int n;
-    float* out_dist;
+    float* out_dist;      // lists: entry i of query g in split s at ((g * splits + s) * K + i)
     std::int32_t* out_label;
+    int splits;           // the points are cut into `splits` ranges, one per blockIdx.y
+    int split_points;     // points per range (a multiple of 256)
 };
 
 // stage geometry by padded dimension DP: PT points per stage, so that the stage
@@ -101,7 +103,10 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     float* const xchg = reinterpret_cast<float*>(buffers + FQ_WAVES * FQ_QW * FQ_CAP);  // [waves][64]
 
     const int dim = a.dim;
-    const int n = a.n;
+    // this workgroup's range of points
+    const int n_begin = static_cast<int>(blockIdx.y) * a.split_points;
+    const int n = a.n < n_begin + a.split_points ? a.n : n_begin + a.split_points;
+    const size_t total_points = static_cast<size_t>(a.n);
     const int t = static_cast<int>(threadIdx.x);
     const int lane = t & (WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(t / WAVE);
@@ -160,7 +165,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 list[r] = PAD_KEY;
                 if (have_list && i < K && gq < a.q)
                 {
-                    const size_t at = static_cast<size_t>(gq) * K + i;
+                    const size_t at = (static_cast<size_t>(gq) * a.splits + blockIdx.y) * K + i;
                     const float dv = __hip_atomic_load(a.out_dist + at, __ATOMIC_RELAXED,
                                                        __HIP_MEMORY_SCOPE_AGENT);
                     const std::int32_t lv = __hip_atomic_load(a.out_label + at, __ATOMIC_RELAXED,
@@ -182,7 +187,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 const int i = sub * R + r;
                 if (i < K && gq < a.q)
                 {
-                    const size_t at = static_cast<size_t>(gq) * K + i;
+                    const size_t at = (static_cast<size_t>(gq) * a.splits + blockIdx.y) * K + i;
                     __hip_atomic_store(a.out_dist + at, key_value(list[r]), __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
                     __hip_atomic_store(a.out_label + at, key_label(list[r]), __ATOMIC_RELAXED,
@@ -260,11 +265,11 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     auto fetch = [&](int base) {
         if (whole_dim && base + PT <= n)
         {
-            const float* __restrict__ src = a.points + static_cast<size_t>(sd0) * n + base + sp;
+            const float* __restrict__ src = a.points + static_cast<size_t>(sd0) * total_points + base + sp;
 #pragma unroll
             for (int i = 0; i < VPT; ++i)
             {
-                pre[i] = src[static_cast<size_t>(TPP * i) * n];
+                pre[i] = src[static_cast<size_t>(TPP * i) * total_points];
             }
         }
         else
@@ -277,7 +282,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 pre[i] = 0.0F;
                 if (dd < dim && j < n)
                 {
-                    pre[i] = a.points[static_cast<size_t>(dd) * n + j];
+                    pre[i] = a.points[static_cast<size_t>(dd) * total_points + j];
                 }
             }
         }
@@ -348,17 +353,17 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     // buffer afterwards; stage s+2 is requested from memory right after that.  One barrier per
     // stage: it separates the last read of a buffer from its next fill and the fill from its
     // first read.
-    fetch(0);
+    fetch(n_begin);
     // the query fragment and the first stage have arrived (nothing else is in flight yet)
     __builtin_amdgcn_s_waitcnt(0x0F70);
-    deposit(stages, 0);
-    if (PT < n)
+    deposit(stages, n_begin);
+    if (n_begin + PT < n)
     {
-        fetch(PT);
+        fetch(n_begin + PT);
     }
     __syncthreads();
     int parity = 0;
-    for (int base = 0; base < n; base += PT)
+    for (int base = n_begin; base < n; base += PT)
     {
         multiply(stages + parity * STAGE_FLOATS, base);
         parity ^= 1;
@@ -392,7 +397,8 @@ hipError_t launch_fused(const fused_args& a, hipStream_t stream)
         }
     }
     const unsigned grid = static_cast<unsigned>((a.q + FQ_QB - 1) / FQ_QB);
-    hipLaunchKernelGGL((fused_kernel<K, DP>), dim3(grid), dim3(FQ_THREADS), lds_bytes, stream, a);
+    hipLaunchKernelGGL((fused_kernel<K, DP>), dim3(grid, static_cast<unsigned>(a.splits)),
+                       dim3(FQ_THREADS), lds_bytes, stream, a);
     return hipGetLastError();
 }
 
@@ -437,13 +443,29 @@ bool in_list(int v, std::initializer_list<int> values)
 } // namespace
 } // namespace bitsknn
 
-extern "C" int bitsknn_fused_l2_topk_f32(const float* queries_dim_major,
-                                         const float* points_dim_major, int dim, int32_t q,
-                                         int32_t n, float* out_dist, int32_t* out_label, int k,
-                                         int query_reg, int db_reg, int dim_reg, int block_query_dim,
-                                         int dim_mult, void* stream)
+namespace bitsknn
 {
-    using namespace bitsknn;
+namespace
+{
+
+// Number of point ranges for a problem: enough workgroups for two per compute unit, ranges of at
+// least 4096 points and a multiple of 256, at most 64 ranges.
+int choose_splits(int q, int n)
+{
+    const int tiles = (q + FQ_QB - 1) / FQ_QB;
+    int splits = 1;
+    while (splits < 64 && tiles * splits < 512 && n / (splits * 2) >= 4096)
+    {
+        splits *= 2;
+    }
+    return splits;
+}
+
+int fused_impl(const float* queries_dim_major, const float* points_dim_major, int dim, std::int32_t q,
+               std::int32_t n, float* out_dist, std::int32_t* out_label, int k, int query_reg,
+               int db_reg, int dim_reg, int block_query_dim, int dim_mult, void* workspace,
+               size_t workspace_bytes, bool use_workspace, void* stream)
+{
     clear_error();
     // the reference's nested dispatch, outermost first (fused_cache_knn.cu:72-144); the tuning
     // parameters are validated like there although the MFMA tiling does not depend on them
@@ -493,7 +515,29 @@ extern "C" int bitsknn_fused_l2_topk_f32(const float* queries_dim_major,
     {
         return fail(BITSKNN_ERR_INVALID, "bitsknn_fused_l2_topk_f32: null pointer");
     }
-    const fused_args a{queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label};
+    if (static_cast<size_t>(q) > 65535U * FQ_QB)
+    {
+        return fail(BITSKNN_ERR_INVALID, "bitsknn_fused_l2_topk_f32: too many queries: %d", q);
+    }
+
+    int splits = use_workspace ? choose_splits(q, n) : 1;
+    const size_t pairs = static_cast<size_t>(q) * static_cast<size_t>(splits) * static_cast<size_t>(k);
+    if (splits > 1 && (workspace == nullptr || workspace_bytes < pairs * 8))
+    {
+        return fail(BITSKNN_ERR_INVALID,
+                    "bitsknn_fused_l2_topk_f32_ws: workspace of %zu bytes is too small, %zu needed",
+                    workspace_bytes, pairs * 8);
+    }
+    fused_args a{queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, 1, 0};
+    if (splits > 1)
+    {
+        // partial lists [q][splits][k] in the workspace: distances first, then labels
+        a.out_dist = static_cast<float*>(workspace);
+        a.out_label = reinterpret_cast<std::int32_t*>(a.out_dist + pairs);
+        a.splits = splits;
+    }
+    a.split_points = ((n + splits - 1) / splits + 255) / 256 * 256;
+
     auto* hip_stream = static_cast<hipStream_t>(stream);
     hipError_t status = hipSuccess;
     switch (k)
@@ -521,5 +565,49 @@ extern "C" int bitsknn_fused_l2_topk_f32(const float* queries_dim_major,
         break;
     }
     BITSKNN_HIP_CHECK(status);
+    if (splits > 1)
+    {
+        // one bits pass over the splits*k candidates of every query, labels carried along
+        const size_t cols = static_cast<size_t>(splits) * static_cast<size_t>(k);
+        return bitsknn_topk_bits_f32(a.out_dist, cols, a.out_label, cols, nullptr, static_cast<size_t>(q),
+                                     cols, out_dist, out_label, static_cast<size_t>(k),
+                                     static_cast<std::uint32_t>(k), 128, 4, 0, stream);
+    }
     return BITSKNN_OK;
+}
+
+} // namespace
+} // namespace bitsknn
+
+extern "C" int bitsknn_fused_l2_topk_f32(const float* queries_dim_major,
+                                         const float* points_dim_major, int dim, int32_t q,
+                                         int32_t n, float* out_dist, int32_t* out_label, int k,
+                                         int query_reg, int db_reg, int dim_reg, int block_query_dim,
+                                         int dim_mult, void* stream)
+{
+    return bitsknn::fused_impl(queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, k,
+                               query_reg, db_reg, dim_reg, block_query_dim, dim_mult, nullptr, 0, false,
+                               stream);
+}
+
+extern "C" size_t bitsknn_fused_workspace_bytes(int32_t q, int32_t n, int k)
+{
+    if (q <= 0 || n <= 0 || k <= 0)
+    {
+        return 0;
+    }
+    const int splits = bitsknn::choose_splits(q, n);
+    return splits > 1 ? static_cast<size_t>(q) * static_cast<size_t>(splits) * static_cast<size_t>(k) * 8 : 0;
+}
+
+extern "C" int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major,
+                                            const float* points_dim_major, int dim, int32_t q,
+                                            int32_t n, float* out_dist, int32_t* out_label, int k,
+                                            int query_reg, int db_reg, int dim_reg,
+                                            int block_query_dim, int dim_mult, void* workspace,
+                                            size_t workspace_bytes, void* stream)
+{
+    return bitsknn::fused_impl(queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, k,
+                               query_reg, db_reg, dim_reg, block_query_dim, dim_mult, workspace,
+                               workspace_bytes, true, stream);
 }

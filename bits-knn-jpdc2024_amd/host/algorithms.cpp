@@ -397,6 +397,9 @@ public:
         const auto queries = to_dim_major(args_.queries, query_count(), dim(), args_.queries_layout);
         points_ = device_buffer<float>{points.size()};
         queries_ = device_buffer<float>{queries.size()};
+        workspace_ = device_buffer<unsigned char>{bitsknn_fused_workspace_bytes(
+            static_cast<std::int32_t>(query_count()), static_cast<std::int32_t>(point_count()),
+            static_cast<int>(k()))};
         transfer_in_.start();
         points_.upload(points.data(), points.size());
         queries_.upload(queries.data(), queries.size());
@@ -408,12 +411,13 @@ public:
 
     void selection() override
     {
-        BITSKNN_CHECK(bitsknn_fused_l2_topk_f32(
+        BITSKNN_CHECK(bitsknn_fused_l2_topk_f32_ws(
             queries_.data(), points_.data(), static_cast<int>(dim()), static_cast<std::int32_t>(query_count()),
             static_cast<std::int32_t>(point_count()), out_dist_.data(), out_label_.data(),
             static_cast<int>(k()), static_cast<int>(args_.items_per_thread[0]),
             static_cast<int>(args_.items_per_thread[1]), static_cast<int>(args_.items_per_thread[2]),
-            static_cast<int>(args_.selection_block_size), static_cast<int>(args_.deg), nullptr));
+            static_cast<int>(args_.selection_block_size), static_cast<int>(args_.deg),
+            workspace_.data(), workspace_.size(), nullptr));
         sync_default_stream();
     }
 
@@ -422,6 +426,7 @@ public:
 private:
     device_buffer<float> points_;
     device_buffer<float> queries_;
+    device_buffer<unsigned char> workspace_; // partial lists when the points are split into ranges
     knn_host::transfer_timer transfer_in_;
 };
 

@@ -118,6 +118,25 @@ int bitsknn_fused_l2_topk_f32(const float* queries_dim_major, const float* point
                               int k, int query_reg, int db_reg, int dim_reg, int block_query_dim,
                               int dim_mult, void* stream);
 
+/*
+ * bits-fused with a caller-provided workspace.  Same results as bitsknn_fused_l2_topk_f32.
+ * When there are too few queries to fill the GPU with one workgroup per 128 queries, the points
+ * are cut into ranges that are searched by separate workgroups; their partial lists go to the
+ * workspace and one bits pass (explicit labels) selects the final k.
+ *
+ * No counterpart in the reference, whose fused kernel always runs one thread block per query tile
+ * (src/topk/singlepass/fused_cache_knn.cu:60-69); the host wrapper that owns the device memory
+ * (fused_cache_knn::initialize, fused_cache_knn.cu:149-195) is where the workspace is allocated.
+ *
+ * bitsknn_fused_workspace_bytes returns the size the call needs (0: no split, workspace unused).
+ * Errors as for bitsknn_fused_l2_topk_f32, plus BITSKNN_ERR_INVALID for a workspace too small.
+ */
+size_t bitsknn_fused_workspace_bytes(int32_t q, int32_t n, int k);
+int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major, const float* points_dim_major,
+                                 int dim, int32_t q, int32_t n, float* out_dist, int32_t* out_label,
+                                 int k, int query_reg, int db_reg, int dim_reg, int block_query_dim,
+                                 int dim_mult, void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

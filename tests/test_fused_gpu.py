@@ -21,11 +21,11 @@ def _dm(a, dev):
     return torch.from_numpy(np.ascontiguousarray(a.T)).contiguous().to(dev)
 
 
-def _fused(bk, dev, points, queries, k, params=(8, 4, 2), bqd=1, dim_mult=1):
+def _fused(bk, dev, points, queries, k, params=(8, 4, 2), bqd=1, dim_mult=1, workspace=None):
     import torch
     pd = _dm(points, dev).reshape(points.shape[1], points.shape[0])
     qd = _dm(queries, dev).reshape(queries.shape[1], queries.shape[0])
-    od, ol = bk.fused_l2_topk(qd, pd, k, params, bqd, dim_mult)
+    od, ol = bk.fused_l2_topk(qd, pd, k, params, bqd, dim_mult, workspace=workspace)
     torch.cuda.synchronize()
     return od.cpu().numpy(), ol.cpu().numpy()
 
@@ -91,6 +91,29 @@ def test_ragged_counts(bk, dev, oracle, n, q):
     for k in (4, 32):
         gd, gl = _fused(bk, dev, p, s, k)
         _check(oracle, p, s, k, gd, gl)
+
+
+@pytest.mark.parametrize("n,q,d,k", [(20000, 150, 8, 32), (70001, 300, 16, 16), (300000, 33, 32, 4),
+                                     (9000, 1000, 8, 64), (131072, 1024, 5, 128), (40000, 128, 8, 256)])
+def test_point_split_variant_with_workspace(bk, dev, oracle, n, q, d, k):
+    """The workspace entry point cuts the points into ranges when queries are few; its result must
+    equal the plain entry point's bit for bit (same distances, canonical ties)."""
+    p, s = oracle.generate(n + q + d, n, q, d)
+    assert bk.fused_workspace_bytes(q, n, k) % (8 * q * k) == 0
+    gd, gl = _fused(bk, dev, p, s, k, workspace="auto")
+    _check(oracle, p, s, k, gd, gl)
+    pd, pl = _fused(bk, dev, p, s, k)
+    assert np.array_equal(gd, pd) and np.array_equal(gl, pl)
+
+
+def test_workspace_too_small_is_rejected(bk, dev):
+    import torch
+    qd = torch.zeros((8, 256), device=dev)
+    pd = torch.zeros((8, 100000), device=dev)
+    need = bk.fused_workspace_bytes(256, 100000, 32)
+    assert need > 0
+    with pytest.raises(bk.BitsKnnError, match="workspace of"):
+        bk.fused_l2_topk(qd, pd, 32, workspace=torch.empty(need - 8, dtype=torch.uint8, device=dev))
 
 
 def test_duplicate_points_are_ordered_by_index(bk, dev, oracle):
