@@ -290,6 +290,215 @@ __global__ void __launch_bounds__(256)
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// ||p||^2 - 2 q.p on fp32 MFMA, query-resident form (dimensions up to 256).
+//
+// A workgroup of 4 waves owns QPW x 4 x 32 queries, whose fragments (q_0..q_{d-1}, 1, 1) stay in
+// registers as the MFMA A operand, and walks over a range of points in stages of PT.  A stage is
+// written to LDS once as the B operand: rows -2*p, then one row per staging thread of a point
+// with its share of ||p||^2, so the product IS the distance and the epilogue is a plain store.
+// In the 32 x 32 result a lane holds one point (column) and 16 queries (rows): for every register
+// the two half-waves write two full 128-byte segments of the row-major output.
+// ---------------------------------------------------------------------------------------------
+template <int DP>
+struct resident_geometry
+{
+    static constexpr int PT = DP <= 64 ? 128 : (DP <= 128 ? 64 : 32);
+    static constexpr int TPP = 256 / PT;                  // staging threads per point
+    static constexpr int NORM_ROWS = TPP > 2 ? TPP : 2;
+    static constexpr int ROWS = DP + NORM_ROWS;
+    static constexpr int STEPS = ROWS / 2;
+    static constexpr int VPT = DP / TPP;                  // staged values per thread
+    static constexpr int NT = PT / 32;                    // column tiles per stage
+    static constexpr int QPW = DP <= 64 ? 2 : 1;          // 32-query row tiles per wave
+    static constexpr int QB = 4 * 32 * QPW;               // queries per workgroup
+    static constexpr int RANGE = 4096;                    // points per workgroup
+};
+
+template <int DP>
+__global__ void __launch_bounds__(256)
+    dist_resident_kernel(int dim, size_t q, size_t n, const float* __restrict__ queries, size_t qs,
+                         const float* __restrict__ points, size_t ps, float* __restrict__ dist, size_t ds)
+{
+    using G = resident_geometry<DP>;
+    constexpr int PT = G::PT;
+    constexpr int TPP = G::TPP;
+    constexpr int STEPS = G::STEPS;
+    constexpr int VPT = G::VPT;
+    constexpr int QPW = G::QPW;
+    constexpr int STAGE_FLOATS = G::ROWS * PT;
+
+    __shared__ float stages[2 * STAGE_FLOATS];
+
+    const int t = static_cast<int>(threadIdx.x);
+    const int lane = t & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(t / WAVE);
+    const int half = lane / 32;
+    const int col = lane & 31;
+    const size_t wave_q0 = static_cast<size_t>(blockIdx.x) * G::QB + static_cast<size_t>(wave) * 32 * QPW;
+    const size_t j_begin = static_cast<size_t>(blockIdx.y) * G::RANGE;
+    const size_t j_end = j_begin + G::RANGE < n ? j_begin + G::RANGE : n;
+
+    // query fragments: step s of this lane is row 2s + half; the norm rows are multiplied by 1
+    float qf[QPW][STEPS];
+#pragma unroll
+    for (int a = 0; a < QPW; ++a)
+    {
+        const size_t i = wave_q0 + a * 32 + col;
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s)
+        {
+            const int dd = 2 * s + half;
+            float val = dd >= DP ? 1.0F : 0.0F;
+            if (dd < dim && i < q)
+            {
+                val = queries[static_cast<size_t>(dd) * qs + i];
+            }
+            qf[a][s] = val;
+        }
+    }
+
+    for (int i = t; i < 2 * STAGE_FLOATS; i += 256)
+    {
+        stages[i] = 0.0F;
+    }
+    __syncthreads();
+
+    const int sp = t % PT;
+    const int sd0 = t / PT;
+    const bool whole_dim = dim == DP;
+    float pre[VPT];
+    auto fetch = [&](size_t base) {
+        if (whole_dim && base + PT <= j_end)
+        {
+            const float* __restrict__ src = points + static_cast<size_t>(sd0) * ps + base + sp;
+#pragma unroll
+            for (int i = 0; i < VPT; ++i)
+            {
+                pre[i] = src[static_cast<size_t>(TPP * i) * ps];
+            }
+        }
+        else
+        {
+            const size_t j = base + sp;
+#pragma unroll
+            for (int i = 0; i < VPT; ++i)
+            {
+                const int dd = sd0 + TPP * i;
+                pre[i] = 0.0F;
+                if (dd < dim && j < j_end)
+                {
+                    pre[i] = points[static_cast<size_t>(dd) * ps + j];
+                }
+            }
+        }
+    };
+    auto deposit = [&](float* stage) {
+        float share = 0.0F;
+#pragma unroll
+        for (int i = 0; i < VPT; ++i)
+        {
+            const int dd = sd0 + TPP * i;
+            share = __builtin_fmaf(pre[i], pre[i], share);
+            if (whole_dim || dd < dim)
+            {
+                stage[dd * PT + sp] = -2.0F * pre[i];
+            }
+        }
+        stage[(DP + sd0) * PT + sp] = share;
+    };
+
+    auto multiply = [&](const float* stage, size_t base) {
+#pragma unroll 1
+        for (int nt = 0; nt < G::NT; ++nt)
+        {
+            vfloat16 acc[QPW];
+#pragma unroll
+            for (int a = 0; a < QPW; ++a)
+            {
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                {
+                    acc[a][r] = 0.0F;
+                }
+            }
+            const float* brow = stage + half * PT + nt * 32 + col;
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+            {
+                const float bv = brow[2 * s * PT];
+#pragma unroll
+                for (int a = 0; a < QPW; ++a)
+                {
+                    acc[a] = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[a][s], bv, acc[a], 0, 0, 0);
+                }
+            }
+            const size_t j = base + nt * 32 + col;
+            if (j < j_end)
+            {
+#pragma unroll
+                for (int a = 0; a < QPW; ++a)
+                {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                    {
+                        const size_t i = wave_q0 + a * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+                        if (i < q)
+                        {
+                            __builtin_nontemporal_store(acc[a][r], dist + i * ds + j);
+                        }
+                    }
+                }
+            }
+        }
+    };
+
+    if (j_begin >= j_end)
+    {
+        return;
+    }
+    fetch(j_begin);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    deposit(stages);
+    if (j_begin + PT < j_end)
+    {
+        fetch(j_begin + PT);
+    }
+    __syncthreads();
+    int parity = 0;
+    for (size_t base = j_begin; base < j_end; base += PT)
+    {
+        multiply(stages + parity * STAGE_FLOATS, base);
+        parity ^= 1;
+        if (base + PT < j_end)
+        {
+            deposit(stages + parity * STAGE_FLOATS);
+            if (base + 2 * PT < j_end)
+            {
+                fetch(base + 2 * PT);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <int DP>
+bool launch_resident(int dim, size_t q, size_t n, const float* queries, size_t qs, const float* points,
+                     size_t ps, float* dist, size_t ds, hipStream_t stream)
+{
+    using G = resident_geometry<DP>;
+    const size_t gx = (q + G::QB - 1) / G::QB;
+    const size_t gy = (n + G::RANGE - 1) / G::RANGE;
+    if (gx > 0x7FFFFFFFULL || gy > 65535)
+    {
+        return false;
+    }
+    hipLaunchKernelGGL(dist_resident_kernel<DP>, dim3(static_cast<unsigned>(gx), static_cast<unsigned>(gy)),
+                       dim3(256), 0, stream, dim, q, n, queries, qs, points, ps, dist, ds);
+    return true;
+}
+
 } // namespace
 } // namespace bitsknn
 
@@ -347,6 +556,38 @@ extern "C" int bitsknn_dist_f32(int op, int dim, size_t q, size_t n, const float
     }
     else
     {
+        bool launched = false;
+        if (dim <= 8)
+        {
+            launched = launch_resident<8>(dim, q, n, queries_dim_major, query_stride, points_dim_major,
+                                          point_stride, dist, dist_row_stride, hip_stream);
+        }
+        else if (dim <= 16)
+        {
+            launched = launch_resident<16>(dim, q, n, queries_dim_major, query_stride, points_dim_major,
+                                           point_stride, dist, dist_row_stride, hip_stream);
+        }
+        else if (dim <= 32)
+        {
+            launched = launch_resident<32>(dim, q, n, queries_dim_major, query_stride, points_dim_major,
+                                           point_stride, dist, dist_row_stride, hip_stream);
+        }
+        else if (dim <= 64)
+        {
+            launched = launch_resident<64>(dim, q, n, queries_dim_major, query_stride, points_dim_major,
+                                           point_stride, dist, dist_row_stride, hip_stream);
+        }
+        else if (dim <= 128)
+        {
+            launched = launch_resident<128>(dim, q, n, queries_dim_major, query_stride, points_dim_major,
+                                            point_stride, dist, dist_row_stride, hip_stream);
+        }
+        if (launched)
+        {
+            BITSKNN_HIP_CHECK(hipGetLastError());
+            return BITSKNN_OK;
+        }
+        // larger dimensions: the generic tiled kernel
         const size_t gx = (q + MM_TILE - 1) / MM_TILE;
         const size_t gy = (n + MM_TILE - 1) / MM_TILE;
         if (gx > 0x7FFFFFFFULL || gy > 65535)
