@@ -64,9 +64,47 @@ __device__ __forceinline__ u64 lane_xor(u64 x)
     return (static_cast<u64>(hi) << 32U) | lo;
 }
 
+// Whether bit X (a power of two) of the thread index `t` is set, as a per-lane predicate.  The
+// lane index is t % 64, so below 64 the answer is a constant lane mask that costs no vector
+// instruction; from 64 on it is the same for the whole wave.
+template <int X>
+__device__ __forceinline__ bool thread_bit(int t)
+{
+    static_assert(X > 0 && (X & (X - 1)) == 0);
+    if constexpr (X == 1)
+    {
+        return __builtin_amdgcn_inverse_ballot_w64(0xAAAAAAAAAAAAAAAAULL);
+    }
+    else if constexpr (X == 2)
+    {
+        return __builtin_amdgcn_inverse_ballot_w64(0xCCCCCCCCCCCCCCCCULL);
+    }
+    else if constexpr (X == 4)
+    {
+        return __builtin_amdgcn_inverse_ballot_w64(0xF0F0F0F0F0F0F0F0ULL);
+    }
+    else if constexpr (X == 8)
+    {
+        return __builtin_amdgcn_inverse_ballot_w64(0xFF00FF00FF00FF00ULL);
+    }
+    else if constexpr (X == 16)
+    {
+        return __builtin_amdgcn_inverse_ballot_w64(0xFFFF0000FFFF0000ULL);
+    }
+    else if constexpr (X == 32)
+    {
+        return __builtin_amdgcn_inverse_ballot_w64(0xFFFFFFFF00000000ULL);
+    }
+    else
+    {
+        return (__builtin_amdgcn_readfirstlane(t) & X) != 0;
+    }
+}
+
 // One compare-exchange layer of a bitonic network over N = BS*IPT keys held IPT per thread in
 // blocked order (thread t owns sorted positions t*IPT .. t*IPT+IPT-1).  K2 is the size of the
 // sequences being merged in this phase, J the exchange distance.  DESC flips the final order.
+// `t` must be the thread index whose low 6 bits are the lane index.
 template <int BS, int IPT, int K2, int J, bool DESC>
 __device__ __forceinline__ void net_step(u64 (&x)[IPT], u64* scratch, int t)
 {
@@ -86,7 +124,7 @@ __device__ __forceinline__ void net_step(u64 (&x)[IPT], u64* scratch, int t)
                 }
                 else if constexpr (K2 < N)
                 {
-                    down = (((t & (K2 / IPT)) != 0) != DESC);
+                    down = thread_bit<K2 / IPT>(t) != DESC;
                 }
                 const u64 a = x[r];
                 const u64 b = x[r | J];
@@ -102,9 +140,9 @@ __device__ __forceinline__ void net_step(u64 (&x)[IPT], u64* scratch, int t)
         bool down = DESC;
         if constexpr (K2 < N)
         {
-            down = (((t & (K2 / IPT)) != 0) != DESC);
+            down = thread_bit<K2 / IPT>(t) != DESC;
         }
-        const bool keep_min = (((t & M) == 0) != down);
+        const bool keep_min = thread_bit<M>(t) == down; // lower thread of the pair keeps the minimum when ascending
         if constexpr (M < WAVE)
         {
 #pragma unroll
