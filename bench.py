@@ -92,6 +92,25 @@ def gemm_knn(bitsknn, torch, dev, q=4096, n=1 << 20, d=64, k=64, runs=3):
             "selection_hbm_frac": (4.0 * q * n + 8.0 * q * k) / t_topk / 1e9 / HBM_PEAK_GBS}
 
 
+def hard_inputs(bitsknn, torch, dev, rows=16384, cols=65536, runs=5):
+    """Config 3: rows sorted ascending, descending, or drawn from 256 distinct values."""
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(24)
+    base = torch.rand((rows, cols), device=dev, generator=gen)
+    asc = torch.sort(base, dim=1).values
+    inputs = {"ascending": asc, "descending": torch.flip(asc, dims=[1]).contiguous(),
+              "256-values": torch.floor(base * 256) / 256}
+    out = []
+    for name, matrix in inputs.items():
+        for k in (32, 256):
+            out_d = torch.empty((rows, k), dtype=torch.float32, device=dev)
+            out_l = torch.empty((rows, k), dtype=torch.int32, device=dev)
+            _, kernel_s = topk_pass(bitsknn, torch, matrix, k, 128, 16, False, out_d, out_l, runs, 2)
+            out.append({"rows": name, "k": k, "block": 128, "elements_per_s": rows * cols / kernel_s,
+                        "hbm_frac": (4.0 * rows * cols + 8.0 * rows * k) / kernel_s / 1e9 / HBM_PEAK_GBS})
+    return out
+
+
 def copy_calibration(torch, dev, gib=1, reps=3):
     """A plain device-to-device copy of known size, so that byte counters read under a profiler
     can be scaled (bytes read = bytes written = gib GiB per copy)."""
@@ -156,6 +175,8 @@ def main():
     ap.add_argument("--no-topk", action="store_true", help="skip the top-k leg (profiling other kernels)")
     ap.add_argument("--gemm-knn", action="store_true",
                     help="also time config 4: MFMA distance matrix (16 GiB) + bits top-k")
+    ap.add_argument("--hard-inputs", action="store_true",
+                    help="also time config 3: 16384 x 65536 sorted / heavily tied rows, k = 32, 256")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run plain 1 GiB device copies (reference traffic for byte counters)")
     args = ap.parse_args()
@@ -234,6 +255,8 @@ def main():
         result["fused"] = fused_headline(bitsknn, torch, dev)
     if args.gemm_knn:
         result["gemm_knn"] = gemm_knn(bitsknn, torch, dev)
+    if args.hard_inputs:
+        result["hard_inputs"] = hard_inputs(bitsknn, torch, dev)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(1024, 65536, 32)
     print(json.dumps(result))

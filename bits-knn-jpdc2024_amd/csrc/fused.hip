@@ -7,11 +7,12 @@
 // distance of each query, append to a per-query buffer, merge buffers into sorted top-k lists --
 // laid out for the matrix cores and 64-wide waves:
 //
-//  * A workgroup of 4 waves owns 128 queries (32 per wave) and walks over all points in stages of
-//    PT points.  A stage is written to LDS once as the MFMA A operand: rows 0..d-1 hold -2*p,
-//    one more row holds ||p||^2 (accumulated in dimension order), so that
-//    v_mfma_f32_32x32x2_f32 against the query fragment (q_0..q_{d-1}, 1) yields
-//    ||p||^2 - 2 q.p directly, with the dot product accumulated first and the norm added last.
+//  * A workgroup of 4 waves owns 128 queries (32 per wave) and walks over its range of points in
+//    stages of PT points, two stages in LDS (one being multiplied, one being filled; one barrier
+//    per stage).  A stage is the MFMA A operand: rows 0..d-1 hold -2*p, the following rows hold
+//    the staging threads' shares of ||p||^2, so that v_mfma_f32_32x32x2_f32 against the query
+//    fragment (q_0..q_{d-1}, 1, 1) yields ||p||^2 - 2 q.p directly, the dot product accumulated
+//    first and the norm added last.
 //  * The query fragment stays in registers for the whole kernel.  In the 32 x 32 result tile a
 //    lane holds 16 distances of ONE query (column), so the filter is a min-tree over 16
 //    registers and one compare against that query's radius.
@@ -20,8 +21,10 @@
 //    Before a tile would overflow any buffer of the wave, the wave merges all its buffers.
 //  * The sorted top-k lists live in the output arrays themselves between merges (they are read
 //    and rewritten through L2 a few hundred times per query while 2^20 distances are computed).
-//    A merge sorts the buffers of 32 (or 16, 8 for large k) queries at once with a segmented
-//    bitonic network in registers, 2 (4, 8) lanes per query.
+//    A merge sorts the buffers of 8 (4, 2, 1 for larger k) queries at a time with a segmented
+//    bitonic network in registers, 4 keys per lane.
+//  * With few queries the points are cut into ranges (blockIdx.y) whose partial lists go to a
+//    caller-provided workspace and are reduced by one bits top-k pass with explicit labels.
 //
 // Equal distances are ordered by lower point index: points are visited in index order, so a
 // value equal to a query's radius can never displace what is already merged.
@@ -320,12 +323,23 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                     acc0[r] = 0.0F;
                     acc1[r] = 0.0F;
                 }
+                // all A operands of the pair are requested from LDS before the first MFMA, so the
+                // chain never waits for a read
                 const float* arow = stage + half * PT + mt * 32 + ql;
+                float a0[STEPS];
+                float a1[STEPS];
 #pragma unroll
                 for (int s = 0; s < STEPS; ++s)
                 {
-                    acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(arow[2 * s * PT], qf[s], acc0, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(arow[2 * s * PT + 32], qf[s], acc1, 0, 0, 0);
+                    a0[s] = arow[2 * s * PT];
+                    a1[s] = arow[2 * s * PT + 32];
+                }
+                __builtin_amdgcn_sched_barrier(0); // keep the reads above the chain
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s)
+                {
+                    acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[s], qf[s], acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[s], qf[s], acc1, 0, 0, 0);
                 }
                 filter_tile(acc0, base + mt * 32);
                 filter_tile(acc1, base + mt * 32 + 32);
