@@ -237,14 +237,22 @@ def main():
     }
 
     if args.sweep:
+        from bitsknn import tuning
         sweep = []
         for k in (16, 32, 128, 512, 2048):
             for block in (128, 256, 512):
                 if k // block > 16:
                     continue
                 s, ks = run(k, block, args.items_per_thread, max(5, args.steps // 2), 3)
-                sweep.append({"k": k, "block": block, "elements_per_s": rows * cols / s,
+                sweep.append({"k": k, "block": block, "items_per_thread": args.items_per_thread,
+                              "elements_per_s": rows * cols / s,
                               "hbm_frac": (4.0 * rows * cols + 8.0 * rows * k) / ks / 1e9 / HBM_PEAK_GBS})
+            # the configuration the shipped optima file names for this problem
+            block, _, batch, _, _ = tuning.config_algorithm("bits", rows, k)
+            s, ks = run(k, block, batch, max(5, args.steps // 2), 3)
+            sweep.append({"k": k, "block": block, "items_per_thread": batch, "tuned": True,
+                          "elements_per_s": rows * cols / s,
+                          "hbm_frac": (4.0 * rows * cols + 8.0 * rows * k) / ks / 1e9 / HBM_PEAK_GBS})
         result["sweep"] = sweep
 
     del matrix

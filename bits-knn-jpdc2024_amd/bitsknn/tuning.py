@@ -1,0 +1,168 @@
+"""Launch-parameter tuning for the bits kernels on one MI355X.
+
+Two halves, matching the reference's tuning workflow:
+
+* ``sweep()`` times `bits` and `bits-prefetch` over the grid of the reference's parameter search
+  (reference scripts/run-opt-ipt.sh:38-47: n = 512k, q in 64..8192, k in 2..2048, batch 1..16,
+  block size 128/256/512) and ``write_optima()`` keeps the fastest configuration of every
+  (algorithm, q, k) in a CSV with the columns of the reference's scripts/optima.csv
+  (hostname, GPU, algorithm, point_count, query_count, k, dim, block_size, items_per_thread,
+  items_per_thread2, items_per_thread3, deg, time), as scripts/plot-analyze-opt.py does.
+* ``config_algorithm()`` is the lookup the reference's run scripts perform on that file
+  (reference scripts/config.sh:97-214, ``config_generic`` / ``config_algorithm``): among the rows
+  of the algorithm (and host), prefer rows whose query_count / k / dim are not below the request,
+  and among those the row with the smallest product of ratios to the request.
+
+    python -m bitsknn.tuning --out optima.csv        # on a GPU box; about two minutes
+
+The timed matrix is generated on the device (uniform [0,1), as `knn -g uniform`); one
+8192 x 524288 matrix (16 GiB) serves every query count as a row prefix.
+"""
+import argparse
+import csv
+import os
+import sys
+
+OPTIMA_COLUMNS = ("hostname", "GPU", "algorithm", "point_count", "query_count", "k", "dim",
+                  "block_size", "items_per_thread", "items_per_thread2", "items_per_thread3",
+                  "deg", "time")
+DEFAULT_OPTIMA = os.path.join(os.path.dirname(os.path.abspath(__file__)), "optima.csv")
+
+QUERY_COUNTS = (64, 256, 512, 1024, 2048, 4096, 8192)
+K_VALUES = (2, 4, 8, 16, 32, 64, 128, 256, 512, 1024, 2048)
+BLOCK_SIZES = (128, 256, 512)
+BATCH_SIZES = tuple(range(1, 17))
+ALGORITHMS = (("bits", False), ("bits-prefetch", True))
+
+
+def config_algorithm(algorithm, query_count=None, k=None, dim=None, hostname=None,
+                     optima_file=DEFAULT_OPTIMA):
+    """(block_size, deg, items_per_thread, items_per_thread2, items_per_thread3) for a problem.
+
+    Restates the awk program of reference scripts/config.sh:103-200.  ``None`` for query_count,
+    k, dim or hostname means "do not care" (the script's literal "None").  Without a matching
+    row the defaults of the script are returned: (256, 1, 1, 1, 1).  A parameter that no row up
+    to the chosen one states comes back as None (an empty word in the script's output, which the
+    run scripts replace by their own default).
+    """
+    names = ("block_size", "deg", "items_per_thread", "items_per_thread2", "items_per_thread3")
+    best = {"block_size": 256, "deg": 1, "items_per_thread": 1, "items_per_thread2": 1,
+            "items_per_thread3": 1}
+    # the script keeps the last non-empty field it saw, row after row; a field it has not seen
+    # yet is empty (None here) and stays empty in the answer
+    carried = dict.fromkeys(names)
+    score, slack = 0, 0.0
+    with open(optima_file, newline="") as handle:
+        reader = csv.reader(handle)
+        header = next(reader, None)
+        if header is None or "algorithm" not in header or "hostname" not in header:
+            raise ValueError(f"{optima_file}: no algorithm/hostname columns")
+        col = {name: i for i, name in enumerate(header)}
+
+        def field(row, name):
+            i = col.get(name)
+            return row[i] if i is not None and i < len(row) else ""
+
+        for row in reader:
+            if field(row, "algorithm") != algorithm:
+                continue
+            if hostname is not None and field(row, "hostname") != hostname:
+                continue
+            new_score, new_slack = 0, 1.0
+            for name in names:
+                text = field(row, name)
+                if text != "":
+                    carried[name] = int(float(text))
+            for name, wanted in (("query_count", query_count), ("k", k), ("dim", dim)):
+                text = field(row, name)
+                if wanted is None or text == "":
+                    continue
+                have = float(text)
+                if have >= wanted:
+                    new_score += 1
+                    new_slack *= have / wanted
+                else:
+                    new_slack *= wanted / have
+            if new_score >= score and (slack == 0 or new_slack < slack):
+                score, slack = new_score, new_slack
+                best = dict(carried)
+    return (best["block_size"], best["deg"], best["items_per_thread"], best["items_per_thread2"],
+            best["items_per_thread3"])
+
+
+def sweep(repeats=10, point_count=512 * 1024, query_counts=QUERY_COUNTS, k_values=K_VALUES,
+          block_sizes=BLOCK_SIZES, batch_sizes=BATCH_SIZES, algorithms=ALGORITHMS, seed=17,
+          progress=None):
+    """Time every grid point on cuda:0; yields dict rows (seconds per pass, mean of `repeats`)."""
+    import torch
+    import bitsknn
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    matrix = torch.rand((max(query_counts), point_count), device=dev, generator=gen)
+    for q in query_counts:
+        rows = matrix[:q]
+        for k in k_values:
+            out_d = torch.empty((q, k), dtype=torch.float32, device=dev)
+            out_l = torch.empty((q, k), dtype=torch.int32, device=dev)
+            for name, prefetch in algorithms:
+                for block in block_sizes:
+                    for batch in batch_sizes:
+                        bitsknn.topk_bits(rows, k, block, batch, prefetch, out_dist=out_d, out_label=out_l)
+                        start = torch.cuda.Event(enable_timing=True)
+                        end = torch.cuda.Event(enable_timing=True)
+                        start.record()
+                        for _ in range(repeats):
+                            bitsknn.topk_bits(rows, k, block, batch, prefetch, out_dist=out_d,
+                                              out_label=out_l)
+                        end.record()
+                        end.synchronize()
+                        yield {"algorithm": name, "point_count": point_count, "query_count": q,
+                               "k": k, "dim": 1, "block_size": block, "items_per_thread": batch,
+                               "items_per_thread2": 1, "items_per_thread3": 1, "deg": 1,
+                               "time": start.elapsed_time(end) / 1e3 / repeats}
+            if progress is not None:
+                progress(q, k)
+
+
+def optima(rows):
+    """Fastest row of every (algorithm, point_count, query_count, k, dim)."""
+    best = {}
+    for row in rows:
+        key = (row["algorithm"], row["point_count"], row["query_count"], row["k"], row["dim"])
+        if key not in best or row["time"] < best[key]["time"]:
+            best[key] = row
+    return [best[key] for key in sorted(best)]
+
+
+def write_optima(rows, path, hostname="mi355x", gpu="MI355X"):
+    with open(path, "w", newline="") as handle:
+        writer = csv.writer(handle, lineterminator="\n")
+        writer.writerow(OPTIMA_COLUMNS)
+        for row in rows:
+            full = dict(row, hostname=hostname, GPU=gpu)
+            full["time"] = f"{row['time']:.10g}"
+            writer.writerow([full[name] for name in OPTIMA_COLUMNS])
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    ap.add_argument("--out", default=DEFAULT_OPTIMA, help="optima CSV to write")
+    ap.add_argument("--all", default=None, help="also write every measurement to this CSV")
+    ap.add_argument("--repeats", type=int, default=10)
+    ap.add_argument("--hostname", default="mi355x")
+    args = ap.parse_args(argv)
+
+    def progress(q, k):
+        print(f"q={q} k={k} done", file=sys.stderr, flush=True)
+
+    rows = list(sweep(repeats=args.repeats, progress=progress))
+    if args.all:
+        write_optima(rows, args.all, args.hostname)
+    write_optima(optima(rows), args.out, args.hostname)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -424,14 +424,38 @@ __global__ void __launch_bounds__(256)
                 }
             }
             const float* brow = stage + half * PT + nt * 32 + col;
+            // operands are requested from LDS one chunk of steps ahead of the multiplies that use them
+            constexpr int CH = STEPS <= 17 ? STEPS : 8;
+            float bv[2][CH];
 #pragma unroll
-            for (int s = 0; s < STEPS; ++s)
+            for (int s = 0; s < CH; ++s)
             {
-                const float bv = brow[2 * s * PT];
+                bv[0][s] = brow[2 * s * PT];
+            }
 #pragma unroll
-                for (int a = 0; a < QPW; ++a)
+            for (int c = 0; c < STEPS; c += CH)
+            {
+#pragma unroll
+                for (int s = 0; s < CH; ++s)
                 {
-                    acc[a] = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[a][s], bv, acc[a], 0, 0, 0);
+                    if (c + CH + s < STEPS)
+                    {
+                        bv[(c / CH + 1) & 1][s] = brow[2 * (c + CH + s) * PT];
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int s = 0; s < CH; ++s)
+                {
+                    if (c + s < STEPS)
+                    {
+#pragma unroll
+                        for (int a = 0; a < QPW; ++a)
+                        {
+                            acc[a] = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[a][c + s], bv[(c / CH) & 1][s],
+                                                                          acc[a], 0, 0, 0);
+                        }
+                    }
                 }
             }
             const size_t j = base + nt * 32 + col;

@@ -1,6 +1,7 @@
 """CPU-side checks of the C-ABI library: it loads, exports every declared symbol, and rejects
 unsupported parameters with the reference's messages before touching the GPU."""
 import ctypes
+import json
 import os
 import re
 
@@ -59,3 +60,51 @@ def test_topk_accepts_reference_parameter_lists_with_zero_rows(bk):
             for k in (1, 16, 17, 32, 64, 128, 256, 512, 1024, 2048):
                 st, text = _topk_status(bk, k, block, batch)
                 assert st == bk.OK, (block, batch, k, text)
+
+
+def _load_tuning():
+    import importlib.util
+    path = os.path.join(ROOT, "bits-knn-jpdc2024_amd", "bitsknn", "tuning.py")
+    spec = importlib.util.spec_from_file_location("bitsknn_tuning", path)
+    module = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(module)
+    return module
+
+
+def test_config_lookup_matches_reference_script():
+    """config_algorithm() against what the reference's awk lookup (scripts/config.sh:97-200)
+    printed for the same requests on tests/golden/optima_sample.csv (vectors written by
+    tests/golden/make_config_vectors.py)."""
+    tuning = _load_tuning()
+    golden = os.path.join(ROOT, "tests", "golden")
+    with open(os.path.join(golden, "config_vectors.json")) as handle:
+        vectors = json.load(handle)
+    assert len(vectors) >= 40
+    for vec in vectors:
+        def arg(x):
+            return None if x == "None" else x
+        got = tuning.config_algorithm(vec["algorithm"], arg(vec["query_count"]), arg(vec["k"]),
+                                      arg(vec["dim"]), arg(vec["hostname"]),
+                                      optima_file=os.path.join(golden, "optima_sample.csv"))
+        want = tuple(None if w == "" else int(w) for w in vec["answer"])
+        assert got == want, (vec, got)
+
+
+def test_shipped_optima_file():
+    """The MI355X optima file has the reference's columns (scripts/optima.csv, line 1) and a row
+    for every (algorithm, q, k) of the reference's search grid (scripts/run-opt-ipt.sh:38-47)."""
+    import csv
+    tuning = _load_tuning()
+    with open(tuning.DEFAULT_OPTIMA, newline="") as handle:
+        rows = list(csv.DictReader(handle))
+    assert tuple(rows[0].keys()) == tuning.OPTIMA_COLUMNS
+    seen = {(r["algorithm"], int(r["query_count"]), int(r["k"])) for r in rows}
+    for name, _ in tuning.ALGORITHMS:
+        for q in tuning.QUERY_COUNTS:
+            for k in tuning.K_VALUES:
+                assert (name, q, k) in seen
+    for r in rows:
+        assert int(r["block_size"]) in (128, 256, 512) and 1 <= int(r["items_per_thread"]) <= 16
+        assert float(r["time"]) > 0
+    block, deg, batch, _, _ = tuning.config_algorithm("bits", 1024, 32)
+    assert block in (128, 256, 512) and deg == 1 and 1 <= batch <= 16
