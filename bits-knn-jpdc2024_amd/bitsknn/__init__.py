@@ -20,6 +20,7 @@ EXPORTS = (
     "bitsknn_last_error",
     "bitsknn_version",
     "bitsknn_topk_bits_f32",
+    "bitsknn_topk_partial_bitonic_f32",
     "bitsknn_label_offsets",
     "bitsknn_fill_f32",
     "bitsknn_dist_f32",
@@ -59,6 +60,8 @@ def lib():
         L.bitsknn_topk_bits_f32.restype = ctypes.c_int
         L.bitsknn_topk_bits_f32.argtypes = [vp, sz, vp, sz, vp, sz, sz, vp, vp, sz, u32, u32, u32,
                                             ctypes.c_int, vp]
+        L.bitsknn_topk_partial_bitonic_f32.restype = ctypes.c_int
+        L.bitsknn_topk_partial_bitonic_f32.argtypes = [vp, sz, sz, sz, vp, vp, sz, u32, u32, vp]
         L.bitsknn_label_offsets.restype = ctypes.c_int
         L.bitsknn_label_offsets.argtypes = [vp, sz, sz, sz, vp]
         L.bitsknn_fill_f32.restype = ctypes.c_int
@@ -125,6 +128,22 @@ def topk_bits(dist, k, block_size=256, items_per_thread=16, prefetch=False, in_l
                                        _ptr(in_label), label_stride, _ptr(label_offsets), rows, cols,
                                        _ptr(out_dist), _ptr(out_label), _row_stride(out_dist), k,
                                        block_size, items_per_thread, 1 if prefetch else 0, _stream()))
+    return out_dist, out_label
+
+
+def topk_partial_bitonic(dist, k, block_size=256, out_dist=None, out_label=None):
+    """partial-bitonic-regs top-k (no filtering) of every row of a 2-D float32 device tensor."""
+    import torch
+    assert dist.is_cuda and dist.dtype == torch.float32 and dist.dim() == 2
+    assert dist.shape[1] == 1 or dist.stride(1) == 1
+    rows, cols = dist.shape
+    if out_dist is None:
+        out_dist = torch.empty((rows, k), dtype=torch.float32, device=dist.device)
+    if out_label is None:
+        out_label = torch.empty((rows, k), dtype=torch.int32, device=dist.device)
+    _check(lib().bitsknn_topk_partial_bitonic_f32(_ptr(dist), _row_stride(dist), rows, cols,
+                                                  _ptr(out_dist), _ptr(out_label),
+                                                  _row_stride(out_dist), k, block_size, _stream()))
     return out_dist, out_label
 
 

@@ -4,8 +4,10 @@ Two halves, matching the reference's tuning workflow:
 
 * ``sweep()`` times `bits` and `bits-prefetch` over the grid of the reference's parameter search
   (reference scripts/run-opt-ipt.sh:38-47: n = 512k, q in 64..8192, k in 2..2048, batch 1..16,
-  block size 128/256/512) and ``write_optima()`` keeps the fastest configuration of every
-  (algorithm, q, k) in a CSV with the columns of the reference's scripts/optima.csv
+  block size 128/256/512), ``sweep_partial_bitonic()`` times `partial-bitonic-regs` over the grid
+  of scripts/run-opt-bitonic-sort.sh:27-43 (q*n = 2^30, q in 64..4096, k in 32..2048, block size
+  64..512), and ``write_optima()`` keeps the fastest configuration of every (algorithm, q, k)
+  in a CSV with the columns of the reference's scripts/optima.csv
   (hostname, GPU, algorithm, point_count, query_count, k, dim, block_size, items_per_thread,
   items_per_thread2, items_per_thread3, deg, time), as scripts/plot-analyze-opt.py does.
 * ``config_algorithm()`` is the lookup the reference's run scripts perform on that file
@@ -126,6 +128,39 @@ def sweep(repeats=10, point_count=512 * 1024, query_counts=QUERY_COUNTS, k_value
                 progress(q, k)
 
 
+def sweep_partial_bitonic(repeats=5, problem_size=1 << 30, query_counts=(64, 256, 1024, 4096),
+                          k_values=(32, 64, 128, 256, 512, 1024, 2048), block_sizes=(64, 128, 256, 512),
+                          seed=17, progress=None):
+    """Time partial-bitonic-regs on cuda:0 over q x (problem_size / q) matrices."""
+    import torch
+    import bitsknn
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    flat = torch.rand(problem_size, device=dev, generator=gen)
+    for q in query_counts:
+        rows = flat.view(q, problem_size // q)
+        for k in k_values:
+            out_d = torch.empty((q, k), dtype=torch.float32, device=dev)
+            out_l = torch.empty((q, k), dtype=torch.int32, device=dev)
+            for block in block_sizes:
+                bitsknn.topk_partial_bitonic(rows, k, block, out_dist=out_d, out_label=out_l)
+                start = torch.cuda.Event(enable_timing=True)
+                end = torch.cuda.Event(enable_timing=True)
+                start.record()
+                for _ in range(repeats):
+                    bitsknn.topk_partial_bitonic(rows, k, block, out_dist=out_d, out_label=out_l)
+                end.record()
+                end.synchronize()
+                yield {"algorithm": "partial-bitonic-regs", "point_count": problem_size // q,
+                       "query_count": q, "k": k, "dim": 1, "block_size": block, "items_per_thread": 1,
+                       "items_per_thread2": 1, "items_per_thread3": 1, "deg": 1,
+                       "time": start.elapsed_time(end) / 1e3 / repeats}
+            if progress is not None:
+                progress(q, k)
+
+
 def optima(rows):
     """Fastest row of every (algorithm, point_count, query_count, k, dim)."""
     best = {}
@@ -152,12 +187,18 @@ def main(argv=None):
     ap.add_argument("--all", default=None, help="also write every measurement to this CSV")
     ap.add_argument("--repeats", type=int, default=10)
     ap.add_argument("--hostname", default="mi355x")
+    ap.add_argument("--only", choices=("bits", "partial-bitonic-regs"), default=None,
+                    help="time one family only (bits covers bits and bits-prefetch)")
     args = ap.parse_args(argv)
 
     def progress(q, k):
         print(f"q={q} k={k} done", file=sys.stderr, flush=True)
 
-    rows = list(sweep(repeats=args.repeats, progress=progress))
+    rows = []
+    if args.only in (None, "bits"):
+        rows += list(sweep(repeats=args.repeats, progress=progress))
+    if args.only in (None, "partial-bitonic-regs"):
+        rows += list(sweep_partial_bitonic(repeats=max(1, args.repeats // 2), progress=progress))
     if args.all:
         write_optima(rows, args.all, args.hostname)
     write_optima(optima(rows), args.out, args.hostname)

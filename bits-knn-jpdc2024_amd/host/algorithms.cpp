@@ -320,6 +320,23 @@ private:
     bool prefetch_;
 };
 
+// `partial-bitonic-regs`: sort-and-merge in registers without a filter
+// (reference: src/topk/singlepass/partial_bitonic.cu:217-294, 341-358)
+class partial_bitonic_regs : public device_knn
+{
+public:
+    std::string id() const override { return "partial-bitonic-regs"; }
+
+    void selection() override
+    {
+        BITSKNN_CHECK(bitsknn_topk_partial_bitonic_f32(
+            in_dist_gpu(), point_count(), query_count(), point_count(), out_dist_.data(),
+            out_label_.data(), k(), static_cast<std::uint32_t>(k()),
+            static_cast<std::uint32_t>(args_.selection_block_size), nullptr));
+        sync_default_stream();
+    }
+};
+
 // `bits-sq`: every row is cut into --deg parts that are selected independently (labels shifted
 // by the part offset), then the deg*k partial results of a row are selected again with their
 // labels.
@@ -465,6 +482,7 @@ std::vector<std::unique_ptr<knn>> make_algorithms()
     algorithms.push_back(std::make_unique<bits_knn>(false));
     algorithms.push_back(std::make_unique<bits_knn>(true));
     algorithms.push_back(std::make_unique<single_query_bits>());
+    algorithms.push_back(std::make_unique<partial_bitonic_regs>());
     algorithms.push_back(std::make_unique<fused_cache_knn>());
     algorithms.push_back(std::make_unique<dist_runner>("cublas-dist", &make_expanded_distance));
     algorithms.push_back(std::make_unique<dist_runner>("magma-dist", &make_l2_distance));

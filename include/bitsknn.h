@@ -66,6 +66,22 @@ int bitsknn_topk_bits_f32(const float* in, size_t in_row_stride, const int32_t* 
                           void* stream);
 
 /*
+ * partial-bitonic-regs: top-k of every row by sorting the row block after block in registers and
+ * merging each sorted block into the running result, with no filtering of the input (the
+ * baseline that the bits kernel's buffer and filter are measured against).  Same matrix and
+ * output layout and the same ordering of equal values as bitsknn_topk_bits_f32; labels are
+ * column indices.
+ *
+ * Replaces partial_bitonic_regs_kernel<K, BLOCK_SIZE> and partial_bitonic_regs_run
+ * (src/topk/singlepass/partial_bitonic.cu:217-294, 341-358).
+ *  block_size  one of 64, 128, 256, 512 ("Unsupported block size: N" otherwise)
+ *  k           1..2048                   ("Unsupported k value: N" otherwise)
+ */
+int bitsknn_topk_partial_bitonic_f32(const float* in, size_t in_row_stride, size_t rows, size_t cols,
+                                     float* out_dist, int32_t* out_label, size_t out_row_stride,
+                                     uint32_t k, uint32_t block_size, void* stream);
+
+/*
  * Label offsets for a row-split single-query problem: offsets[i] = (i % parts) * cols_per_part
  * for i < rows*parts.  Replaces populate_label_offsets_kernel
  * (src/topk/singlepass/bits_knn.cu:67-76).

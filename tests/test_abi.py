@@ -62,6 +62,24 @@ def test_topk_accepts_reference_parameter_lists_with_zero_rows(bk):
                 assert st == bk.OK, (block, batch, k, text)
 
 
+# messages of the reference dispatch (src/topk/singlepass/partial_bitonic.cu:341-358)
+@pytest.mark.parametrize("k,block,msg", [
+    (32, 100, "Unsupported block size: 100"),
+    (32, 1024, "Unsupported block size: 1024"),
+    (0, 256, "Unsupported k value: 0"),
+    (4096, 64, "Unsupported k value: 4096"),
+])
+def test_partial_bitonic_rejects_unsupported_parameters(bk, k, block, msg):
+    L = bk.lib()
+    st = L.bitsknn_topk_partial_bitonic_f32(None, 0, 0, 0, None, None, 0, k, block, None)
+    assert st == bk.ERR_UNSUPPORTED
+    assert L.bitsknn_last_error().decode() == msg
+    for good_block in (64, 128, 256, 512):
+        for good_k in (1, 16, 100, 2048):
+            assert L.bitsknn_topk_partial_bitonic_f32(None, 0, 0, 0, None, None, 0, good_k, good_block,
+                                                      None) == bk.OK
+
+
 def _load_tuning():
     import importlib.util
     path = os.path.join(ROOT, "bits-knn-jpdc2024_amd", "bitsknn", "tuning.py")
@@ -103,8 +121,9 @@ def test_shipped_optima_file():
         for q in tuning.QUERY_COUNTS:
             for k in tuning.K_VALUES:
                 assert (name, q, k) in seen
+    assert sum(r["algorithm"] == "partial-bitonic-regs" for r in rows) == 28
     for r in rows:
-        assert int(r["block_size"]) in (128, 256, 512) and 1 <= int(r["items_per_thread"]) <= 16
+        assert int(r["block_size"]) in (64, 128, 256, 512) and 1 <= int(r["items_per_thread"]) <= 16
         assert float(r["time"]) > 0
     block, deg, batch, _, _ = tuning.config_algorithm("bits", 1024, 32)
     assert block in (128, 256, 512) and deg == 1 and 1 <= batch <= 16

@@ -111,6 +111,23 @@ def test_golden_buffer_checksums_end_to_end(golden, pre):
 
 
 @pytest.mark.gpu
+def test_golden_buffer_checksums_partial_bitonic_regs(golden):
+    """The reference's runs of partial-bitonic-regs (data/buffer-*.err) on the same seeded input."""
+    done = 0
+    for rec in golden:
+        if rec["family"] != "buffer" or "partial-bitonic-regs" not in rec["algorithms"]:
+            continue
+        if (rec["n"], rec["q"]) != (1 << 18, 4096) or rec["preprocessor"] != "descending" or rec["k"] not in (32, 512):
+            continue
+        p = run("-a", "partial-bitonic-regs", "-n", "256k", "-q", "4k", "-k", str(rec["k"]), "--seed", "24",
+                "-p", "descending", "--block-size", "256")
+        assert p.returncode == 0, p.stderr
+        assert str(checksums(p)[0]) in rec["checksums"], (rec["k"], checksums(p))
+        done += 1
+    assert done == 2
+
+
+@pytest.mark.gpu
 def test_golden_fused_checksums_end_to_end(golden):
     done = 0
     for rec in golden:
