@@ -84,6 +84,15 @@ __host__ __device__ __forceinline__ std::int32_t key_label(u64 key)
 // (+inf, INT32_MAX): sorts after every finite value and after real +inf entries
 constexpr u64 PAD_KEY = 0xFF800000FFFFFFFFULL;
 
+// Workgroup barrier that orders LDS traffic only, so that global loads issued earlier stay in
+// flight across it.
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 } // namespace bitsknn
 
 #endif // BITSKNN_CSRC_COMMON_HPP_

@@ -14,6 +14,8 @@
 // Inputs are dim-major (component t of vector v at base[t*stride + v]), the output is the
 // row-major q x n matrix; all index arithmetic on the output is 64-bit (q*n reaches 2^32).
 
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace bitsknn
@@ -316,10 +318,13 @@ struct resident_geometry
     static constexpr int RANGE = 4096;                    // points per workgroup
 };
 
+// Covers queries q_first.. and points n_first.. of the matrix (the pipelined kernel below takes
+// the interior, this one the ragged edges, or everything when the pipelined one does not apply).
 template <int DP>
 __global__ void __launch_bounds__(256)
     dist_resident_kernel(int dim, size_t q, size_t n, const float* __restrict__ queries, size_t qs,
-                         const float* __restrict__ points, size_t ps, float* __restrict__ dist, size_t ds)
+                         const float* __restrict__ points, size_t ps, float* __restrict__ dist, size_t ds,
+                         size_t q_first, size_t n_first)
 {
     using G = resident_geometry<DP>;
     constexpr int PT = G::PT;
@@ -336,8 +341,9 @@ __global__ void __launch_bounds__(256)
     const int wave = __builtin_amdgcn_readfirstlane(t / WAVE);
     const int half = lane / 32;
     const int col = lane & 31;
-    const size_t wave_q0 = static_cast<size_t>(blockIdx.x) * G::QB + static_cast<size_t>(wave) * 32 * QPW;
-    const size_t j_begin = static_cast<size_t>(blockIdx.y) * G::RANGE;
+    const size_t wave_q0 =
+        q_first + static_cast<size_t>(blockIdx.x) * G::QB + static_cast<size_t>(wave) * 32 * QPW;
+    const size_t j_begin = n_first + static_cast<size_t>(blockIdx.y) * G::RANGE;
     const size_t j_end = j_begin + G::RANGE < n ? j_begin + G::RANGE : n;
 
     // query fragments: step s of this lane is row 2s + half; the norm rows are multiplied by 1
@@ -507,20 +513,358 @@ __global__ void __launch_bounds__(256)
     }
 }
 
+// f(integral_constant<int, BEGIN>) ... f(integral_constant<int, END - 1>), expanded by the front
+// end so that register arrays are indexed by constants whatever the size of the body
+template <int BEGIN, int END, typename F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (BEGIN < END)
+    {
+        f(std::integral_constant<int, BEGIN>{});
+        static_for<BEGIN + 1, END>(f);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Pipelined form of the query-resident kernel for the interior of the matrix: whole blocks of
+// 128 queries, whole stages of PT points, dimensions up to 128.
+//
+// On gfx950 a wave that issues matrix instructions back to back leaves no issue slots to the
+// other waves of its SIMD, and vector-ALU instructions of the same wave are not overlapped with
+// its matrix instructions; LDS and memory instructions are.  So the loop over stages keeps the
+// vector ALU out of the way: one wave per SIMD, and between two multiplies only LDS reads and
+// writes, buffer loads and buffer stores whose addresses are a constant lane offset plus a
+// scalar offset.
+//  * The -2 of -2 q.p is folded into the query fragment (the B operand, in registers); a stage in
+//    LDS holds the raw point values and the staging threads' shares of ||p||^2 (A operand).
+//  * With the points as A operand a lane holds, in four consecutive result registers, four
+//    consecutive points of ONE query.  A finished stage (32 queries x PT points per wave) is
+//    written to a per-wave LDS tile with 16-byte writes, read back row by row during the next
+//    stage, and stored with 16-byte buffer stores: 512 contiguous bytes per row and half-wave.
+//  * Point values of the next stage are requested with buffer loads during the first third of a
+//    stage and written to LDS during the last third; the only vector instructions per stage are
+//    the VPT multiply-adds of the norm shares, issued in one burst.
+// Results are bit-identical to the plain kernel: same products (scaling by -2 is exact) added in
+// the same order.
+// ---------------------------------------------------------------------------------------------
+template <int DP>
+struct pipelined_geometry
+{
+    static constexpr int PT = DP <= 64 ? 128 : 64;       // points per stage
+    static constexpr int TPP = 256 / PT;                  // staging threads per point
+    static constexpr int ROWS = DP + TPP;                 // dimensions + norm shares
+    static constexpr int STEPS = ROWS / 2;
+    static constexpr int VPT = DP / TPP;                  // staged values per thread
+    static constexpr int NT = PT / 32;                    // 32-point tiles per stage
+    static constexpr int QB = 128;                        // queries per workgroup (32 per wave)
+    static constexpr int TP = PT + 4;                     // row pitch of the result tile in LDS
+    static constexpr int STAGE_FLOATS = ROWS * PT;
+    static constexpr int LDS_FLOATS = 2 * STAGE_FLOATS + 4 * 32 * TP;
+};
+
+typedef unsigned int vuint4 __attribute__((ext_vector_type(4)));
+
+template <int DP>
+__global__ void __launch_bounds__(256)
+    dist_pipelined_kernel(int dim, size_t q_full, size_t n_full, const float* __restrict__ queries, size_t qs,
+                          const float* __restrict__ points, size_t ps, float* __restrict__ dist, size_t ds,
+                          unsigned range)
+{
+    using G = pipelined_geometry<DP>;
+    constexpr int PT = G::PT;
+    constexpr int TPP = G::TPP;
+    constexpr int STEPS = G::STEPS;
+    constexpr int VPT = G::VPT;
+    constexpr int NT = G::NT;
+    constexpr int TP = G::TP;
+    constexpr int SLOTS = STEPS * NT;   // one slot per multiply
+    static_assert(SLOTS >= 16 && VPT <= SLOTS / 3);
+
+    __shared__ float lds[G::LDS_FLOATS];
+    float* const stages = lds;
+
+    const int t = static_cast<int>(threadIdx.x);
+    const int lane = t & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(t / WAVE);
+    const int half = lane / 32;
+    const int col = lane & 31;
+    const size_t wave_q0 = static_cast<size_t>(blockIdx.x) * G::QB + static_cast<size_t>(wave) * 32;
+    // `range` points (a multiple of PT) per workgroup
+    const size_t j_begin = static_cast<size_t>(blockIdx.y) * range;
+    const size_t j_end = j_begin + range < n_full ? j_begin + range : n_full;
+    const int stage_count = static_cast<int>((j_end - j_begin) / PT);
+    float* const tile = lds + 2 * G::STAGE_FLOATS + wave * 32 * TP;
+
+    // B operand: step s of this lane is dimension 2s + half of query `col`, times -2; the norm
+    // rows are multiplied by 1
+    float qf[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s)
+    {
+        const int dd = 2 * s + half;
+        float val = dd >= DP ? 1.0F : 0.0F;
+        if (dd < dim)
+        {
+            val = -2.0F * queries[static_cast<size_t>(dd) * qs + wave_q0 + col];
+        }
+        qf[s] = val;
+    }
+
+    // Buffer resources: base + constant lane offset + scalar offset.
+    const auto point_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(points + j_begin), 0,
+        static_cast<int>((static_cast<size_t>(dim) * ps - j_begin) * sizeof(float)), 0x00020000);
+    const auto dist_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        dist + wave_q0 * ds + j_begin, 0, static_cast<int>((31 * ds + (j_end - j_begin)) * sizeof(float)),
+        0x00020000);
+    const int sp = t % PT;
+    const int sd0 = t / PT;
+    // a row of a finished stage is PT/4 16-byte pieces: one store instruction covers RPI rows
+    constexpr int QPR = PT / 4;
+    constexpr int RPI = WAVE / QPR;
+    constexpr int NE = 32 / RPI;   // store instructions per stage
+    const int store_lane_off =
+        static_cast<int>((static_cast<size_t>(lane / QPR) * ds + 4 * (lane % QPR)) * sizeof(float));
+
+    // Byte offset of value i of this thread (dimension sd0 + TPP*i of point sp) inside the point
+    // resource; the stage is selected by the scalar offset.  The hardware checks only the lane
+    // offset against the size of the resource, so dimensions dim .. DP-1 get an offset beyond it
+    // and read as zero.
+    int load_off[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i)
+    {
+        const int dd = sd0 + TPP * i;
+        load_off[i] = dd < dim ? static_cast<int>((static_cast<size_t>(dd) * ps + sp) * sizeof(float)) : 0x7FFFFFF0;
+    }
+    float pre[VPT];
+    auto request = [&](auto i_tag, int first) {
+        constexpr int i = decltype(i_tag)::value;
+        pre[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                               point_rsrc, load_off[i], first * static_cast<int>(sizeof(float)), 0));
+    };
+    auto write_value = [&](auto i_tag, float* stage) {
+        constexpr int i = decltype(i_tag)::value;
+        stage[(sd0 + TPP * i) * PT + sp] = pre[i];
+    };
+    auto write_share = [&](float* stage) {
+        float share = 0.0F;
+#pragma unroll
+        for (int i = 0; i < VPT; ++i)
+        {
+            share = __builtin_fmaf(pre[i], pre[i], share);
+        }
+        stage[(DP + sd0) * PT + sp] = share;
+    };
+    // row group e (rows RPI*e .. RPI*e + RPI-1 of the wave's 32 queries) of the finished stage at `first`
+    auto read_rows = [&](auto e_tag) -> vfloat4 {
+        constexpr int e = decltype(e_tag)::value;
+        return *reinterpret_cast<const vfloat4*>(tile + (RPI * e + lane / QPR) * TP + 4 * (lane % QPR));
+    };
+    auto store_rows = [&](auto e_tag, vfloat4 rows, int first) {
+        constexpr int e = decltype(e_tag)::value;
+        const int scalar_off =
+            static_cast<int>((static_cast<size_t>(RPI * e) * ds + static_cast<size_t>(first)) * sizeof(float));
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(vuint4, rows), dist_rsrc, store_lane_off,
+                                               scalar_off, 2 /* non-temporal */);
+    };
+
+    vfloat16 acc[NT];
+    // lane (query col, half) holds in acc[k][4g .. 4g+3] the points 32k + 8g + 4*half + 0..3
+    auto park_results = [&]() {
+        static_for<0, NT>([&](auto k_tag) {
+            constexpr int k = decltype(k_tag)::value;
+            static_for<0, 4>([&](auto g_tag) {
+                constexpr int g = decltype(g_tag)::value;
+                vfloat4 v;
+                v[0] = acc[k][4 * g + 0];
+                v[1] = acc[k][4 * g + 1];
+                v[2] = acc[k][4 * g + 2];
+                v[3] = acc[k][4 * g + 3];
+                *reinterpret_cast<vfloat4*>(tile + col * TP + 32 * k + 8 * g + 4 * half) = v;
+            });
+        });
+    };
+
+    // One stage.  HAVE_PREV: the LDS tile holds the results of the stage before (at first - PT),
+    // to be stored.  HAVE_NEXT: the stage after this one exists; its values are requested during
+    // the first third of the multiplies and written to `stage_next` during the last third (the
+    // middle third covers the latency of the loads).  Both are types: a branch between two
+    // multiplies would cost an instruction fetch that nothing hides.
+    auto run_stage = [&](auto prev_tag, auto next_tag, const float* stage, float* stage_next, int first) {
+        constexpr bool have_prev = decltype(prev_tag)::value;
+        constexpr bool have_next = decltype(next_tag)::value;
+        constexpr int THIRD = SLOTS / 3;
+        constexpr int STRIDE = SLOTS / NE;
+        const float* arow = stage + half * PT + col;
+        float av[2][NT];
+        static_for<0, NT>([&](auto k_tag) { av[0][decltype(k_tag)::value] = arow[32 * decltype(k_tag)::value]; });
+        vfloat4 rows;
+        static_for<0, STEPS>([&](auto s_tag) {
+            constexpr int s = decltype(s_tag)::value;
+            static_for<0, NT>([&](auto k_tag) {
+                constexpr int k = decltype(k_tag)::value;
+                constexpr int slot = s * NT + k;
+                if constexpr (s + 1 < STEPS)
+                {
+                    av[(s + 1) & 1][k] = arow[2 * (s + 1) * PT + 32 * k];
+                }
+                if constexpr (s == 0)
+                {
+                    vfloat16 zero;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                    {
+                        zero[r] = 0.0F;
+                    }
+                    acc[k] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[0][k], qf[0], zero, 0, 0, 0);
+                }
+                else
+                {
+                    acc[k] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[s & 1][k], qf[s], acc[k], 0, 0, 0);
+                }
+                if constexpr (have_prev && slot / STRIDE < NE)
+                {
+                    // row group slot / STRIDE of the previous stage: read here, stored half a stride on
+                    if constexpr (slot % STRIDE == 0)
+                    {
+                        rows = read_rows(std::integral_constant<int, slot / STRIDE>{});
+                    }
+                    if constexpr (slot % STRIDE == STRIDE / 2)
+                    {
+                        store_rows(std::integral_constant<int, slot / STRIDE>{}, rows, first - PT);
+                    }
+                }
+                if constexpr (have_next)
+                {
+                    if constexpr (slot < THIRD)
+                    {
+                        static_for<slot * VPT / THIRD, (slot + 1) * VPT / THIRD>(
+                            [&](auto i_tag) { request(i_tag, first + PT); });
+                    }
+                    else if constexpr (slot >= SLOTS - THIRD)
+                    {
+                        constexpr int w = slot - (SLOTS - THIRD);
+                        if constexpr (w == 0)
+                        {
+                            write_share(stage_next);
+                        }
+                        static_for<w * VPT / THIRD, (w + 1) * VPT / THIRD>(
+                            [&](auto i_tag) { write_value(i_tag, stage_next); });
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        });
+        park_results();
+    };
+
+    if (stage_count <= 0)
+    {
+        return;
+    }
+    // prologue: stage 0 into LDS
+    static_for<0, VPT>([&](auto i_tag) { request(i_tag, 0); });
+    write_share(stages);
+    static_for<0, VPT>([&](auto i_tag) { write_value(i_tag, stages); });
+    lds_barrier();
+
+    constexpr std::true_type yes{};
+    constexpr std::false_type no{};
+    for (int st = 0; st < stage_count; ++st)
+    {
+        const float* const stage = stages + (st & 1) * G::STAGE_FLOATS;
+        float* const stage_next = stages + ((st & 1) ^ 1) * G::STAGE_FLOATS;
+        const int first = st * PT;
+        const bool have_next = st + 1 < stage_count;
+        if (st == 0)
+        {
+            if (have_next)
+            {
+                run_stage(no, yes, stage, stage_next, first);
+            }
+            else
+            {
+                run_stage(no, no, stage, stage_next, first);
+            }
+        }
+        else if (have_next)
+        {
+            run_stage(yes, yes, stage, stage_next, first);
+        }
+        else
+        {
+            run_stage(yes, no, stage, stage_next, first);
+        }
+        lds_barrier();
+    }
+    // the results of the last stage are still in the LDS tile
+    static_for<0, NE>([&](auto e_tag) { store_rows(e_tag, read_rows(e_tag), (stage_count - 1) * PT); });
+}
+
 template <int DP>
 bool launch_resident(int dim, size_t q, size_t n, const float* queries, size_t qs, const float* points,
                      size_t ps, float* dist, size_t ds, hipStream_t stream)
 {
-    using G = resident_geometry<DP>;
-    const size_t gx = (q + G::QB - 1) / G::QB;
-    const size_t gy = (n + G::RANGE - 1) / G::RANGE;
-    if (gx > 0x7FFFFFFFULL || gy > 65535)
+    using P = resident_geometry<DP>;
+    size_t q_full = 0;
+    size_t n_full = 0;
+    if constexpr (DP <= 128)
     {
-        return false;
+        // the pipelined kernel takes whole query blocks x whole stages when rows are 16-byte
+        // aligned and every offset inside a workgroup's share fits the 32-bit buffer offsets
+        using F = pipelined_geometry<DP>;
+        const bool aligned = reinterpret_cast<std::uintptr_t>(dist) % 16 == 0 && ds % 4 == 0;
+        const bool in_range = 32 * ds * sizeof(float) < (1ULL << 31) &&
+                              static_cast<size_t>(dim) * ps * sizeof(float) < (1ULL << 31);
+        if (aligned && in_range)
+        {
+            q_full = q / F::QB * F::QB;
+            n_full = n / F::PT * F::PT;
+            if (q_full == 0 || n_full == 0)
+            {
+                q_full = 0;
+                n_full = 0;
+            }
+        }
+        if (q_full > 0)
+        {
+            // One workgroup fits a compute unit (LDS), so its prologue and epilogue are not
+            // overlapped with anything: give every workgroup as long a range of points as still
+            // leaves about 8 workgroups per compute unit, at least 4096 points.
+            const size_t gx = q_full / F::QB;
+            size_t range = n_full * gx / 2048;
+            range = range < 4096 ? 4096 : (range > (1U << 20) ? (1U << 20) : range);
+            range = (range + F::PT - 1) / F::PT * F::PT;
+            const size_t gy = (n_full + range - 1) / range;
+            if (gx > 0x7FFFFFFFULL || gy > 65535)
+            {
+                return false;
+            }
+            hipLaunchKernelGGL((dist_pipelined_kernel<DP>), dim3(static_cast<unsigned>(gx), static_cast<unsigned>(gy)),
+                               dim3(256), 0, stream, dim, q_full, n_full, queries, qs, points, ps, dist, ds,
+                               static_cast<unsigned>(range));
+        }
     }
-    hipLaunchKernelGGL(dist_resident_kernel<DP>, dim3(static_cast<unsigned>(gx), static_cast<unsigned>(gy)),
-                       dim3(256), 0, stream, dim, q, n, queries, qs, points, ps, dist, ds);
-    return true;
+    // the plain kernel covers what is left: points n_full.. of the first q_full queries, and all
+    // points of the queries q_full..
+    auto plain = [&](size_t q_first, size_t q_end, size_t n_first) -> bool {
+        if (q_first >= q_end || n_first >= n)
+        {
+            return true;
+        }
+        const size_t gx = (q_end - q_first + P::QB - 1) / P::QB;
+        const size_t gy = (n - n_first + P::RANGE - 1) / P::RANGE;
+        if (gx > 0x7FFFFFFFULL || gy > 65535)
+        {
+            return false;
+        }
+        hipLaunchKernelGGL(dist_resident_kernel<DP>, dim3(static_cast<unsigned>(gx), static_cast<unsigned>(gy)),
+                           dim3(256), 0, stream, dim, q_end, n, queries, qs, points, ps, dist, ds, q_first,
+                           n_first);
+        return true;
+    };
+    return plain(0, q_full, n_full) && plain(q_full, q, 0);
 }
 
 } // namespace

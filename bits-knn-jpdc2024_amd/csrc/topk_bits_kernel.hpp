@@ -45,15 +45,6 @@ struct topk_args
     u32 k;
 };
 
-// Workgroup barrier that orders LDS traffic only, so that global loads issued earlier stay in
-// flight across it.
-__device__ __forceinline__ void lds_barrier()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
 // Merge the filled part of every wave's buffer slice into the ascending top-k list.  Slice w
 // holds fill[w] keys from buffer[w*CAP].  The buffer memory doubles as exchange scratch once its
 // keys are in registers.
