@@ -11,7 +11,7 @@
 //    stages of PT points, two stages in LDS (one being multiplied, one being filled; one barrier
 //    per stage).  A stage is the MFMA A operand: rows 0..d-1 hold -2*p, the following rows hold
 //    the staging threads' shares of ||p||^2, so that v_mfma_f32_32x32x2_f32 against the query
-//    fragment (q_0..q_{d-1}, 1, 1) yields ||p||^2 - 2 q.p directly, the dot product accumulated
+//    fragment (-2q_0..-2q_{d-1}, 1, 1) yields ||p||^2 - 2 q.p directly, the dot product accumulated
 //    first and the norm added last.
 //  * The query fragment stays in registers for the whole kernel.  In the 32 x 32 result tile a
 //    lane holds 16 distances of ONE query (column), so the filter is a min-tree over 16
@@ -29,6 +29,8 @@
 // Equal distances are ordered by lower point index: points are visited in index order, so a
 // value equal to a query's radius can never displace what is already merged.
 
+#include <type_traits>
+
 #include "bitonic_net.hpp"
 #include "common.hpp"
 
@@ -36,6 +38,18 @@ namespace bitsknn
 {
 namespace
 {
+
+// f(integral_constant<int, BEGIN>) ... f(integral_constant<int, END - 1>), expanded by the front end
+template <int BEGIN, int END, typename F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (BEGIN < END)
+    {
+        f(std::integral_constant<int, BEGIN>{});
+        static_for<BEGIN + 1, END>(f);
+    }
+}
+
 
 typedef float vfloat16 __attribute__((ext_vector_type(16)));
 
@@ -65,7 +79,7 @@ struct fused_geometry
 {
     static constexpr int PT = DP <= 16 ? 256 : (DP <= 32 ? 128 : (DP <= 64 ? 64 : 32));
     static constexpr int TPP = FQ_THREADS / PT; // threads per point when staging
-    // -2p rows (zero beyond dim), then one row per staging thread of a point with its share of
+    // point rows (zero beyond dim), then one row per staging thread of a point with its share of
     // ||p||^2 (at least two rows, so that the row count is even)
     static constexpr int NORM_ROWS = TPP > 2 ? TPP : 2;
     static constexpr int ROWS = DP + NORM_ROWS;
@@ -120,7 +134,8 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     u64* const wbuf = buffers + static_cast<size_t>(wave) * FQ_QW * FQ_CAP;
     float* const wx = xchg + wave * WAVE;     // 32 radii, then 32 fills (as int bits)
 
-    // query fragment: step s of this lane is row 2s + half; the norm rows are multiplied by 1
+    // query fragment: step s of this lane is row 2s + half, times -2 (the stages hold the plain
+    // point values); the norm rows are multiplied by 1
     float qf[STEPS];
 #pragma unroll
     for (int s = 0; s < STEPS; ++s)
@@ -129,7 +144,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         float val = dd >= DP ? 1.0F : 0.0F;
         if (dd < dim && my_q < a.q)
         {
-            val = a.queries[static_cast<size_t>(dd) * a.q + my_q];
+            val = -2.0F * a.queries[static_cast<size_t>(dd) * a.q + my_q];
         }
         qf[s] = val;
     }
@@ -259,20 +274,54 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     };
 
     // ---- staging: global -> registers -> LDS ---------------------------------------------------
-    // thread t carries dimensions (t / PT) + TPP*i of point t % PT, turns them into -2p rows and
-    // adds up its share of ||p||^2 (the shares of a point meet inside the MFMA)
+    // thread t carries dimensions (t / PT) + TPP*i of point t % PT, writes them as rows of the
+    // stage and adds up its share of ||p||^2 (the shares of a point meet inside the MFMA)
     const int sp = t % PT;
     const int sd0 = t / PT;
     const bool whole_dim = dim == DP;
     float pre[VPT];
-    auto fetch = [&](int base) {
-        if (whole_dim && base + PT <= n)
-        {
-            const float* __restrict__ src = a.points + static_cast<size_t>(sd0) * total_points + base + sp;
+    // Point values are read with buffer loads: a constant byte offset per value and lane (beyond
+    // the resource for dimensions dim .. DP-1, which then read as zero; the hardware checks the
+    // lane offset only) plus the scalar offset of the stage, so that a load needs no vector
+    // arithmetic.  Point matrices of 2 GiB and more take the plain loads.
+    const bool small_points = static_cast<size_t>(dim) * total_points * sizeof(float) < (1ULL << 31);
+    const auto point_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(a.points), 0,
+        small_points ? static_cast<int>(static_cast<size_t>(dim) * total_points * sizeof(float)) : 0, 0x00020000);
+    constexpr int OUTSIDE = 0x7FFFFFF0;
+    int load_off[VPT];
 #pragma unroll
-            for (int i = 0; i < VPT; ++i)
+    for (int i = 0; i < VPT; ++i)
+    {
+        const int dd = sd0 + TPP * i;
+        load_off[i] = dd < dim && small_points
+                          ? static_cast<int>((static_cast<size_t>(dd) * total_points + sp) * sizeof(float))
+                          : OUTSIDE;
+    }
+    auto fetch = [&](int base) {
+        if (small_points)
+        {
+            const int stage_off = base * static_cast<int>(sizeof(float));
+            if (base + PT <= n)
             {
-                pre[i] = src[static_cast<size_t>(TPP * i) * total_points];
+#pragma unroll
+                for (int i = 0; i < VPT; ++i)
+                {
+                    pre[i] = __builtin_bit_cast(
+                        float, __builtin_amdgcn_raw_buffer_load_b32(point_rsrc, load_off[i], stage_off, 0));
+                }
+            }
+            else
+            {
+                // ragged last stage: points from n on read as zero
+                const bool inside = base + sp < n;
+#pragma unroll
+                for (int i = 0; i < VPT; ++i)
+                {
+                    pre[i] = __builtin_bit_cast(
+                        float, __builtin_amdgcn_raw_buffer_load_b32(point_rsrc, inside ? load_off[i] : OUTSIDE,
+                                                                    stage_off, 0));
+                }
             }
         }
         else
@@ -299,7 +348,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             share = __builtin_fmaf(pre[i], pre[i], share);
             if (whole_dim || dd < dim)
             {
-                stage[dd * PT + sp] = -2.0F * pre[i];
+                stage[dd * PT + sp] = pre[i];
             }
         }
         // points beyond the end get an infinite distance and never pass the filter
@@ -310,11 +359,23 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     auto multiply = [&](const float* stage, int base) {
         if constexpr (MT >= 2)
         {
-            // two row tiles at a time: two independent accumulator chains keep the matrix core
-            // issuing back to back
-#pragma unroll 1
-            for (int mt = 0; mt < MT; mt += 2)
+            // Two row tiles at a time: two independent accumulator chains keep the matrix core
+            // issuing back to back.  The A operands of a pair sit in registers before its first
+            // MFMA; those of the next pair are requested from LDS between the MFMAs of this one
+            // (LDS instructions are overlapped with matrix instructions, vector-ALU ones are not).
+            constexpr int PAIRS = MT / 2;
+            float a[2][2][STEPS];
+            const float* arow = stage + half * PT + ql;
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
             {
+                a[0][0][s] = arow[2 * s * PT];
+                a[0][1][s] = arow[2 * s * PT + 32];
+            }
+            __builtin_amdgcn_sched_barrier(0); // keep the reads above the chain
+            static_for<0, PAIRS>([&](auto p_tag) {
+                constexpr int p = decltype(p_tag)::value;
+                constexpr int cur = p & 1;
                 vfloat16 acc0;
                 vfloat16 acc1;
 #pragma unroll
@@ -323,27 +384,20 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                     acc0[r] = 0.0F;
                     acc1[r] = 0.0F;
                 }
-                // all A operands of the pair are requested from LDS before the first MFMA, so the
-                // chain never waits for a read
-                const float* arow = stage + half * PT + mt * 32 + ql;
-                float a0[STEPS];
-                float a1[STEPS];
-#pragma unroll
-                for (int s = 0; s < STEPS; ++s)
-                {
-                    a0[s] = arow[2 * s * PT];
-                    a1[s] = arow[2 * s * PT + 32];
-                }
-                __builtin_amdgcn_sched_barrier(0); // keep the reads above the chain
-#pragma unroll
-                for (int s = 0; s < STEPS; ++s)
-                {
-                    acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[s], qf[s], acc0, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[s], qf[s], acc1, 0, 0, 0);
-                }
-                filter_tile(acc0, base + mt * 32);
-                filter_tile(acc1, base + mt * 32 + 32);
-            }
+                static_for<0, STEPS>([&](auto s_tag) {
+                    constexpr int s = decltype(s_tag)::value;
+                    if constexpr (p + 1 < PAIRS)
+                    {
+                        a[cur ^ 1][0][s] = arow[2 * s * PT + 64 * (p + 1)];
+                        a[cur ^ 1][1][s] = arow[2 * s * PT + 64 * (p + 1) + 32];
+                    }
+                    acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][0][s], qf[s], acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][1][s], qf[s], acc1, 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+                filter_tile(acc0, base + p * 64);
+                filter_tile(acc1, base + p * 64 + 32);
+            });
         }
         else
         {
