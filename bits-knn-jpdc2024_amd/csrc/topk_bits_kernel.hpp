@@ -146,7 +146,15 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     const u32 full_end =
         n > static_cast<u32>(NL) ? static_cast<u32>(NL) + ((n - static_cast<u32>(NL)) / CHUNK) * CHUNK
                                  : static_cast<u32>(NL);
-    u32 chunk = NL;
+    // The chunks after the first NL values are visited from both ends of the row inwards
+    // (first, last, second, last but one, ...): whichever end of a sorted row holds the small
+    // values, the radius is tight after two chunks, where a front-to-back pass over a descending
+    // row would let every value through the filter.  The result does not depend on the order.
+    const u32 chunk_count = n > static_cast<u32>(NL) ? (n - static_cast<u32>(NL) + CHUNK - 1) / CHUNK : 0;
+    u32 left = chunk_count;            // chunks not yet visited
+    u32 chunk = NL;                    // the next chunk to visit
+    // distance to the chunk after it: alternating in sign and shrinking by one chunk per visit
+    std::int32_t jump = chunk_count > 0 ? static_cast<std::int32_t>((chunk_count - 1) * CHUNK) : 0;
 
     // the first NL values go straight to the buffer: column c into slot c
 #pragma unroll
@@ -235,7 +243,7 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     {
         // ---- rendezvous: every wave arrives here when it needs a merge, saw the flag, or ran
         // out of values
-        const bool more_work = pending || chunk < n;
+        const bool more_work = pending || left > 0;
         if (lane == 0)
         {
             s_fill[wave] = fill;
@@ -291,7 +299,7 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
         }
 
         // ---- streaming: no synchronisation with the other waves except polling the flag
-        while (chunk < n)
+        while (left > 0)
         {
             if (chunk < full_end)
             {
@@ -330,7 +338,9 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
             }
             const int flag = *static_cast<volatile int*>(&s_flag);
             cur_chunk = chunk;
-            chunk += CHUNK;
+            left -= 1;
+            chunk += static_cast<u32>(jump);
+            jump = (jump > 0 ? static_cast<std::int32_t>(CHUNK) : -static_cast<std::int32_t>(CHUNK)) - jump;
 
             float smallest = v[0];
 #pragma unroll
