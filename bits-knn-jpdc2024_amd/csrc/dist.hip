@@ -320,7 +320,8 @@ struct resident_geometry
 
 // Covers queries q_first.. and points n_first.. of the matrix (the pipelined kernel below takes
 // the interior, this one the ragged edges, or everything when the pipelined one does not apply).
-template <int DP>
+// STREAMING: rows start on 128-byte boundaries (see the stores).
+template <int DP, bool STREAMING>
 __global__ void __launch_bounds__(256)
     dist_resident_kernel(int dim, size_t q, size_t n, const float* __restrict__ queries, size_t qs,
                          const float* __restrict__ points, size_t ps, float* __restrict__ dist, size_t ds,
@@ -476,7 +477,17 @@ __global__ void __launch_bounds__(256)
                         const size_t i = wave_q0 + a * 32 + 8 * (r / 4) + 4 * half + (r % 4);
                         if (i < q)
                         {
-                            __builtin_nontemporal_store(acc[a][r], dist + i * ds + j);
+                            // Rows that are not 128-byte aligned share cache lines between
+                            // neighbouring tiles: ordinary stores let L2 merge the pieces, where
+                            // streaming stores would write partial lines to memory.
+                            if constexpr (STREAMING)
+                            {
+                                __builtin_nontemporal_store(acc[a][r], dist + i * ds + j);
+                            }
+                            else
+                            {
+                                dist[i * ds + j] = acc[a][r];
+                            }
                         }
                     }
                 }
@@ -859,9 +870,17 @@ bool launch_resident(int dim, size_t q, size_t n, const float* queries, size_t q
         {
             return false;
         }
-        hipLaunchKernelGGL(dist_resident_kernel<DP>, dim3(static_cast<unsigned>(gx), static_cast<unsigned>(gy)),
-                           dim3(256), 0, stream, dim, q_end, n, queries, qs, points, ps, dist, ds, q_first,
-                           n_first);
+        const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(gy));
+        if (reinterpret_cast<std::uintptr_t>(dist) % 128 == 0 && ds % 32 == 0)
+        {
+            hipLaunchKernelGGL((dist_resident_kernel<DP, true>), grid, dim3(256), 0, stream, dim, q_end, n, queries,
+                               qs, points, ps, dist, ds, q_first, n_first);
+        }
+        else
+        {
+            hipLaunchKernelGGL((dist_resident_kernel<DP, false>), grid, dim3(256), 0, stream, dim, q_end, n, queries,
+                               qs, points, ps, dist, ds, q_first, n_first);
+        }
         return true;
     };
     return plain(0, q_full, n_full) && plain(q_full, q, 0);
