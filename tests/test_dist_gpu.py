@@ -129,3 +129,30 @@ def test_dist_errors(bk, dev):
     a = torch.zeros((4, 10), device=dev)
     with pytest.raises(bk.BitsKnnError, match="Unsupported distance"):
         bk.distances(a, a, 7)
+
+
+@pytest.mark.parametrize("d", [8, 16, 32, 48, 64, 100, 128])
+def test_pipelined_and_plain_kernels_give_the_same_bits(bk, dev, d):
+    """Whole 128-query blocks x whole stages take the pipelined kernel, everything else (here: the
+    same problem written into a matrix whose rows are not 16-byte aligned) the plain one.  Both
+    add the same products in the same order."""
+    import torch
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(d)
+    q, n = 384, 4096 * 2 + 640 + 37          # interior + a ragged last stage + ragged columns
+    queries = torch.rand((d, q), device=dev, generator=gen) - 0.5
+    points = torch.rand((d, n), device=dev, generator=gen) - 0.5
+    out_a = torch.full((q, n + 3), -7.0, device=dev)
+    assert (n + 3) % 4 == 0
+    bk.distances(queries, points, bk.DIST_PARTIAL_L2, out=out_a[:, :n])       # row stride n+3: aligned
+    out_b = torch.full((q, n + 2), -7.0, device=dev)
+    bk.distances(queries, points, bk.DIST_PARTIAL_L2, out=out_b[:, :n])       # row stride n+2: unaligned
+    torch.cuda.synchronize()
+    assert torch.equal(out_a[:, :n].view(torch.int32), out_b[:, :n].view(torch.int32))
+    assert (out_a[:, n:] == -7.0).all() and (out_b[:, n:] == -7.0).all()
+    # ragged query count: the last 5 queries go through the plain kernel
+    out_c = torch.full((q + 5, n + 3), -7.0, device=dev)
+    more = torch.cat([queries, queries[:, :5]], dim=1).contiguous()
+    bk.distances(more, points, bk.DIST_PARTIAL_L2, out=out_c[:, :n])
+    torch.cuda.synchronize()
+    assert torch.equal(out_c[:q, :n], out_a[:, :n]) and torch.equal(out_c[q:, :n], out_a[:5, :n])
