@@ -17,15 +17,32 @@
 namespace bitsknn
 {
 
-// Value of `x` held by lane (lane ^ MASK), MASK a power of two below 64.  Distances 1, 2, 4 and 8
-// are data-parallel-primitive moves inside a row of 16 lanes (full VALU rate, no LDS); 16 and 32
-// use the row / half-wave swap instructions of gfx950.
-template <int MASK>
+// Value of `x` held by lane (lane ^ MASK), MASK a power of two below 64.  Distances 1, 2 and 8 are
+// single data-parallel-primitive moves inside a row of 16 lanes (full VALU rate); 4 takes two
+// masked row shifts, 16 and 32 a row / half-wave swap of gfx950 plus a select.
+// XBAR: bit set of the distances that go through the LDS crossbar instead (ds_swizzle /
+// ds_bpermute, no memory access).  That takes instructions off the vector ALU at the price of
+// LDS latency: it pays where a merge is an occasional, vector-ALU-bound burst (bits top-k at
+// large k: +1 % at k = 512, +2.4 % at k = 2048 on 1024 x 2^20 rows) and costs where all waves
+// sort all the time (partial-bitonic-regs: -15 % at k = 32).
+constexpr int XBAR_NONE = 0;
+constexpr int XBAR_4_16_32 = 4 | 16 | 32;
+
+template <int MASK, int XBAR = XBAR_NONE>
 __device__ __forceinline__ u32 lane_xor32(u32 x)
 {
     static_assert(MASK == 1 || MASK == 2 || MASK == 4 || MASK == 8 || MASK == 16 || MASK == 32);
     const int v = static_cast<int>(x);
-    if constexpr (MASK == 1)
+    if constexpr ((XBAR & MASK) != 0 && MASK < 32)
+    {
+        // bit-mask mode: lane' = (lane & 0x1F) ^ MASK inside each half-wave
+        return static_cast<u32>(__builtin_amdgcn_ds_swizzle(v, 0x1F | (MASK << 10)));
+    }
+    else if constexpr ((XBAR & MASK) != 0)
+    {
+        return static_cast<u32>(__builtin_amdgcn_ds_bpermute(static_cast<int>((threadIdx.x ^ 32U) << 2U), v));
+    }
+    else if constexpr (MASK == 1)
     {
         return static_cast<u32>(__builtin_amdgcn_mov_dpp(v, 0xB1, 0xF, 0xF, false)); // quad_perm [1,0,3,2]
     }
@@ -56,11 +73,11 @@ __device__ __forceinline__ u32 lane_xor32(u32 x)
     }
 }
 
-template <int MASK>
+template <int MASK, int XBAR = XBAR_NONE>
 __device__ __forceinline__ u64 lane_xor(u64 x)
 {
-    const u32 lo = lane_xor32<MASK>(static_cast<u32>(x));
-    const u32 hi = lane_xor32<MASK>(static_cast<u32>(x >> 32U));
+    const u32 lo = lane_xor32<MASK, XBAR>(static_cast<u32>(x));
+    const u32 hi = lane_xor32<MASK, XBAR>(static_cast<u32>(x >> 32U));
     return (static_cast<u64>(hi) << 32U) | lo;
 }
 
@@ -105,7 +122,7 @@ __device__ __forceinline__ bool thread_bit(int t)
 // blocked order (thread t owns sorted positions t*IPT .. t*IPT+IPT-1).  K2 is the size of the
 // sequences being merged in this phase, J the exchange distance.  DESC flips the final order.
 // `t` must be the thread index whose low 6 bits are the lane index.
-template <int BS, int IPT, int K2, int J, bool DESC>
+template <int BS, int IPT, int K2, int J, bool DESC, int XBAR = XBAR_NONE>
 __device__ __forceinline__ void net_step(u64 (&x)[IPT], u64* scratch, int t)
 {
     constexpr int N = BS * IPT;
@@ -148,7 +165,7 @@ __device__ __forceinline__ void net_step(u64 (&x)[IPT], u64* scratch, int t)
 #pragma unroll
             for (int r = 0; r < IPT; ++r)
             {
-                const u64 o = lane_xor<M>(x[r]);
+                const u64 o = lane_xor<M, XBAR>(x[r]);
                 const bool take = (o < x[r]) == keep_min;
                 x[r] = take ? o : x[r];
             }
@@ -175,24 +192,24 @@ __device__ __forceinline__ void net_step(u64 (&x)[IPT], u64* scratch, int t)
     }
 }
 
-template <int BS, int IPT, int K2, int J, bool DESC>
+template <int BS, int IPT, int K2, int J, bool DESC, int XBAR = XBAR_NONE>
 __device__ __forceinline__ void net_phase(u64 (&x)[IPT], u64* scratch, int t)
 {
-    net_step<BS, IPT, K2, J, DESC>(x, scratch, t);
+    net_step<BS, IPT, K2, J, DESC, XBAR>(x, scratch, t);
     if constexpr (J > 1)
     {
-        net_phase<BS, IPT, K2, J / 2, DESC>(x, scratch, t);
+        net_phase<BS, IPT, K2, J / 2, DESC, XBAR>(x, scratch, t);
     }
 }
 
 // full bitonic sort: phases K2 = 2, 4, ..., N
-template <int BS, int IPT, int K2, bool DESC>
+template <int BS, int IPT, int K2, bool DESC, int XBAR = XBAR_NONE>
 __device__ __forceinline__ void net_sort(u64 (&x)[IPT], u64* scratch, int t)
 {
-    net_phase<BS, IPT, K2, K2 / 2, DESC>(x, scratch, t);
+    net_phase<BS, IPT, K2, K2 / 2, DESC, XBAR>(x, scratch, t);
     if constexpr (K2 < BS * IPT)
     {
-        net_sort<BS, IPT, K2 * 2, DESC>(x, scratch, t);
+        net_sort<BS, IPT, K2 * 2, DESC, XBAR>(x, scratch, t);
     }
 }
 

@@ -61,7 +61,7 @@ __device__ __forceinline__ void merge_buffer(u64 (&topk)[IPT], u64* buffer, cons
         tmp[r] = (idx % CAP) < fill[idx / CAP] ? buffer[idx] : PAD_KEY;
     }
     // (the first LDS exchange of the sort starts with a barrier, so the loads above are done)
-    net_sort<BS, IPT, 2, true>(tmp, buffer, t);
+    net_sort<BS, IPT, 2, true, XBAR_4_16_32>(tmp, buffer, t);
     // ascending list vs descending buffer: element-wise minimum keeps the N smallest of the 2N
     // keys and leaves them as a bitonic sequence
 #pragma unroll
@@ -69,7 +69,7 @@ __device__ __forceinline__ void merge_buffer(u64 (&topk)[IPT], u64* buffer, cons
     {
         topk[r] = tmp[r] < topk[r] ? tmp[r] : topk[r];
     }
-    net_phase<BS, IPT, N, N / 2, false>(topk, buffer, t);
+    net_phase<BS, IPT, N, N / 2, false, XBAR_4_16_32>(topk, buffer, t);
 }
 
 // key of sorted element k-1, broadcast to the whole workgroup (includes a barrier)
