@@ -156,3 +156,32 @@ def test_pipelined_and_plain_kernels_give_the_same_bits(bk, dev, d):
     bk.distances(more, points, bk.DIST_PARTIAL_L2, out=out_c[:, :n])
     torch.cuda.synchronize()
     assert torch.equal(out_c[:q, :n], out_a[:, :n]) and torch.equal(out_c[q:, :n], out_a[:5, :n])
+
+
+def test_config_4_full_size_samples(bk, dev):
+    """The 4096 x 2^20 x 64 distance matrix (16 GiB): a million sampled entries against float64
+    arithmetic on the same inputs (1e-5 of the scale of the cancelling terms), and whole rows
+    against the plain kernel on an unaligned copy of the problem (bit for bit)."""
+    import torch
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(4)
+    q, n, d = 4096, 1 << 20, 64
+    queries = torch.rand((d, q), device=dev, generator=gen)
+    points = torch.rand((d, n), device=dev, generator=gen)
+    out = bk.distances(queries, points, bk.DIST_PARTIAL_L2)
+    torch.cuda.synchronize()
+    qi = torch.randint(0, q, (1 << 20,), device=dev, generator=gen)
+    pj = torch.randint(0, n, (1 << 20,), device=dev, generator=gen)
+    qs = queries.double()[:, qi]
+    ps = points.double()[:, pj]
+    exact = (ps * ps).sum(0) - 2.0 * (qs * ps).sum(0)
+    scale = 2.0 * (ps * ps).sum(0) + (qs * qs).sum(0)
+    got = out[qi, pj].double()
+    assert float(((got - exact).abs() / scale).max()) < 1e-5
+    # first and last 128-query block, a slice of columns that starts inside a stage
+    sub = points[:, 5000:5000 + 8192 + 77].contiguous()
+    for q0 in (0, q - 128):
+        ref = torch.empty((128, sub.shape[1] + 1), device=dev)
+        bk.distances(queries[:, q0:q0 + 128].contiguous(), sub, bk.DIST_PARTIAL_L2, out=ref[:, :sub.shape[1]])
+        torch.cuda.synchronize()
+        assert torch.equal(ref[:, :sub.shape[1]], out[q0:q0 + 128, 5000:5000 + sub.shape[1]])
