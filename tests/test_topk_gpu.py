@@ -212,3 +212,30 @@ def test_full_size_properties(bk, dev):
         assert bool(((m < kth).sum(dim=1) <= k - 1).all())
     del m
     torch.cuda.empty_cache()
+
+
+def test_random_shapes_against_the_oracle(bk, dev, oracle):
+    """150 random problems: ragged lengths around every chunk boundary, all block and batch sizes,
+    uniform / heavily tied / sorted rows, with and without the prefetching variant."""
+    rng = np.random.default_rng(2024)
+    for case in range(150):
+        block = int(rng.choice([128, 256, 512]))
+        batch = int(rng.integers(1, 17))
+        k = int(rng.choice([1, 7, 16, 32, 100, 256, 512, 1000, 2048]))
+        if k // block > 16:
+            k = block * 16
+        rows = int(rng.integers(1, 5))
+        kind = case % 5
+        cols = int(rng.integers(1, 150000)) if kind else int(block * 4 * ((batch + 3) // 4) * rng.integers(1, 9) + rng.integers(-2, 3) + max(k, block))
+        cols = max(cols, 1)
+        m = oracle.uniform_matrix(5000 + case, rows, cols)
+        if kind == 1:
+            m = (np.floor(m * 8) / 8).astype(np.float32)
+        elif kind == 2:
+            m = np.sort(m, axis=1)
+        elif kind == 3:
+            m = np.ascontiguousarray(np.sort(m, axis=1)[:, ::-1])
+        gd, gl = _run(bk, dev, m, k, block=block, batch=batch, prefetch=bool(case & 1))
+        ed, el = oracle.topk(m, k)
+        assert np.array_equal(gd.view(np.uint32), ed.view(np.uint32)), (case, block, batch, k, rows, cols, kind)
+        assert np.array_equal(gl, el), (case, block, batch, k, rows, cols, kind)
