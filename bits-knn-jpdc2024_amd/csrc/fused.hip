@@ -228,34 +228,46 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 
     // ---- filter one 32 x 32 tile held in `acc` and append what passes ---------------------------
     // lane holds 16 distances of query ql: rows 8*(r/4) + 4*half + r%4 of the tile
+    const int partner_addr = (lane ^ 32) << 2; // byte address of the lane that shares this lane's query
     auto append_tile = [&](const vfloat16& acc, int tile_base) {
-        int mine = 0;
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-        {
-            mine += acc[r] < radius ? 1 : 0;
-        }
-        int other = __shfl_xor(mine, 32, WAVE);
-        if (__builtin_amdgcn_ballot_w64(fill + mine + other > FQ_CAP) != 0)
-        {
-            merge_event();
-            mine = 0;
+        // One compare per value: its lane mask stays in scalar registers and serves the count and
+        // the predicate of the write (scalar instructions cost a quarter of a vector one, and
+        // vector instructions are not overlapped with the matrix instructions of either wave).
+        u64 pass[16];
+        auto compare = [&]() -> int {
 #pragma unroll
             for (int r = 0; r < 16; ++r)
             {
-                mine += acc[r] < radius ? 1 : 0;
+                pass[r] = __builtin_amdgcn_ballot_w64(acc[r] < radius);
             }
-            other = __shfl_xor(mine, 32, WAVE);
+            int count = 0;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+            {
+                count += __builtin_amdgcn_inverse_ballot_w64(pass[r]) ? 1 : 0;
+            }
+            return count;
+        };
+        int mine = compare();
+        int other = __builtin_amdgcn_ds_bpermute(partner_addr, mine);
+        if (__builtin_amdgcn_ballot_w64(fill + mine + other > FQ_CAP) != 0)
+        {
+            merge_event();
+            mine = compare();
+            other = __builtin_amdgcn_ds_bpermute(partner_addr, mine);
         }
         int slot = fill + (half != 0 ? other : 0);
         const int first_point = tile_base + 4 * half;
 #pragma unroll
         for (int r = 0; r < 16; ++r)
         {
-            if (acc[r] < radius)
+            if (pass[r] != 0)
             {
-                wbuf[ql * FQ_CAP + slot] = make_key(acc[r], first_point + 8 * (r / 4) + (r % 4));
-                ++slot;
+                if (__builtin_amdgcn_inverse_ballot_w64(pass[r]))
+                {
+                    wbuf[ql * FQ_CAP + slot] = make_key(acc[r], first_point + 8 * (r / 4) + (r % 4));
+                    ++slot;
+                }
             }
         }
         fill += mine + other;
