@@ -183,6 +183,60 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     {
         v[j] = 0.0F;
     }
+    // the values of the chunk that starts at column `first`, value j of thread t as column_of says
+    auto load_chunk = [&](float (&dst)[E], u32 first) {
+        if (first < full_end)
+        {
+            if constexpr (VEC)
+            {
+                const vfloat4* __restrict__ p = reinterpret_cast<const vfloat4*>(row + first) + t;
+#pragma unroll
+                for (int l = 0; l < L; ++l)
+                {
+                    const vfloat4 x = __builtin_nontemporal_load(p + l * BS);
+                    dst[4 * l + 0] = x.x;
+                    dst[4 * l + 1] = x.y;
+                    dst[4 * l + 2] = x.z;
+                    dst[4 * l + 3] = x.w;
+                }
+            }
+            else
+            {
+                const float* __restrict__ p = row + first + t;
+#pragma unroll
+                for (int j = 0; j < E; ++j)
+                {
+                    dst[j] = __builtin_nontemporal_load(p + j * BS);
+                }
+            }
+        }
+        else
+        {
+            // ragged tail: bounds-checked 4-byte loads in the same value-to-thread mapping
+#pragma unroll
+            for (int j = 0; j < E; ++j)
+            {
+                const u32 col = column_of(first, j);
+                dst[j] = col < n ? row[col] : __builtin_inff();
+            }
+        }
+    };
+    // Software pipelining for small batches: the next chunk is requested before the current one
+    // is filtered, at the price of E more registers and E moves per chunk.
+    constexpr bool PIPE = L <= 2;
+    float ahead[E];
+#pragma unroll
+    for (int j = 0; j < E; ++j)
+    {
+        ahead[j] = 0.0F;
+    }
+    if constexpr (PIPE)
+    {
+        if (left > 0)
+        {
+            load_chunk(ahead, chunk);
+        }
+    }
 
     // Fill of this wave's slice (wave-uniform).  Passing values take slots in the order
     // (value index j, lane): value j of the lanes in its pass mask gets consecutive slots after
@@ -301,46 +355,33 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
         // ---- streaming: no synchronisation with the other waves except polling the flag
         while (left > 0)
         {
-            if (chunk < full_end)
+            if constexpr (PIPE)
             {
-                if constexpr (VEC)
-                {
-                    const vfloat4* __restrict__ p = reinterpret_cast<const vfloat4*>(row + chunk) + t;
+                // the values of this chunk were requested an iteration (or a merge) ago
 #pragma unroll
-                    for (int l = 0; l < L; ++l)
-                    {
-                        const vfloat4 x = __builtin_nontemporal_load(p + l * BS);
-                        v[4 * l + 0] = x.x;
-                        v[4 * l + 1] = x.y;
-                        v[4 * l + 2] = x.z;
-                        v[4 * l + 3] = x.w;
-                    }
-                }
-                else
+                for (int j = 0; j < E; ++j)
                 {
-                    const float* __restrict__ p = row + chunk + t;
-#pragma unroll
-                    for (int j = 0; j < E; ++j)
-                    {
-                        v[j] = __builtin_nontemporal_load(p + j * BS);
-                    }
+                    v[j] = ahead[j];
                 }
             }
             else
             {
-                // ragged tail: bounds-checked 4-byte loads in the same value-to-thread mapping
-#pragma unroll
-                for (int j = 0; j < E; ++j)
-                {
-                    const u32 col = column_of(chunk, j);
-                    v[j] = col < n ? row[col] : __builtin_inff();
-                }
+                load_chunk(v, chunk);
             }
             const int flag = *static_cast<volatile int*>(&s_flag);
             cur_chunk = chunk;
             left -= 1;
             chunk += static_cast<u32>(jump);
             jump = (jump > 0 ? static_cast<std::int32_t>(CHUNK) : -static_cast<std::int32_t>(CHUNK)) - jump;
+            if constexpr (PIPE)
+            {
+                // request the next chunk before this one is filtered: the loads stay in flight
+                // through the filter and through a merge, if one comes
+                if (left > 0)
+                {
+                    load_chunk(ahead, chunk);
+                }
+            }
 
             float smallest = v[0];
 #pragma unroll
