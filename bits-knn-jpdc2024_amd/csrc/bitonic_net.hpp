@@ -122,8 +122,11 @@ __device__ __forceinline__ bool thread_bit(int t)
 // blocked order (thread t owns sorted positions t*IPT .. t*IPT+IPT-1).  K2 is the size of the
 // sequences being merged in this phase, J the exchange distance.  DESC flips the final order.
 // `t` must be the thread index whose low 6 bits are the lane index.
-template <int BS, int IPT, int K2, int J, bool DESC, int XBAR = XBAR_NONE>
-__device__ __forceinline__ void net_step(u64 (&x)[IPT], u64* scratch, int t)
+// PP: `scratch` has room for 2N keys and consecutive LDS exchanges alternate between its halves
+// (`flip`, the same in every thread), which saves the barrier that otherwise protects the readers
+// of one exchange from the writers of the next.
+template <int BS, int IPT, int K2, int J, bool DESC, int XBAR = XBAR_NONE, bool PP = false>
+__device__ __forceinline__ void net_step(u64 (&x)[IPT], u64* scratch, int t, int& flip)
 {
     constexpr int N = BS * IPT;
     if constexpr (J < IPT)
@@ -174,17 +177,26 @@ __device__ __forceinline__ void net_step(u64 (&x)[IPT], u64* scratch, int t)
         {
             // partner lives in another wave: exchange through LDS, striped so that neighbouring
             // lanes touch neighbouring 8-byte slots
-            __syncthreads();
+            u64* half = scratch;
+            if constexpr (PP)
+            {
+                half = scratch + (flip != 0 ? N : 0);
+                flip ^= 1;
+            }
+            else
+            {
+                __syncthreads();
+            }
 #pragma unroll
             for (int r = 0; r < IPT; ++r)
             {
-                scratch[r * BS + t] = x[r];
+                half[r * BS + t] = x[r];
             }
             __syncthreads();
 #pragma unroll
             for (int r = 0; r < IPT; ++r)
             {
-                const u64 o = scratch[r * BS + (t ^ M)];
+                const u64 o = half[r * BS + (t ^ M)];
                 const bool take = (o < x[r]) == keep_min;
                 x[r] = take ? o : x[r];
             }
@@ -192,25 +204,40 @@ __device__ __forceinline__ void net_step(u64 (&x)[IPT], u64* scratch, int t)
     }
 }
 
-template <int BS, int IPT, int K2, int J, bool DESC, int XBAR = XBAR_NONE>
-__device__ __forceinline__ void net_phase(u64 (&x)[IPT], u64* scratch, int t)
+template <int BS, int IPT, int K2, int J, bool DESC, int XBAR = XBAR_NONE, bool PP = false>
+__device__ __forceinline__ void net_phase(u64 (&x)[IPT], u64* scratch, int t, int& flip)
 {
-    net_step<BS, IPT, K2, J, DESC, XBAR>(x, scratch, t);
+    net_step<BS, IPT, K2, J, DESC, XBAR, PP>(x, scratch, t, flip);
     if constexpr (J > 1)
     {
-        net_phase<BS, IPT, K2, J / 2, DESC, XBAR>(x, scratch, t);
+        net_phase<BS, IPT, K2, J / 2, DESC, XBAR, PP>(x, scratch, t, flip);
     }
 }
 
 // full bitonic sort: phases K2 = 2, 4, ..., N
-template <int BS, int IPT, int K2, bool DESC, int XBAR = XBAR_NONE>
-__device__ __forceinline__ void net_sort(u64 (&x)[IPT], u64* scratch, int t)
+template <int BS, int IPT, int K2, bool DESC, int XBAR = XBAR_NONE, bool PP = false>
+__device__ __forceinline__ void net_sort(u64 (&x)[IPT], u64* scratch, int t, int& flip)
 {
-    net_phase<BS, IPT, K2, K2 / 2, DESC, XBAR>(x, scratch, t);
+    net_phase<BS, IPT, K2, K2 / 2, DESC, XBAR, PP>(x, scratch, t, flip);
     if constexpr (K2 < BS * IPT)
     {
-        net_sort<BS, IPT, K2 * 2, DESC, XBAR>(x, scratch, t);
+        net_sort<BS, IPT, K2 * 2, DESC, XBAR, PP>(x, scratch, t, flip);
     }
+}
+
+// single-buffer forms (two barriers per LDS exchange)
+template <int BS, int IPT, int K2, int J, bool DESC>
+__device__ __forceinline__ void net_phase(u64 (&x)[IPT], u64* scratch, int t)
+{
+    int unused = 0;
+    net_phase<BS, IPT, K2, J, DESC, XBAR_NONE, false>(x, scratch, t, unused);
+}
+
+template <int BS, int IPT, int K2, bool DESC>
+__device__ __forceinline__ void net_sort(u64 (&x)[IPT], u64* scratch, int t)
+{
+    int unused = 0;
+    net_sort<BS, IPT, K2, DESC, XBAR_NONE, false>(x, scratch, t, unused);
 }
 
 } // namespace bitsknn

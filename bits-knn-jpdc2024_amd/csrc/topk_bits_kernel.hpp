@@ -60,8 +60,11 @@ __device__ __forceinline__ void merge_buffer(u64 (&topk)[IPT], u64* buffer, cons
         const int idx = r * BS + t;
         tmp[r] = (idx % CAP) < fill[idx / CAP] ? buffer[idx] : PAD_KEY;
     }
-    // (the first LDS exchange of the sort starts with a barrier, so the loads above are done)
-    net_sort<BS, IPT, 2, true, XBAR_4_16_32>(tmp, buffer, t);
+    // LDS exchanges alternate between the N keys after the buffer and the buffer itself,
+    // starting with the former: by the time the buffer is overwritten every thread has passed the
+    // barrier of the first exchange and so has read its keys above.  One barrier per exchange.
+    int flip = 1;
+    net_sort<BS, IPT, 2, true, XBAR_4_16_32, true>(tmp, buffer, t, flip);
     // ascending list vs descending buffer: element-wise minimum keeps the N smallest of the 2N
     // keys and leaves them as a bitonic sequence
 #pragma unroll
@@ -69,7 +72,7 @@ __device__ __forceinline__ void merge_buffer(u64 (&topk)[IPT], u64* buffer, cons
     {
         topk[r] = tmp[r] < topk[r] ? tmp[r] : topk[r];
     }
-    net_phase<BS, IPT, N, N / 2, false, XBAR_4_16_32>(topk, buffer, t);
+    net_phase<BS, IPT, N, N / 2, false, XBAR_4_16_32, true>(topk, buffer, t, flip);
 }
 
 // key of sorted element k-1, broadcast to the whole workgroup (includes a barrier)
@@ -100,7 +103,7 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     constexpr u32 CHUNK = BS * E;    // values per workgroup and iteration
     static_assert(E <= 32, "one pass bit per value in a 32-bit lane mask");
 
-    __shared__ u64 buffer[NL];
+    __shared__ u64 buffer[2 * NL];   // candidates; the second half is exchange space of the merges
     __shared__ u64 s_radius;
     __shared__ int s_fill[W];
     __shared__ int s_flag;  // some wave wants a merge
