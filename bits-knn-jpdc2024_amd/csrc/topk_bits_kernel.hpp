@@ -320,19 +320,26 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
         if (total > 0)
         {
             merge_buffer<BS, IPT>(topk, buffer, s_fill, t);
+            // the barriers of the merge lie between the reads above and this reset; the barrier
+            // of the broadcast publishes it together with the radius
+            if (t == 0)
+            {
+                s_flag = 0;
+                s_more = 0;
+            }
             radius_key = broadcast_radius<IPT>(topk, a.k, &s_radius, t);
             radius = key_value(radius_key);
         }
         else
         {
             __syncthreads(); // orders the reads above before the reset below
+            if (t == 0)
+            {
+                s_flag = 0;
+                s_more = 0;
+            }
+            __syncthreads();
         }
-        if (t == 0)
-        {
-            s_flag = 0;
-            s_more = 0;
-        }
-        __syncthreads();
         if (!more)
         {
             break;
