@@ -16,7 +16,10 @@
 //    in LDS and waits at a barrier; the others poll the flag once per batch and join.  The only
 //    barriers are those of a merge;
 //  * exchange distances below 64 lanes stay inside a wave, only distances of 64 lanes and more
-//    go through LDS.
+//    go through LDS (two alternating regions, one barrier per exchange);
+//  * the chunks of a row are visited from both ends inwards, so that sorted rows of either
+//    direction tighten the radius at once, and for small batches the next chunk is requested
+//    before the current one is filtered.
 // Because waves drift apart, the filter compares full keys when a value equals the radius, so
 // that "equal values by lower label" holds no matter which wave saw which value first.
 
