@@ -541,6 +541,20 @@ int choose_splits(int q, int n)
     return splits;
 }
 
+// Long lists (k >= 64): the 32-slot buffers of the fused kernel make every merge pay for the whole
+// list, and its time grows almost linearly with k.  When the caller's workspace can hold the
+// q x n distance matrix (at most 16 GiB), the entry point with a workspace therefore computes the
+// matrix there with the MFMA distance kernel and selects with the bits kernel: two passes whose
+// time does not depend on k.  The matrix never leaves the workspace.
+constexpr int TWO_PASS_MIN_K = 64;
+constexpr size_t TWO_PASS_MAX_BYTES = 16ULL << 30;
+
+size_t two_pass_bytes(std::int32_t q, std::int32_t n, int k)
+{
+    const size_t bytes = static_cast<size_t>(q) * static_cast<size_t>(n) * sizeof(float);
+    return k >= TWO_PASS_MIN_K && bytes <= TWO_PASS_MAX_BYTES ? bytes : 0;
+}
+
 int fused_impl(const float* queries_dim_major, const float* points_dim_major, int dim, std::int32_t q,
                std::int32_t n, float* out_dist, std::int32_t* out_label, int k, int query_reg,
                int db_reg, int dim_reg, int block_query_dim, int dim_mult, void* workspace,
@@ -598,6 +612,26 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     if (static_cast<size_t>(q) > 65535U * FQ_QB)
     {
         return fail(BITSKNN_ERR_INVALID, "bitsknn_fused_l2_topk_f32: too many queries: %d", q);
+    }
+
+    const size_t matrix_bytes = use_workspace ? two_pass_bytes(q, n, k) : 0;
+    if (matrix_bytes != 0 && workspace != nullptr && workspace_bytes >= matrix_bytes &&
+        reinterpret_cast<std::uintptr_t>(workspace) % 16 == 0)
+    {
+        auto* matrix = static_cast<float*>(workspace);
+        const int status = bitsknn_dist_f32(BITSKNN_DIST_PARTIAL_L2, dim, static_cast<size_t>(q),
+                                            static_cast<size_t>(n), queries_dim_major, static_cast<size_t>(q),
+                                            points_dim_major, static_cast<size_t>(n), matrix,
+                                            static_cast<size_t>(n), stream);
+        if (status != BITSKNN_OK)
+        {
+            return status;
+        }
+        // block size and batch as tuned for rows of this length (k = 64: 256 x 8, longer lists: 512 x 3)
+        return bitsknn_topk_bits_f32(matrix, static_cast<size_t>(n), nullptr, 0, nullptr, static_cast<size_t>(q),
+                                     static_cast<size_t>(n), out_dist, out_label, static_cast<size_t>(k),
+                                     static_cast<std::uint32_t>(k), k <= 64 ? 256 : 512, k <= 64 ? 8 : 3, 0,
+                                     stream);
     }
 
     int splits = use_workspace ? choose_splits(q, n) : 1;
@@ -675,6 +709,11 @@ extern "C" size_t bitsknn_fused_workspace_bytes(int32_t q, int32_t n, int k)
     if (q <= 0 || n <= 0 || k <= 0)
     {
         return 0;
+    }
+    const size_t matrix_bytes = bitsknn::two_pass_bytes(q, n, k);
+    if (matrix_bytes != 0)
+    {
+        return matrix_bytes;
     }
     const int splits = bitsknn::choose_splits(q, n);
     return splits > 1 ? static_cast<size_t>(q) * static_cast<size_t>(splits) * static_cast<size_t>(k) * 8 : 0;

@@ -135,17 +135,22 @@ int bitsknn_fused_l2_topk_f32(const float* queries_dim_major, const float* point
                               int dim_mult, void* stream);
 
 /*
- * bits-fused with a caller-provided workspace.  Same results as bitsknn_fused_l2_topk_f32.
+ * bits-fused with a caller-provided workspace.  Same neighbours as bitsknn_fused_l2_topk_f32.
  * When there are too few queries to fill the GPU with one workgroup per 128 queries, the points
  * are cut into ranges that are searched by separate workgroups; their partial lists go to the
  * workspace and one bits pass (explicit labels) selects the final k.
+ * For k >= 64, when the q x n distance matrix fits 16 GiB, bitsknn_fused_workspace_bytes asks for
+ * room for that matrix and the call runs the MFMA distance kernel into the workspace followed by
+ * the bits kernel (the fused kernel's 32-slot buffers make its time grow with k; the two passes
+ * do not).  A smaller workspace, or bitsknn_fused_l2_topk_f32, keeps the single fused kernel.
  *
  * No counterpart in the reference, whose fused kernel always runs one thread block per query tile
  * (src/topk/singlepass/fused_cache_knn.cu:60-69); the host wrapper that owns the device memory
  * (fused_cache_knn::initialize, fused_cache_knn.cu:149-195) is where the workspace is allocated.
  *
- * bitsknn_fused_workspace_bytes returns the size the call needs (0: no split, workspace unused).
- * Errors as for bitsknn_fused_l2_topk_f32, plus BITSKNN_ERR_INVALID for a workspace too small.
+ * bitsknn_fused_workspace_bytes returns the size the call wants (0: workspace unused).
+ * Errors as for bitsknn_fused_l2_topk_f32, plus BITSKNN_ERR_INVALID for a workspace too small
+ * for the partial lists.
  */
 size_t bitsknn_fused_workspace_bytes(int32_t q, int32_t n, int k);
 int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major, const float* points_dim_major,

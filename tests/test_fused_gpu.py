@@ -98,9 +98,18 @@ def test_ragged_counts(bk, dev, oracle, n, q):
 def test_point_split_variant_with_workspace(bk, dev, oracle, n, q, d, k):
     """The workspace entry point cuts the points into ranges when queries are few; its result must
     equal the plain entry point's bit for bit (same distances, canonical ties)."""
+    import torch
     p, s = oracle.generate(n + q + d, n, q, d)
-    assert bk.fused_workspace_bytes(q, n, k) % (8 * q * k) == 0
-    gd, gl = _fused(bk, dev, p, s, k, workspace="auto")
+    if k < 64:
+        assert bk.fused_workspace_bytes(q, n, k) % (8 * q * k) == 0
+        workspace = "auto"
+    else:
+        # long lists ask for the whole distance matrix (two passes); a workspace for the partial
+        # lists of up to 64 ranges only keeps the fused kernel
+        assert bk.fused_workspace_bytes(q, n, k) == q * n * 4
+        assert 8 * q * 64 * k < q * n * 4
+        workspace = torch.empty(8 * q * 64 * k, dtype=torch.uint8, device=dev)
+    gd, gl = _fused(bk, dev, p, s, k, workspace=workspace)
     _check(oracle, p, s, k, gd, gl)
     pd, pl = _fused(bk, dev, p, s, k)
     assert np.array_equal(gd, pd) and np.array_equal(gl, pl)
@@ -192,3 +201,24 @@ def test_point_matrix_of_2_gib_takes_the_plain_loads(bk, dev):
     # and the reported distances belong to the reported labels
     at = torch.gather(dist, 1, fl.long())
     assert float(((fd.double() - at.double()).abs() / scale).max()) < 1e-5
+
+
+@pytest.mark.parametrize("k", [64, 128, 256])
+def test_long_lists_with_a_workspace_take_two_passes(bk, dev, oracle, k):
+    """k >= 64 with a workspace that holds the q x n matrix: MFMA distances + bits top-k.  Same
+    bar as the fused kernel, and the same neighbours as the fused kernel without a workspace."""
+    import torch
+    n, q, d = 20000, 300, 24
+    points, queries = oracle.generate(77, n, q, d)
+    assert bk.fused_workspace_bytes(q, n, k) == q * n * 4
+    assert bk.fused_workspace_bytes(q, n, 32) < q * n * 4
+    gd, gl = _fused(bk, dev, points, queries, k, workspace="auto")
+    _check(oracle, points, queries, k, gd, gl)
+    fd, fl = _fused(bk, dev, points, queries, k)
+    same = np.mean([len(set(a) & set(b)) / k for a, b in zip(gl, fl)])
+    assert same >= 0.999
+    # a workspace that only holds the partial lists keeps the fused kernel
+    small = torch.empty(8 * q * 8 * k, dtype=torch.uint8, device=dev)
+    assert small.numel() < q * n * 4
+    sd, sl = _fused(bk, dev, points, queries, k, workspace=small)
+    _check(oracle, points, queries, k, sd, sl)
