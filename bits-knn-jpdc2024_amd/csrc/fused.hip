@@ -108,7 +108,8 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     constexpr int MT = G::MT;
     // merge layout: S keys per query spread over LPQ lanes, R keys per lane
     constexpr int S = K > FQ_CAP ? K : FQ_CAP;
-    constexpr int R = 4;
+    // (16 lanes per query for long lists: fewer, wider passes hide the latency of the list traffic)
+    constexpr int R = S <= 64 ? 4 : 8;
     constexpr int LPQ = S / R;
     constexpr int QPP = WAVE / LPQ;           // queries per merge pass
     constexpr int PASSES = FQ_QW / QPP;
@@ -161,11 +162,41 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     bool have_list = false;          // wave-uniform: the lists in the output arrays are valid
 
     // ---- merge of all buffers of this wave into the lists --------------------------------------
-    auto merge_event = [&]() {
+    auto merge_event = [&]() __attribute__((always_inline)) {
         reinterpret_cast<int*>(wx)[32 + ql] = fill;
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if constexpr (K > FQ_CAP)
+        {
+            // Lists longer than a buffer: the buffers are sorted in place first, 8 queries at a
+            // time, so that the passes below only pay for the merge network of the list.
+            constexpr int BR = 4;           // keys per lane
+            constexpr int BL = FQ_CAP / BR; // lanes per buffer
+#pragma unroll 1
+            for (int pass = 0; pass < FQ_QW / (WAVE / BL); ++pass)
+            {
+                const int qm = pass * (WAVE / BL) + lane / BL;
+                const int sub = lane % BL;
+                const int used = reinterpret_cast<const int*>(wx)[32 + qm];
+                u64 buf[BR];
+#pragma unroll
+                for (int r = 0; r < BR; ++r)
+                {
+                    const int i = sub * BR + r;
+                    buf[r] = i < used ? wbuf[qm * FQ_CAP + i] : PAD_KEY;
+                }
+                net_sort<BL, BR, 2, true>(buf, nullptr, sub);
+#pragma unroll
+                for (int r = 0; r < BR; ++r)
+                {
+                    wbuf[qm * FQ_CAP + sub * BR + r] = buf[r];
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
 #pragma unroll 1
         for (int pass = 0; pass < PASSES; ++pass)
         {
@@ -179,7 +210,16 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             for (int r = 0; r < R; ++r)
             {
                 const int i = sub * R + r;
-                buf[r] = i < used ? wbuf[qm * FQ_CAP + (i < FQ_CAP ? i : 0)] : PAD_KEY;
+                if constexpr (K > FQ_CAP)
+                {
+                    // the sorted buffer (descending, padding first) is the tail of a descending
+                    // sequence of K keys
+                    buf[r] = i >= K - FQ_CAP ? wbuf[qm * FQ_CAP + i - (K - FQ_CAP)] : PAD_KEY;
+                }
+                else
+                {
+                    buf[r] = i < used ? wbuf[qm * FQ_CAP + (i < FQ_CAP ? i : 0)] : PAD_KEY;
+                }
                 list[r] = PAD_KEY;
                 if (have_list && i < K && gq < a.q)
                 {
@@ -192,7 +232,10 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 }
             }
             // buffer descending, element-wise minimum with the ascending list, re-sort
-            net_sort<LPQ, R, 2, true>(buf, nullptr, sub);
+            if constexpr (K <= FQ_CAP)
+            {
+                net_sort<LPQ, R, 2, true>(buf, nullptr, sub);
+            }
 #pragma unroll
             for (int r = 0; r < R; ++r)
             {
@@ -229,7 +272,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     // ---- filter one 32 x 32 tile held in `acc` and append what passes ---------------------------
     // lane holds 16 distances of query ql: rows 8*(r/4) + 4*half + r%4 of the tile
     const int partner_addr = (lane ^ 32) << 2; // byte address of the lane that shares this lane's query
-    auto append_tile = [&](const vfloat16& acc, int tile_base) {
+    auto append_tile = [&](const vfloat16& acc, int tile_base) __attribute__((always_inline)) {
         // One compare per value: its lane mask stays in scalar registers and serves the count and
         // the predicate of the write (scalar instructions cost a quarter of a vector one, and
         // vector instructions are not overlapped with the matrix instructions of either wave).
@@ -272,7 +315,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         }
         fill += mine + other;
     };
-    auto filter_tile = [&](const vfloat16& acc, int tile_base) {
+    auto filter_tile = [&](const vfloat16& acc, int tile_base) __attribute__((always_inline)) {
         float smallest = acc[0];
 #pragma unroll
         for (int r = 1; r < 16; ++r)
