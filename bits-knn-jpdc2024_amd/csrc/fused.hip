@@ -197,15 +197,46 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
+        // The list of a query is read by the lanes that wrote it in the previous merge (same
+        // pass, same positions), so plain loads and stores in program order are enough.  The list
+        // of the next pass is requested before the network of this one runs.
+        const int sub = lane % LPQ;
+        float next_dist[R];
+        std::int32_t next_label[R];
+        auto request_list = [&](int pass) __attribute__((always_inline)) {
+            const int gq = wave_q0 + pass * QPP + lane / LPQ;
+            const size_t at = (static_cast<size_t>(gq) * a.splits + blockIdx.y) * K + sub * R;
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+            {
+                next_dist[r] = __builtin_inff();
+                next_label[r] = 0x7FFFFFFF;
+                if (have_list && sub * R + r < K && gq < a.q)
+                {
+                    next_dist[r] = a.out_dist[at + r];
+                    next_label[r] = a.out_label[at + r];
+                }
+            }
+        };
+        // (with 8 keys per lane the registers for a request in flight would cost a workgroup per
+        // compute unit)
+        constexpr bool AHEAD = R <= 4;
+        if constexpr (AHEAD)
+        {
+            request_list(0);
+        }
 #pragma unroll 1
         for (int pass = 0; pass < PASSES; ++pass)
         {
             const int qm = pass * QPP + lane / LPQ; // query (inside the wave) of this lane group
-            const int sub = lane % LPQ;
             const int gq = wave_q0 + qm;
             const int used = reinterpret_cast<const int*>(wx)[32 + qm];
             u64 buf[R];
             u64 list[R];
+            if constexpr (!AHEAD)
+            {
+                request_list(pass);
+            }
 #pragma unroll
             for (int r = 0; r < R; ++r)
             {
@@ -220,16 +251,11 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 {
                     buf[r] = i < used ? wbuf[qm * FQ_CAP + (i < FQ_CAP ? i : 0)] : PAD_KEY;
                 }
-                list[r] = PAD_KEY;
-                if (have_list && i < K && gq < a.q)
-                {
-                    const size_t at = (static_cast<size_t>(gq) * a.splits + blockIdx.y) * K + i;
-                    const float dv = __hip_atomic_load(a.out_dist + at, __ATOMIC_RELAXED,
-                                                       __HIP_MEMORY_SCOPE_AGENT);
-                    const std::int32_t lv = __hip_atomic_load(a.out_label + at, __ATOMIC_RELAXED,
-                                                              __HIP_MEMORY_SCOPE_AGENT);
-                    list[r] = make_key(dv, lv);
-                }
+                list[r] = make_key(next_dist[r], next_label[r]);
+            }
+            if (AHEAD && pass + 1 < PASSES)
+            {
+                request_list(pass + 1);
             }
             // buffer descending, element-wise minimum with the ascending list, re-sort
             if constexpr (K <= FQ_CAP)
@@ -249,10 +275,8 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 if (i < K && gq < a.q)
                 {
                     const size_t at = (static_cast<size_t>(gq) * a.splits + blockIdx.y) * K + i;
-                    __hip_atomic_store(a.out_dist + at, key_value(list[r]), __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-                    __hip_atomic_store(a.out_label + at, key_label(list[r]), __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
+                    a.out_dist[at] = key_value(list[r]);
+                    a.out_label[at] = key_label(list[r]);
                 }
                 if (i == K - 1)
                 {
@@ -260,10 +284,9 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 }
             }
         }
-        // the next merge of this wave reads the lists back with other lanes
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         radius = wx[ql];
         fill = 0;
         have_list = true;
