@@ -607,12 +607,12 @@ int choose_splits(int q, int n)
     return splits;
 }
 
-// Long lists (k >= 64): the 32-slot buffers of the fused kernel make every merge pay for the whole
-// list, and its time grows almost linearly with k.  When the caller's workspace can hold the
+// Long lists (k >= 128): the 32-slot buffers of the fused kernel make every merge pay for the whole
+// list, and its time grows with k.  When the caller's workspace can hold the
 // q x n distance matrix (at most 16 GiB), the entry point with a workspace therefore computes the
 // matrix there with the MFMA distance kernel and selects with the bits kernel: two passes whose
 // time does not depend on k.  The matrix never leaves the workspace.
-constexpr int TWO_PASS_MIN_K = 64;
+constexpr int TWO_PASS_MIN_K = 128;
 constexpr size_t TWO_PASS_MAX_BYTES = 16ULL << 30;
 
 size_t two_pass_bytes(std::int32_t q, std::int32_t n, int k)
@@ -693,10 +693,9 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
         {
             return status;
         }
-        // block size and batch as tuned for rows of this length (k = 64: 256 x 8, longer lists: 512 x 3)
         return bitsknn_topk_bits_f32(matrix, static_cast<size_t>(n), nullptr, 0, nullptr, static_cast<size_t>(q),
                                      static_cast<size_t>(n), out_dist, out_label, static_cast<size_t>(k),
-                                     static_cast<std::uint32_t>(k), k <= 64 ? 256 : 512, k <= 64 ? 8 : 3, 0,
+                                     static_cast<std::uint32_t>(k), 512, 3, 0,
                                      stream);
     }
 

@@ -139,7 +139,7 @@ int bitsknn_fused_l2_topk_f32(const float* queries_dim_major, const float* point
  * When there are too few queries to fill the GPU with one workgroup per 128 queries, the points
  * are cut into ranges that are searched by separate workgroups; their partial lists go to the
  * workspace and one bits pass (explicit labels) selects the final k.
- * For k >= 64, when the q x n distance matrix fits 16 GiB, bitsknn_fused_workspace_bytes asks for
+ * For k >= 128, when the q x n distance matrix fits 16 GiB, bitsknn_fused_workspace_bytes asks for
  * room for that matrix and the call runs the MFMA distance kernel into the workspace followed by
  * the bits kernel (the fused kernel's 32-slot buffers make its time grow with k; the two passes
  * do not).  A smaller workspace, or bitsknn_fused_l2_topk_f32, keeps the single fused kernel.
