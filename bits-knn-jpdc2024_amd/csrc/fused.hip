@@ -53,6 +53,14 @@ __device__ __forceinline__ void static_for(F&& f)
 
 typedef float vfloat16 __attribute__((ext_vector_type(16)));
 
+// minimum of three values in one instruction; a NaN operand is ignored
+__device__ __forceinline__ float min3(float a, float b, float c)
+{
+    float r;
+    asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 constexpr int FQ_WAVES = 4;                   // waves per workgroup
 constexpr int FQ_THREADS = FQ_WAVES * WAVE;   // 256
 constexpr int FQ_QW = 32;                     // queries per wave (one MFMA column tile)
@@ -339,12 +347,14 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         fill += mine + other;
     };
     auto filter_tile = [&](const vfloat16& acc, int tile_base) __attribute__((always_inline)) {
-        float smallest = acc[0];
+        // (written out: fminf would first quieten each operand with an instruction of its own)
+        float smallest = min3(acc[0], acc[1], acc[2]);
 #pragma unroll
-        for (int r = 1; r < 16; ++r)
+        for (int r = 3; r < 15; r += 2)
         {
-            smallest = fminf(smallest, acc[r]);
+            smallest = min3(smallest, acc[r], acc[r + 1]);
         }
+        smallest = min3(smallest, acc[15], acc[15]);
         if (__builtin_amdgcn_ballot_w64(smallest < radius) != 0)
         {
             append_tile(acc, tile_base);
@@ -356,7 +366,6 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     // stage and adds up its share of ||p||^2 (the shares of a point meet inside the MFMA)
     const int sp = t % PT;
     const int sd0 = t / PT;
-    const bool whole_dim = dim == DP;
     float pre[VPT];
     // Point values are read with buffer loads: a constant byte offset per value and lane (beyond
     // the resource for dimensions dim .. DP-1, which then read as zero; the hardware checks the
@@ -424,10 +433,8 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         {
             const int dd = sd0 + TPP * i;
             share = __builtin_fmaf(pre[i], pre[i], share);
-            if (whole_dim || dd < dim)
-            {
-                stage[dd * PT + sp] = pre[i];
-            }
+            // (dimensions from dim on were read as zero: their rows stay zero)
+            stage[dd * PT + sp] = pre[i];
         }
         // points beyond the end get an infinite distance and never pass the filter
         stage[(DP + sd0) * PT + sp] = base + sp < n ? share : __builtin_inff();
