@@ -300,25 +300,27 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         have_list = true;
     };
 
+    // position of this lane's A operands inside a stage row, for the two tiles of a pair (the
+    // second one is kept opaque so that it stays a base register of its own)
+    int tile_at[2] = {half * PT + ql, half * PT + ql + 32};
+    asm volatile("" : "+v"(tile_at[1]));
+
     // ---- filter one 32 x 32 tile held in `acc` and append what passes ---------------------------
     // lane holds 16 distances of query ql: rows 8*(r/4) + 4*half + r%4 of the tile
     const int partner_addr = (lane ^ 32) << 2; // byte address of the lane that shares this lane's query
     auto append_tile = [&](const vfloat16& acc, int tile_base) __attribute__((always_inline)) {
         // One compare per value: its lane mask stays in scalar registers and serves the count and
-        // the predicate of the write (scalar instructions cost a quarter of a vector one, and
-        // vector instructions are not overlapped with the matrix instructions of either wave).
+        // the predicate of the write (vector instructions take their cycles from the matrix
+        // instructions of both waves of the SIMD, scalar ones do not).
         u64 pass[16];
-        auto compare = [&]() -> int {
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-            {
-                pass[r] = __builtin_amdgcn_ballot_w64(acc[r] < radius);
-            }
+        auto compare = [&]() __attribute__((always_inline)) -> int {
             int count = 0;
 #pragma unroll
             for (int r = 0; r < 16; ++r)
             {
-                count += __builtin_amdgcn_inverse_ballot_w64(pass[r]) ? 1 : 0;
+                const bool below = acc[r] < radius;
+                pass[r] = __builtin_amdgcn_ballot_w64(below);
+                count += below ? 1 : 0;
             }
             return count;
         };
@@ -347,14 +349,15 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         fill += mine + other;
     };
     auto filter_tile = [&](const vfloat16& acc, int tile_base) __attribute__((always_inline)) {
-        // (written out: fminf would first quieten each operand with an instruction of its own)
-        float smallest = min3(acc[0], acc[1], acc[2]);
+        // (min3 written out: fminf would first quieten each operand with an instruction of its own)
+        float low[5];
 #pragma unroll
-        for (int r = 3; r < 15; r += 2)
+        for (int g = 0; g < 5; ++g)
         {
-            smallest = min3(smallest, acc[r], acc[r + 1]);
+            low[g] = min3(acc[3 * g], acc[3 * g + 1], acc[3 * g + 2]);
         }
-        smallest = min3(smallest, acc[15], acc[15]);
+        const float smallest = min3(min3(low[0], low[1], low[2]), min3(low[3], low[4], acc[15]),
+                                    acc[15]);
         if (__builtin_amdgcn_ballot_w64(smallest < radius) != 0)
         {
             append_tile(acc, tile_base);
@@ -450,12 +453,20 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             // (LDS instructions are overlapped with matrix instructions, vector-ALU ones are not).
             constexpr int PAIRS = MT / 2;
             float a[2][2][STEPS];
-            const float* arow = stage + half * PT + ql;
+            // The reads of one tile are 2*PT floats apart, which a two-address LDS read with
+            // offsets in units of 64 floats covers from one base register per tile; pairing the
+            // two tiles of a step instead needs an address computation per step.
+            const float* arow0 = stage + tile_at[0];
+            const float* arow1 = stage + tile_at[1];
 #pragma unroll
             for (int s = 0; s < STEPS; ++s)
             {
-                a[0][0][s] = arow[2 * s * PT];
-                a[0][1][s] = arow[2 * s * PT + 32];
+                a[0][0][s] = arow0[2 * s * PT];
+            }
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+            {
+                a[0][1][s] = arow1[2 * s * PT];
             }
             __builtin_amdgcn_sched_barrier(0); // keep the reads above the chain
             static_for<0, PAIRS>([&](auto p_tag) {
@@ -473,8 +484,26 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                     constexpr int s = decltype(s_tag)::value;
                     if constexpr (p + 1 < PAIRS)
                     {
-                        a[cur ^ 1][0][s] = arow[2 * s * PT + 64 * (p + 1)];
-                        a[cur ^ 1][1][s] = arow[2 * s * PT + 64 * (p + 1) + 32];
+                        // steps (s, s+1) of the first tile in even steps, (s-1, s) of the second
+                        // tile in odd ones
+                        constexpr int next = 64 * (p + 1);
+                        if constexpr (s % 2 == 0)
+                        {
+                            a[cur ^ 1][0][s] = arow0[2 * s * PT + next];
+                            if constexpr (s + 1 < STEPS)
+                            {
+                                a[cur ^ 1][0][s + 1] = arow0[2 * (s + 1) * PT + next];
+                            }
+                            else
+                            {
+                                a[cur ^ 1][1][s] = arow1[2 * s * PT + next];
+                            }
+                        }
+                        else
+                        {
+                            a[cur ^ 1][1][s - 1] = arow1[2 * (s - 1) * PT + next];
+                            a[cur ^ 1][1][s] = arow1[2 * s * PT + next];
+                        }
                     }
                     acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][0][s], qf[s], acc0, 0, 0, 0);
                     acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][1][s], qf[s], acc1, 0, 0, 0);
