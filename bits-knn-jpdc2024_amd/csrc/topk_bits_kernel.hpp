@@ -402,7 +402,13 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
             {
                 smallest = fminf(smallest, v[j]);
             }
-            if (__builtin_amdgcn_ballot_w64(smallest <= radius) != 0)
+            // A value equal to the radius passes only with a label below the radius key's.  With
+            // implicit labels every label of this chunk is at least that of its first column, so
+            // when that one is not below, equal values need no look (rows with few distinct
+            // values have one in every chunk).
+            const bool no_ties =
+                lrow == nullptr && static_cast<std::int32_t>(cur_chunk + label_offset) >= key_label(radius_key);
+            if (__builtin_amdgcn_ballot_w64(no_ties ? smallest < radius : smallest <= radius) != 0)
             {
                 int running = fill;
 #pragma unroll
