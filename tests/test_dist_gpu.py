@@ -185,3 +185,38 @@ def test_config_4_full_size_samples(bk, dev):
         bk.distances(queries[:, q0:q0 + 128].contiguous(), sub, bk.DIST_PARTIAL_L2, out=ref[:, :sub.shape[1]])
         torch.cuda.synchronize()
         assert torch.equal(ref[:, :sub.shape[1]], out[q0:q0 + 128, 5000:5000 + sub.shape[1]])
+
+
+def test_random_shapes_and_strides_against_the_oracle(bk, dev, oracle):
+    """40 random problems: all three operations, dimensions on both sides of every padded size,
+    padded and offset views of queries, points and the output matrix (aligned and unaligned rows,
+    which select between the pipelined kernel, the plain kernel and their store variants)."""
+    import torch
+    rng = np.random.default_rng(31)
+    dims = [1, 2, 3, 5, 8, 9, 16, 17, 31, 32, 33, 63, 64, 65, 100, 128, 129, 200, 256]
+    codes = {"l2": bk.DIST_L2, "partial": bk.DIST_PARTIAL_L2, "expanded": bk.DIST_EXPANDED}
+    for case in range(40):
+        d = int(rng.choice(dims))
+        n = int(rng.choice([rng.integers(1, 300), rng.integers(300, 9000), rng.integers(9000, 50000)]))
+        q = int(rng.choice([rng.integers(1, 140), rng.integers(128, 600), rng.integers(256, 1200)]))
+        q = max(1, min(q, int(2e9 / (n * d))))
+        op = ["l2", "partial", "expanded"][case % 3]
+        qpad, ppad, opad, off = (int(rng.choice(c)) for c in ([0, 0, 1, 3, 4], [0, 0, 1, 4, 5],
+                                                              [0, 0, 1, 4, 28, 32], [0, 0, 1, 4]))
+        p, s = oracle.generate(700 + case, n, q, d)
+        pd = torch.zeros((d, n + ppad + off), device=dev)
+        qd = torch.zeros((d, q + qpad + off), device=dev)
+        pd[:, off:off + n] = torch.from_numpy(np.ascontiguousarray(p.T)).to(dev)
+        qd[:, off:off + q] = torch.from_numpy(np.ascontiguousarray(s.T)).to(dev)
+        out = torch.full((q, n + opad + off), -7.0, device=dev)
+        bk.distances(qd[:, off:off + q], pd[:, off:off + n], codes[op], out=out[:, off:off + n])
+        torch.cuda.synchronize()
+        what = (case, n, q, d, op, qpad, ppad, opad, off)
+        got = out[:, off:off + n].cpu().numpy()
+        assert (out[:, :off] == -7).all() and (out[:, off + n:] == -7).all(), what
+        if op == "l2":
+            assert np.array_equal(got.view(np.uint32), oracle.dist(s, p, "l2").view(np.uint32)), what
+        else:
+            exp = oracle.dist(s, p, "partial")
+            scale = (p.astype(np.float64) ** 2).sum(1)[None, :] * 2 + (s.astype(np.float64) ** 2).sum(1)[:, None]
+            assert np.max(np.abs(got - exp) / np.maximum(scale, 1e-30)) < 1e-5, what

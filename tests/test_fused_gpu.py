@@ -222,3 +222,30 @@ def test_long_lists_with_a_workspace_take_two_passes(bk, dev, oracle, k):
     assert small.numel() < q * n * 4
     sd, sl = _fused(bk, dev, points, queries, k, workspace=small)
     _check(oracle, points, queries, k, sd, sl)
+
+
+def test_random_shapes_against_the_oracle(bk, dev, oracle):
+    """40 random problems over dimensions on both sides of every padded size, all list lengths,
+    ragged point and query counts, with the plain entry point, the workspace the library asks for
+    and a workspace that only holds partial lists."""
+    import torch
+    rng = np.random.default_rng(77)
+    dims = [1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 24, 31, 32, 33, 40, 63, 64, 65, 100, 128, 129, 200, 256]
+    for case in range(40):
+        d = int(rng.choice(dims))
+        k = int(rng.choice([4, 8, 16, 32, 64, 128, 256]))
+        n = int(rng.choice([rng.integers(1, 300), rng.integers(300, 5000), rng.integers(5000, 30000)]))
+        q = int(rng.choice([rng.integers(1, 40), rng.integers(40, 300), rng.integers(300, 600)]))
+        q = max(1, min(q, int(1.5e9 / (n * d))))
+        kind = case % 3
+        workspace = None
+        if kind == 1:
+            workspace = "auto"
+        elif kind == 2:
+            workspace = torch.empty(max(8, 8 * q * 64 * k), dtype=torch.uint8, device=dev)
+        p, s = oracle.generate(3000 + case, n, q, d)
+        gd, gl = _fused(bk, dev, p, s, k, (2, 4, 1), 1, 1, workspace=workspace)
+        try:
+            _check(oracle, p, s, k, gd, gl)
+        except AssertionError as e:
+            raise AssertionError((case, n, q, d, k, kind)) from e
