@@ -99,7 +99,7 @@ struct fused_geometry
         // two stages (one being multiplied, one being filled), the query buffers, exchange slots
         return 2 * static_cast<size_t>(ROWS) * PT * sizeof(float) +
                static_cast<size_t>(FQ_WAVES) * FQ_QW * FQ_CAP * sizeof(u64) +
-               static_cast<size_t>(FQ_WAVES) * WAVE * sizeof(float);
+               static_cast<size_t>(FQ_WAVES) * WAVE * sizeof(float) + 4 * sizeof(int);
     }
 };
 
@@ -127,6 +127,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     float* const stages = lds;                                                    // [2][ROWS][PT]
     u64* const buffers = reinterpret_cast<u64*>(lds + 2 * STAGE_FLOATS);          // [waves][32][CAP]
     float* const xchg = reinterpret_cast<float*>(buffers + FQ_WAVES * FQ_QW * FQ_CAP);  // [waves][64]
+    int* const merge_wanted = reinterpret_cast<int*>(xchg + FQ_WAVES * WAVE);           // [3]
 
     const int dim = a.dim;
     // this workgroup's range of points
@@ -163,11 +164,17 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     {
         lds[i] = 0.0F;
     }
+    if (t < 3)
+    {
+        merge_wanted[t] = 0;
+    }
     __syncthreads();
 
     float radius = __builtin_inff(); // k-th smallest distance of my query so far
     int fill = 0;                    // used slots of my query's buffer (same in both lanes of a query)
     bool have_list = false;          // wave-uniform: the lists in the output arrays are valid
+    bool merged = false;             // wave-uniform: this wave has merged during the current stage
+    int stage_slot = 0;              // stage index modulo 3: the slot of merge_wanted in use
 
     // ---- merge of all buffers of this wave into the lists --------------------------------------
     auto merge_event = [&]() __attribute__((always_inline)) {
@@ -298,6 +305,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         radius = wx[ql];
         fill = 0;
         have_list = true;
+        merged = true;
     };
 
     // position of this lane's A operands inside a stage row, for the two tiles of a pair (the
@@ -328,6 +336,12 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         int other = __builtin_amdgcn_ds_bpermute(partner_addr, mine);
         if (__builtin_amdgcn_ballot_w64(fill + mine + other > FQ_CAP) != 0)
         {
+            // the other waves of the workgroup would wait for this wave at the stage barrier:
+            // they are asked to merge their buffers in the meantime
+            if (lane == 0)
+            {
+                __hip_atomic_store(merge_wanted + stage_slot, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
             merge_event();
             mine = compare();
             other = __builtin_amdgcn_ds_bpermute(partner_addr, mine);
@@ -534,7 +548,17 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     // Stage s is multiplied while stage s+1 sits in registers and is written to the other LDS
     // buffer afterwards; stage s+2 is requested from memory right after that.  One barrier per
     // stage: it separates the last read of a buffer from its next fill and the fill from its
-    // first read.
+    // first read.  A wave that had to merge in stage s raises merge_wanted[s % 3]; the others look
+    // at it before and after the barrier of that stage (the flag for stage s + 2 is cleared after the
+    // barrier of stage s: its last readers passed it before that barrier, its next writers come
+    // after the following one).
+    auto merge_if_wanted = [&]() __attribute__((always_inline)) {
+        if (!merged && __hip_atomic_load(merge_wanted + stage_slot, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_WORKGROUP) != 0)
+        {
+            merge_event();
+        }
+    };
     fetch(n_begin);
     // the query fragment and the first stage have arrived (nothing else is in flight yet)
     __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -547,6 +571,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     int parity = 0;
     for (int base = n_begin; base < n; base += PT)
     {
+        merged = false;
         multiply(stages + parity * STAGE_FLOATS, base);
         parity ^= 1;
         if (base + PT < n)
@@ -557,7 +582,14 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 fetch(base + 2 * PT);
             }
         }
+        merge_if_wanted();
         __syncthreads();
+        merge_if_wanted();
+        if (t == 0)
+        {
+            merge_wanted[(stage_slot + 2) % 3] = 0;
+        }
+        stage_slot = stage_slot == 2 ? 0 : stage_slot + 1;
     }
 
     // whatever is left in the buffers; also writes the lists of queries that never merged
