@@ -116,8 +116,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     constexpr int MT = G::MT;
     // merge layout: S keys per query spread over LPQ lanes, R keys per lane
     constexpr int S = K > FQ_CAP ? K : FQ_CAP;
-    // (16 lanes per query for long lists: fewer, wider passes hide the latency of the list traffic)
-    constexpr int R = S <= 64 ? 4 : 8;
+    constexpr int R = 4;
     constexpr int LPQ = S / R;
     constexpr int QPP = WAVE / LPQ;           // queries per merge pass
     constexpr int PASSES = FQ_QW / QPP;
@@ -233,13 +232,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 }
             }
         };
-        // (with 8 keys per lane the registers for a request in flight would cost a workgroup per
-        // compute unit)
-        constexpr bool AHEAD = R <= 4;
-        if constexpr (AHEAD)
-        {
-            request_list(0);
-        }
+        request_list(0);
 #pragma unroll 1
         for (int pass = 0; pass < PASSES; ++pass)
         {
@@ -248,10 +241,6 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             const int used = reinterpret_cast<const int*>(wx)[32 + qm];
             u64 buf[R];
             u64 list[R];
-            if constexpr (!AHEAD)
-            {
-                request_list(pass);
-            }
 #pragma unroll
             for (int r = 0; r < R; ++r)
             {
@@ -268,7 +257,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 }
                 list[r] = make_key(next_dist[r], next_label[r]);
             }
-            if (AHEAD && pass + 1 < PASSES)
+            if (pass + 1 < PASSES)
             {
                 request_list(pass + 1);
             }
