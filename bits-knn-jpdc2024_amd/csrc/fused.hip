@@ -9,7 +9,7 @@
 //
 //  * A workgroup of 4 waves owns 128 queries (32 per wave) and walks over its range of points in
 //    stages of PT points, two stages in LDS (one being multiplied, one being filled; one barrier
-//    per stage).  A stage is the MFMA A operand: rows 0..d-1 hold -2*p, the following rows hold
+//    per stage).  A stage is the MFMA A operand: rows 0..d-1 hold the points, the following rows hold
 //    the staging threads' shares of ||p||^2, so that v_mfma_f32_32x32x2_f32 against the query
 //    fragment (-2q_0..-2q_{d-1}, 1, 1) yields ||p||^2 - 2 q.p directly, the dot product accumulated
 //    first and the norm added last.
@@ -18,11 +18,14 @@
 //    registers and one compare against that query's radius.
 //  * Every query has a 32-slot buffer in LDS.  Slots are handed out without atomics: the two
 //    lanes that share a query exchange their pass counts, and the fill is kept in a register.
-//    Before a tile would overflow any buffer of the wave, the wave merges all its buffers.
-//  * The sorted top-k lists live in the output arrays themselves between merges (they are read
-//    and rewritten through L2 a few hundred times per query while 2^20 distances are computed).
-//    A merge sorts the buffers of 8 (4, 2, 1 for larger k) queries at a time with a segmented
-//    bitonic network in registers, 4 keys per lane.
+//    Before a tile would overflow any buffer of the wave, the wave merges all its buffers; the
+//    other waves of the workgroup, which would wait for it at the stage barrier, then merge
+//    theirs in the same stage.
+//  * The sorted top-k lists live in the output arrays themselves between merges, read back by the
+//    lanes that wrote them (plain loads and stores, requested one pass ahead).  A merge is a
+//    segmented bitonic network in registers, 4 keys per lane: 8 queries per pass for k <= 32;
+//    for longer lists the buffers are sorted in place first (8 queries per pass) and then merged
+//    into the lists of 4, 2 or 1 queries per pass.
 //  * With few queries the points are cut into ranges (blockIdx.y) whose partial lists go to a
 //    caller-provided workspace and are reduced by one bits top-k pass with explicit labels.
 //
