@@ -9,10 +9,10 @@
 //
 //  * A workgroup of 4 waves owns 128 queries (32 per wave) and walks over its range of points in
 //    stages of PT points, two stages in LDS (one being multiplied, one being filled; one barrier
-//    per stage).  A stage is the MFMA A operand: rows 0..d-1 hold the points, the following rows hold
-//    the staging threads' shares of ||p||^2, so that v_mfma_f32_32x32x2_f32 against the query
+//    per stage).  A stage is the MFMA A operand: rows 0..d-1 hold the points, the following rows
+//    hold the staging threads' shares of ||p||^2, so that v_mfma_f32_32x32x2_f32 against the query
 //    fragment (-2q_0..-2q_{d-1}, 1, 1) yields ||p||^2 - 2 q.p directly, the dot product accumulated
-//    first and the norm added last.
+//    first and the norm added last.  For d <= 16 the norm is the initial accumulator instead.
 //  * The query fragment stays in registers for the whole kernel.  In the 32 x 32 result tile a
 //    lane holds 16 distances of ONE query (column), so the filter is a min-tree over 16
 //    registers and one compare against that query's radius.
@@ -55,6 +55,7 @@ __device__ __forceinline__ void static_for(F&& f)
 
 
 typedef float vfloat16 __attribute__((ext_vector_type(16)));
+typedef float vfloat4 __attribute__((ext_vector_type(4)));
 
 // minimum of three values in one instruction; a NaN operand is ignored
 __device__ __forceinline__ float min3(float a, float b, float c)
@@ -113,7 +114,13 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 {
     using G = fused_geometry<DP>;
     constexpr int PT = G::PT;
-    constexpr int STEPS = G::STEPS;
+    // Norms in the accumulator: where one staging thread carries a whole point (DP <= 16) its
+    // ||p||^2 is one row after the point rows and is read as the initial value of the
+    // accumulators, which saves the matrix step that would add it (one of 5 at DP = 8, one of 9 at
+    // DP = 16; at DP = 32 the 32 registers it takes cost as much as the 17th step).  The sum then
+    // starts from the norm instead of ending with it: same terms, another rounding order.
+    constexpr bool NORM_IN_C = G::TPP == 1 && G::MT >= 2;
+    constexpr int STEPS = NORM_IN_C ? DP / 2 : G::STEPS;
     constexpr int TPP = G::TPP;
     constexpr int VPT = G::VPT;
     constexpr int MT = G::MT;
@@ -446,6 +453,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             stage[dd * PT + sp] = pre[i];
         }
         // points beyond the end get an infinite distance and never pass the filter
+        // (with one staging thread per point the share is the norm, in row DP)
         stage[(DP + sd0) * PT + sp] = base + sp < n ? share : __builtin_inff();
     };
 
@@ -474,18 +482,43 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             {
                 a[0][1][s] = arow1[2 * s * PT];
             }
+            // initial accumulators of a pair: zero, or the norms of the lane's 16 points
+            vfloat16 init0;
+            vfloat16 init1;
+            auto request_init = [&](int pair) __attribute__((always_inline)) {
+                if constexpr (NORM_IN_C)
+                {
+                    const float* norms = stage + DP * PT + pair * 64 + 4 * half;
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                    {
+                        const vfloat4 x = *reinterpret_cast<const vfloat4*>(norms + 8 * g);
+                        const vfloat4 y = *reinterpret_cast<const vfloat4*>(norms + 32 + 8 * g);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                        {
+                            init0[4 * g + e] = x[e];
+                            init1[4 * g + e] = y[e];
+                        }
+                    }
+                }
+                else
+                {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                    {
+                        init0[r] = 0.0F;
+                        init1[r] = 0.0F;
+                    }
+                }
+            };
+            request_init(0);
             __builtin_amdgcn_sched_barrier(0); // keep the reads above the chain
             static_for<0, PAIRS>([&](auto p_tag) {
                 constexpr int p = decltype(p_tag)::value;
                 constexpr int cur = p & 1;
-                vfloat16 acc0;
-                vfloat16 acc1;
-#pragma unroll
-                for (int r = 0; r < 16; ++r)
-                {
-                    acc0[r] = 0.0F;
-                    acc1[r] = 0.0F;
-                }
+                vfloat16 acc0 = init0;
+                vfloat16 acc1 = init1;
                 static_for<0, STEPS>([&](auto s_tag) {
                     constexpr int s = decltype(s_tag)::value;
                     if constexpr (p + 1 < PAIRS)
@@ -513,6 +546,10 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                     }
                     acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][0][s], qf[s], acc0, 0, 0, 0);
                     acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][1][s], qf[s], acc1, 0, 0, 0);
+                    if constexpr (NORM_IN_C && s == 0 && p + 1 < PAIRS)
+                    {
+                        request_init(p + 1); // the first step has taken this pair's
+                    }
                     __builtin_amdgcn_sched_barrier(0);
                 });
                 filter_tile(acc0, base + p * 64);

@@ -49,6 +49,14 @@ def _check(oracle, points, queries, k, gd, gl, min_recall=0.999):
     scale_k = np.abs(ed[:, kk - 1]) + qn[:, 0]
     assert np.max(np.abs(gd[:, kk - 1] - ed[:, kk - 1]) / scale_k) <= REL
     recall = np.mean([len(set(a[:kk]) & set(b[:kk])) / kk for a, b in zip(gl, el)])
+    if recall < min_recall:
+        # Neighbours closer together than fp32 resolves (many points on a line, say): which of
+        # them a correct kernel reports depends on its rounding order.  A reported label then
+        # counts when its exact distance lies within the tolerance of the exact k-th distance.
+        truth = oracle.dist(queries, points, "f64-partial")
+        kth = np.sort(truth, axis=1)[:, kk - 1]
+        at = np.take_along_axis(truth, gl[:, :kk].astype(np.int64), axis=1)
+        recall = np.mean(at <= (kth + REL * (np.abs(kth) + qn[:, 0]))[:, None])
     assert recall >= min_recall, recall
     # where the oracle's neighbour gaps are far above the rounding noise the sets must be identical
     if n > kk:
