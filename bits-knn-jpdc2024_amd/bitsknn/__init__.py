@@ -27,6 +27,8 @@ EXPORTS = (
     "bitsknn_fused_l2_topk_f32",
     "bitsknn_fused_workspace_bytes",
     "bitsknn_fused_l2_topk_f32_ws",
+    "bitsknn_fused_set_arithmetic",
+    "bitsknn_fused_get_arithmetic",
 )
 
 
@@ -72,6 +74,10 @@ def lib():
         L.bitsknn_fused_l2_topk_f32.argtypes = [vp, vp, ctypes.c_int, i32, i32, vp, vp, ctypes.c_int,
                                                 ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                 ctypes.c_int, ctypes.c_int, vp]
+        L.bitsknn_fused_set_arithmetic.restype = ctypes.c_int
+        L.bitsknn_fused_set_arithmetic.argtypes = [ctypes.c_int]
+        L.bitsknn_fused_get_arithmetic.restype = ctypes.c_int
+        L.bitsknn_fused_get_arithmetic.argtypes = []
         L.bitsknn_fused_workspace_bytes.restype = ctypes.c_size_t
         L.bitsknn_fused_workspace_bytes.argtypes = [i32, i32, ctypes.c_int]
         L.bitsknn_fused_l2_topk_f32_ws.restype = ctypes.c_int
@@ -200,6 +206,18 @@ def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1,
                                               params[1], params[2], block_query_dim, dim_mult,
                                               _ptr(workspace), workspace.numel(), _stream()))
     return out_dist, out_label
+
+
+FUSED_FP32, FUSED_BF16X3 = 0, 1
+
+
+def fused_set_arithmetic(arithmetic):
+    """Arithmetic of the products in the fused kernels for dim <= 32 (process-wide)."""
+    _check(lib().bitsknn_fused_set_arithmetic(int(arithmetic)))
+
+
+def fused_get_arithmetic():
+    return int(lib().bitsknn_fused_get_arithmetic())
 
 
 def fused_workspace_bytes(q, n, k):

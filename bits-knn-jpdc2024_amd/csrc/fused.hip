@@ -32,6 +32,7 @@
 // Equal distances are ordered by lower point index: points are visited in index order, so a
 // value equal to a query's radius can never displace what is already merged.
 
+#include <atomic>
 #include <type_traits>
 
 #include "bitonic_net.hpp"
@@ -56,6 +57,8 @@ __device__ __forceinline__ void static_for(F&& f)
 
 typedef float vfloat16 __attribute__((ext_vector_type(16)));
 typedef float vfloat4 __attribute__((ext_vector_type(4)));
+typedef u32 vuint4 __attribute__((ext_vector_type(4)));
+typedef __bf16 vbf16x8 __attribute__((ext_vector_type(8)));
 
 // minimum of three values in one instruction; a NaN operand is ignored
 __device__ __forceinline__ float min3(float a, float b, float c)
@@ -63,6 +66,32 @@ __device__ __forceinline__ float min3(float a, float b, float c)
     float r;
     asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
     return r;
+}
+
+// x[i] = x1 + x2 + x3 exactly, each piece with at most 8 significant bits (a bf16): the upper
+// halves of x, of x - x1 and of x - x1 - x2.  Piece c of values 2j and 2j+1 shares word j of pc.
+__device__ __forceinline__ void split_bf16x3(const float (&x)[8], vuint4& p1, vuint4& p2, vuint4& p3)
+{
+    u32 b1[8];
+    u32 b2[8];
+    u32 b3[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+    {
+        b1[i] = __builtin_bit_cast(u32, x[i]);
+        const float r = x[i] - __builtin_bit_cast(float, b1[i] & 0xFFFF0000U);
+        b2[i] = __builtin_bit_cast(u32, r);
+        const float l = r - __builtin_bit_cast(float, b2[i] & 0xFFFF0000U);
+        b3[i] = __builtin_bit_cast(u32, l);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        // bytes 3:2 of the odd value above bytes 3:2 of the even one
+        p1[j] = __builtin_amdgcn_perm(b1[2 * j + 1], b1[2 * j], 0x07060302U);
+        p2[j] = __builtin_amdgcn_perm(b2[2 * j + 1], b2[2 * j], 0x07060302U);
+        p3[j] = __builtin_amdgcn_perm(b3[2 * j + 1], b3[2 * j], 0x07060302U);
+    }
 }
 
 constexpr int FQ_WAVES = 4;                   // waves per workgroup
@@ -84,24 +113,40 @@ struct fused_args
     int split_points;     // points per range (a multiple of 256)
 };
 
-// stage geometry by padded dimension DP: PT points per stage, so that the stage
-// ((DP + 2) x PT floats) stays below 20 KB for DP <= 128
-template <int DP>
+// Stage geometry by padded dimension DP.
+//
+// SPLIT = false: fp32 matrix instructions; a stage is (DP + norm rows) x PT floats, PT points per
+// stage so that it stays below 20 KB for DP <= 128.
+//
+// SPLIT = true (DP <= 32): every fp32 value x is cut into three bf16 pieces x = x1 + x2 + x3
+// (exactly: 8 + 8 + 8 significant bits) and a product x*y is the sum of the bf16 products
+// x3*y1 + x2*y2 + x1*y3 + x2*y1 + x1*y2 + x1*y1 accumulated in fp32 (what is left out is below
+// 2^-23 of the product, the size of one fp32 rounding).  The bf16 matrix path runs at 16 times
+// the fp32 one and does not share the vector unit with it.  A stage holds, per piece and per 8
+// dimensions, one 16-byte cell per point (the A operand of v_mfma_f32_32x32x16_bf16), then the
+// norms of the points.
+template <int DP, bool SPLIT>
 struct fused_geometry
 {
-    static constexpr int PT = DP <= 16 ? 256 : (DP <= 32 ? 128 : (DP <= 64 ? 64 : 32));
+    static constexpr int DK = DP < 16 ? 16 : DP;       // SPLIT: dimensions padded to whole matrix steps
+    static constexpr int KB = DK / 16;                 // SPLIT: matrix steps of 16 dimensions
+    static constexpr int KS = DK / 8;                  // SPLIT: cells of 8 dimensions per point and piece
+    static constexpr int PT = SPLIT ? (DK <= 16 ? 128 : 64)
+                                    : (DP <= 16 ? 256 : (DP <= 32 ? 128 : (DP <= 64 ? 64 : 32)));
     static constexpr int TPP = FQ_THREADS / PT; // threads per point when staging
     // point rows (zero beyond dim), then one row per staging thread of a point with its share of
     // ||p||^2 (at least two rows, so that the row count is even)
     static constexpr int NORM_ROWS = TPP > 2 ? TPP : 2;
     static constexpr int ROWS = DP + NORM_ROWS;
     static constexpr int STEPS = ROWS / 2;    // MFMA steps of 2 rows
-    static constexpr int VPT = DP / TPP;      // values a thread carries from global memory to LDS
+    static constexpr int VPT = SPLIT ? 8 : DP / TPP; // values a thread carries from global memory to LDS
     static constexpr int MT = PT / 32;        // MFMA row tiles per stage
+    static constexpr int STAGE_FLOATS = SPLIT ? 3 * KS * PT * 4 + PT : ROWS * PT;
+    static_assert(!SPLIT || (DP <= 32 && TPP == KS), "one staging thread per point and cell");
     static constexpr size_t lds_bytes()
     {
         // two stages (one being multiplied, one being filled), the query buffers, exchange slots
-        return 2 * static_cast<size_t>(ROWS) * PT * sizeof(float) +
+        return 2 * static_cast<size_t>(STAGE_FLOATS) * sizeof(float) +
                static_cast<size_t>(FQ_WAVES) * FQ_QW * FQ_CAP * sizeof(u64) +
                static_cast<size_t>(FQ_WAVES) * WAVE * sizeof(float) + 4 * sizeof(int);
     }
@@ -109,18 +154,20 @@ struct fused_geometry
 
 // K: list length.  DP: dimension padded to 8, 16, 32, 64, 128 or 256 (padding rows are zero on
 // both sides of the product).
-template <int K, int DP>
+template <int K, int DP, bool SPLIT>
 __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 {
-    using G = fused_geometry<DP>;
+    using G = fused_geometry<DP, SPLIT>;
     constexpr int PT = G::PT;
     // Norms in the accumulator: where one staging thread carries a whole point (DP <= 16) its
     // ||p||^2 is one row after the point rows and is read as the initial value of the
     // accumulators, which saves the matrix step that would add it (one of 5 at DP = 8, one of 9 at
     // DP = 16; at DP = 32 the 32 registers it takes cost as much as the 17th step).  The sum then
     // starts from the norm instead of ending with it: same terms, another rounding order.
-    constexpr bool NORM_IN_C = G::TPP == 1 && G::MT >= 2;
+    constexpr bool NORM_IN_C = SPLIT || (G::TPP == 1 && G::MT >= 2);
     constexpr int STEPS = NORM_IN_C ? DP / 2 : G::STEPS;
+    constexpr int KB = G::KB;
+    constexpr int KS = G::KS;
     constexpr int TPP = G::TPP;
     constexpr int VPT = G::VPT;
     constexpr int MT = G::MT;
@@ -132,8 +179,8 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     constexpr int PASSES = FQ_QW / QPP;
 
     extern __shared__ float lds[];
-    constexpr int STAGE_FLOATS = G::ROWS * PT;
-    float* const stages = lds;                                                    // [2][ROWS][PT]
+    constexpr int STAGE_FLOATS = G::STAGE_FLOATS;
+    float* const stages = lds;                                                    // [2][STAGE_FLOATS]
     u64* const buffers = reinterpret_cast<u64*>(lds + 2 * STAGE_FLOATS);          // [waves][32][CAP]
     float* const xchg = reinterpret_cast<float*>(buffers + FQ_WAVES * FQ_QW * FQ_CAP);  // [waves][64]
     int* const merge_wanted = reinterpret_cast<int*>(xchg + FQ_WAVES * WAVE);           // [3]
@@ -155,17 +202,43 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 
     // query fragment: step s of this lane is row 2s + half, times -2 (the stages hold the plain
     // point values); the norm rows are multiplied by 1
-    float qf[STEPS];
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s)
+    float qf[SPLIT ? 1 : STEPS];
+    // SPLIT: the three bf16 pieces of -2q for the 8 dimensions 16*kb + 8*half .. + 7 of step kb
+    vuint4 qs[SPLIT ? 3 : 1][SPLIT ? KB : 1];
+    if constexpr (SPLIT)
     {
-        const int dd = 2 * s + half;
-        float val = dd >= DP ? 1.0F : 0.0F;
-        if (dd < dim && my_q < a.q)
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
         {
-            val = -2.0F * a.queries[static_cast<size_t>(dd) * a.q + my_q];
+            float val[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+            {
+                const int dd = 16 * kb + 8 * half + j;
+                val[j] = 0.0F;
+                if (dd < dim && my_q < a.q)
+                {
+                    val[j] = -2.0F * a.queries[static_cast<size_t>(dd) * a.q + my_q];
+                }
+            }
+            split_bf16x3(val, qs[0][kb], qs[1][kb], qs[2][kb]);
         }
-        qf[s] = val;
+        qf[0] = 0.0F;
+    }
+    else
+    {
+        qs[0][0] = vuint4{0, 0, 0, 0};
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s)
+        {
+            const int dd = 2 * s + half;
+            float val = dd >= DP ? 1.0F : 0.0F;
+            if (dd < dim && my_q < a.q)
+            {
+                val = -2.0F * a.queries[static_cast<size_t>(dd) * a.q + my_q];
+            }
+            qf[s] = val;
+        }
     }
 
     // rows that never change in either stage: padding dimensions, unused norm rows
@@ -362,16 +435,20 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         fill += mine + other;
     };
     auto filter_tile = [&](const vfloat16& acc, int tile_base) __attribute__((always_inline)) {
-        // (min3 written out: fminf would first quieten each operand with an instruction of its own)
+        // The first read of the tile is a compare the compiler sees, so that it places the wait
+        // states a matrix result needs before them; the minimum of the other 15 values is written
+        // out as v_min3 (fminf would first quieten each operand with an instruction of its own),
+        // and assembly operands are not covered by that hazard handling.
+        const u64 last_passes = __builtin_amdgcn_ballot_w64(acc[15] < radius);
+        __builtin_amdgcn_sched_barrier(0);
         float low[5];
 #pragma unroll
         for (int g = 0; g < 5; ++g)
         {
             low[g] = min3(acc[3 * g], acc[3 * g + 1], acc[3 * g + 2]);
         }
-        const float smallest = min3(min3(low[0], low[1], low[2]), min3(low[3], low[4], acc[15]),
-                                    acc[15]);
-        if (__builtin_amdgcn_ballot_w64(smallest < radius) != 0)
+        const float smallest = min3(min3(low[0], low[1], low[2]), low[3], low[4]);
+        if ((last_passes | __builtin_amdgcn_ballot_w64(smallest < radius)) != 0)
         {
             append_tile(acc, tile_base);
         }
@@ -380,8 +457,11 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     // ---- staging: global -> registers -> LDS ---------------------------------------------------
     // thread t carries dimensions (t / PT) + TPP*i of point t % PT, writes them as rows of the
     // stage and adds up its share of ||p||^2 (the shares of a point meet inside the MFMA)
-    const int sp = t % PT;
-    const int sd0 = t / PT;
+    // SPLIT: thread t carries the 8 dimensions 8*(t % TPP) .. + 7 of point t / TPP (the threads of
+    // a point are neighbouring lanes, which add up their shares of the norm among themselves)
+    const int sp = SPLIT ? t / TPP : t % PT;
+    const int sd0 = SPLIT ? 8 * (t % TPP) : t / PT;
+    auto dim_of = [&](int i) -> int { return SPLIT ? sd0 + i : sd0 + TPP * i; };
     float pre[VPT];
     // Point values are read with buffer loads: a constant byte offset per value and lane (beyond
     // the resource for dimensions dim .. DP-1, which then read as zero; the hardware checks the
@@ -396,7 +476,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 #pragma unroll
     for (int i = 0; i < VPT; ++i)
     {
-        const int dd = sd0 + TPP * i;
+        const int dd = dim_of(i);
         load_off[i] = dd < dim && small_points
                           ? static_cast<int>((static_cast<size_t>(dd) * total_points + sp) * sizeof(float))
                           : OUTSIDE;
@@ -433,7 +513,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 #pragma unroll
             for (int i = 0; i < VPT; ++i)
             {
-                const int dd = sd0 + TPP * i;
+                const int dd = dim_of(i);
                 pre[i] = 0.0F;
                 if (dd < dim && j < n)
                 {
@@ -444,22 +524,107 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     };
     auto deposit = [&](float* stage, int base) {
         float share = 0.0F;
-#pragma unroll
-        for (int i = 0; i < VPT; ++i)
+        if constexpr (SPLIT)
         {
-            const int dd = sd0 + TPP * i;
-            share = __builtin_fmaf(pre[i], pre[i], share);
-            // (dimensions from dim on were read as zero: their rows stay zero)
-            stage[dd * PT + sp] = pre[i];
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+            {
+                share = __builtin_fmaf(pre[i], pre[i], share);
+            }
+            vuint4 piece[3];
+            split_bf16x3(pre, piece[0], piece[1], piece[2]);
+            vuint4* const cells = reinterpret_cast<vuint4*>(stage);
+            const int ks = sd0 / 8;
+#pragma unroll
+            for (int c = 0; c < 3; ++c)
+            {
+                cells[(c * KS + ks) * PT + sp] = piece[c];
+            }
+            // the threads of a point are TPP neighbouring lanes
+            share += __builtin_bit_cast(float, lane_xor32<1>(__builtin_bit_cast(u32, share)));
+            if constexpr (TPP == 4)
+            {
+                share += __builtin_bit_cast(float, lane_xor32<2>(__builtin_bit_cast(u32, share)));
+            }
+            // points beyond the end get an infinite distance and never pass the filter
+            stage[3 * KS * PT * 4 + sp] = base + sp < n ? share : __builtin_inff();
         }
-        // points beyond the end get an infinite distance and never pass the filter
-        // (with one staging thread per point the share is the norm, in row DP)
-        stage[(DP + sd0) * PT + sp] = base + sp < n ? share : __builtin_inff();
+        else
+        {
+#pragma unroll
+            for (int i = 0; i < VPT; ++i)
+            {
+                const int dd = sd0 + TPP * i;
+                share = __builtin_fmaf(pre[i], pre[i], share);
+                // (dimensions from dim on were read as zero: their rows stay zero)
+                stage[dd * PT + sp] = pre[i];
+            }
+            // points beyond the end get an infinite distance and never pass the filter
+            // (with one staging thread per point the share is the norm, in row DP)
+            stage[(DP + sd0) * PT + sp] = base + sp < n ? share : __builtin_inff();
+        }
     };
 
     // all row tiles of a stage: distances, filter, append
     auto multiply = [&](const float* stage, int base) {
-        if constexpr (MT >= 2)
+        if constexpr (SPLIT)
+        {
+            constexpr int PAIRS = MT / 2;
+            const vuint4* const cells = reinterpret_cast<const vuint4*>(stage);
+            const float* const norm_row = stage + 3 * KS * PT * 4;
+            static_for<0, PAIRS>([&](auto p_tag) {
+                constexpr int p = decltype(p_tag)::value;
+                // A operands of the two tiles: piece c of dimensions 16*kb + 8*half .. + 7
+                vuint4 af[2][3][KB];
+#pragma unroll
+                for (int tile = 0; tile < 2; ++tile)
+                {
+#pragma unroll
+                    for (int c = 0; c < 3; ++c)
+                    {
+#pragma unroll
+                        for (int kb = 0; kb < KB; ++kb)
+                        {
+                            af[tile][c][kb] = cells[(c * KS + 2 * kb + half) * PT + p * 64 + tile * 32 + ql];
+                        }
+                    }
+                }
+                // the accumulators start from the norms of the lane's 16 points
+                vfloat16 acc0;
+                vfloat16 acc1;
+                const float* norms = norm_row + p * 64 + 4 * half;
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                {
+                    const vfloat4 x = *reinterpret_cast<const vfloat4*>(norms + 8 * g);
+                    const vfloat4 y = *reinterpret_cast<const vfloat4*>(norms + 32 + 8 * g);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                    {
+                        acc0[4 * g + e] = x[e];
+                        acc1[4 * g + e] = y[e];
+                    }
+                }
+                // the six products of a step, smallest terms first
+                constexpr int order[6][2] = {{2, 0}, {1, 1}, {0, 2}, {1, 0}, {0, 1}, {0, 0}};
+                static_for<0, KB>([&](auto kb_tag) {
+                    constexpr int kb = decltype(kb_tag)::value;
+                    static_for<0, 6>([&](auto o_tag) {
+                        constexpr int ca = order[decltype(o_tag)::value][0];
+                        constexpr int cb = order[decltype(o_tag)::value][1];
+                        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(vbf16x8, af[0][ca][kb]), __builtin_bit_cast(vbf16x8, qs[cb][kb]),
+                            acc0, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(vbf16x8, af[1][ca][kb]), __builtin_bit_cast(vbf16x8, qs[cb][kb]),
+                            acc1, 0, 0, 0);
+                    });
+                });
+                filter_tile(acc0, base + p * 64);
+                filter_tile(acc1, base + p * 64 + 32);
+            });
+        }
+        else if constexpr (MT >= 2)
         {
             // Two row tiles at a time: two independent accumulator chains keep the matrix core
             // issuing back to back.  The A operands of a pair sit in registers before its first
@@ -625,14 +790,14 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     merge_event();
 }
 
-template <int K, int DP>
+template <int K, int DP, bool SPLIT>
 hipError_t launch_fused(const fused_args& a, hipStream_t stream)
 {
-    constexpr size_t lds_bytes = fused_geometry<DP>::lds_bytes();
+    constexpr size_t lds_bytes = fused_geometry<DP, SPLIT>::lds_bytes();
     if (lds_bytes > 48 * 1024)
     {
         const hipError_t status =
-            hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<K, DP>),
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<K, DP, SPLIT>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
         if (status != hipSuccess)
         {
@@ -640,35 +805,42 @@ hipError_t launch_fused(const fused_args& a, hipStream_t stream)
         }
     }
     const unsigned grid = static_cast<unsigned>((a.q + FQ_QB - 1) / FQ_QB);
-    hipLaunchKernelGGL((fused_kernel<K, DP>), dim3(grid, static_cast<unsigned>(a.splits)),
+    hipLaunchKernelGGL((fused_kernel<K, DP, SPLIT>), dim3(grid, static_cast<unsigned>(a.splits)),
                        dim3(FQ_THREADS), lds_bytes, stream, a);
     return hipGetLastError();
 }
 
+// arithmetic of the products for d <= 32 (bitsknn_fused_set_arithmetic)
+std::atomic<int> g_arithmetic{BITSKNN_FUSED_FP32};
+
 template <int K>
 hipError_t launch_fused_k(const fused_args& a, hipStream_t stream)
 {
+    if (a.dim <= 32 && g_arithmetic.load(std::memory_order_relaxed) == BITSKNN_FUSED_BF16X3)
+    {
+        return a.dim <= 16 ? launch_fused<K, 16, true>(a, stream) : launch_fused<K, 32, true>(a, stream);
+    }
     if (a.dim <= 8)
     {
-        return launch_fused<K, 8>(a, stream);
+        return launch_fused<K, 8, false>(a, stream);
     }
     if (a.dim <= 16)
     {
-        return launch_fused<K, 16>(a, stream);
+        return launch_fused<K, 16, false>(a, stream);
     }
     if (a.dim <= 32)
     {
-        return launch_fused<K, 32>(a, stream);
+        return launch_fused<K, 32, false>(a, stream);
     }
     if (a.dim <= 64)
     {
-        return launch_fused<K, 64>(a, stream);
+        return launch_fused<K, 64, false>(a, stream);
     }
     if (a.dim <= 128)
     {
-        return launch_fused<K, 128>(a, stream);
+        return launch_fused<K, 128, false>(a, stream);
     }
-    return launch_fused<K, 256>(a, stream);
+    return launch_fused<K, 256, false>(a, stream);
 }
 
 bool in_list(int v, std::initializer_list<int> values)
@@ -864,6 +1036,22 @@ extern "C" int bitsknn_fused_l2_topk_f32(const float* queries_dim_major,
     return bitsknn::fused_impl(queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, k,
                                query_reg, db_reg, dim_reg, block_query_dim, dim_mult, nullptr, 0, false,
                                stream);
+}
+
+extern "C" int bitsknn_fused_set_arithmetic(int arithmetic)
+{
+    bitsknn::clear_error();
+    if (arithmetic != BITSKNN_FUSED_FP32 && arithmetic != BITSKNN_FUSED_BF16X3)
+    {
+        return bitsknn::fail(BITSKNN_ERR_INVALID, "bitsknn_fused_set_arithmetic: unknown arithmetic %d", arithmetic);
+    }
+    bitsknn::g_arithmetic.store(arithmetic, std::memory_order_relaxed);
+    return BITSKNN_OK;
+}
+
+extern "C" int bitsknn_fused_get_arithmetic(void)
+{
+    return bitsknn::g_arithmetic.load(std::memory_order_relaxed);
 }
 
 extern "C" size_t bitsknn_fused_workspace_bytes(int32_t q, int32_t n, int k)
