@@ -1,0 +1,803 @@
+// bits-fused for gfx950: partial squared L2 distance (||p||^2 - 2 q.p) and top-k in one kernel.
+// The q x n distance matrix never leaves the registers of the wave that computes it.
+//
+// Replaces the reference's fused_cache_kernel
+// (include/bits/topk/singlepass/fused_cache_kernel_structs.cuh:663-800: distance tiles :315-632,
+// per-query buffers and merges :25-305).  Same phases -- distance tile, filter against the k-th
+// distance of each query, append to a per-query buffer, merge buffers into sorted top-k lists --
+// laid out for the matrix cores and 64-wide waves:
+//
+//  * A workgroup of 4 waves owns 128 queries (32 per wave) and walks over its range of points in
+//    stages of PT points, two stages in LDS (one being multiplied, one being filled; one barrier
+//    per stage).  A stage is the MFMA A operand: rows 0..d-1 hold the points, the following rows
+//    hold the staging threads' shares of ||p||^2, so that v_mfma_f32_32x32x2_f32 against the query
+//    fragment (-2q_0..-2q_{d-1}, 1, 1) yields ||p||^2 - 2 q.p directly, the dot product accumulated
+//    first and the norm added last.  For d <= 16 the norm is the initial accumulator instead.
+//  * The query fragment stays in registers for the whole kernel.  In the 32 x 32 result tile a
+//    lane holds 16 distances of ONE query (column), so the filter is a min-tree over 16
+//    registers and one compare against that query's radius.
+//  * Every query has a 32-slot buffer in LDS.  Slots are handed out without atomics: the two
+//    lanes that share a query exchange their pass counts, and the fill is kept in a register.
+//    Before a tile would overflow any buffer of the wave, the wave merges all its buffers; the
+//    other waves of the workgroup, which would wait for it at the stage barrier, then merge
+//    theirs in the same stage.
+//  * The sorted top-k lists live in the output arrays themselves between merges, read back by the
+//    lanes that wrote them (plain loads and stores, requested one pass ahead).  A merge is a
+//    segmented bitonic network in registers, 4 keys per lane: 8 queries per pass for k <= 32;
+//    for longer lists the buffers are sorted in place first (8 queries per pass) and then merged
+//    into the lists of 4, 2 or 1 queries per pass.
+//  * With few queries the points are cut into ranges (blockIdx.y) whose partial lists go to a
+//    caller-provided workspace and are reduced by one bits top-k pass with explicit labels.
+//
+// Equal distances are ordered by lower point index: points are visited in index order, so a
+// value equal to a query's radius can never displace what is already merged.
+
+#ifndef BITSKNN_CSRC_FUSED_KERNEL_HPP_
+#define BITSKNN_CSRC_FUSED_KERNEL_HPP_
+
+#include <type_traits>
+
+#include "bitonic_net.hpp"
+#include "common.hpp"
+#include "fused_args.hpp"
+
+namespace bitsknn
+{
+
+namespace
+{
+
+// f(integral_constant<int, BEGIN>) ... f(integral_constant<int, END - 1>), expanded by the front end
+template <int BEGIN, int END, typename F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (BEGIN < END)
+    {
+        f(std::integral_constant<int, BEGIN>{});
+        static_for<BEGIN + 1, END>(f);
+    }
+}
+
+
+typedef float vfloat16 __attribute__((ext_vector_type(16)));
+typedef float vfloat4 __attribute__((ext_vector_type(4)));
+typedef u32 vuint4 __attribute__((ext_vector_type(4)));
+typedef __bf16 vbf16x8 __attribute__((ext_vector_type(8)));
+
+// minimum of three values in one instruction; a NaN operand is ignored
+__device__ __forceinline__ float min3(float a, float b, float c)
+{
+    float r;
+    asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// x[i] = x1 + x2 + x3 exactly, each piece with at most 8 significant bits (a bf16): the upper
+// halves of x, of x - x1 and of x - x1 - x2.  Piece c of values 2j and 2j+1 shares word j of pc.
+__device__ __forceinline__ void split_bf16x3(const float (&x)[8], vuint4& p1, vuint4& p2, vuint4& p3)
+{
+    u32 b1[8];
+    u32 b2[8];
+    u32 b3[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+    {
+        b1[i] = __builtin_bit_cast(u32, x[i]);
+        const float r = x[i] - __builtin_bit_cast(float, b1[i] & 0xFFFF0000U);
+        b2[i] = __builtin_bit_cast(u32, r);
+        const float l = r - __builtin_bit_cast(float, b2[i] & 0xFFFF0000U);
+        b3[i] = __builtin_bit_cast(u32, l);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        // bytes 3:2 of the odd value above bytes 3:2 of the even one
+        p1[j] = __builtin_amdgcn_perm(b1[2 * j + 1], b1[2 * j], 0x07060302U);
+        p2[j] = __builtin_amdgcn_perm(b2[2 * j + 1], b2[2 * j], 0x07060302U);
+        p3[j] = __builtin_amdgcn_perm(b3[2 * j + 1], b3[2 * j], 0x07060302U);
+    }
+}
+
+
+
+// Stage geometry by padded dimension DP.
+//
+// SPLIT = false: fp32 matrix instructions; a stage is (DP + norm rows) x PT floats, PT points per
+// stage so that it stays below 20 KB for DP <= 128.
+//
+// SPLIT = true (DP <= 32): every fp32 value x is cut into three bf16 pieces x = x1 + x2 + x3
+// (exactly: 8 + 8 + 8 significant bits) and a product x*y is the sum of the bf16 products
+// x3*y1 + x2*y2 + x1*y3 + x2*y1 + x1*y2 + x1*y1 accumulated in fp32 (what is left out is below
+// 2^-23 of the product, the size of one fp32 rounding).  The bf16 matrix path runs at 16 times
+// the fp32 one and does not share the vector unit with it.  A stage holds, per piece and per 8
+// dimensions, one 16-byte cell per point (the A operand of v_mfma_f32_32x32x16_bf16), then the
+// norms of the points.
+template <int DP, bool SPLIT>
+struct fused_geometry
+{
+    static constexpr int DK = DP < 16 ? 16 : DP;       // SPLIT: dimensions padded to whole matrix steps
+    static constexpr int KB = DK / 16;                 // SPLIT: matrix steps of 16 dimensions
+    static constexpr int KS = DK / 8;                  // SPLIT: cells of 8 dimensions per point and piece
+    static constexpr int PT = SPLIT ? (DK <= 16 ? 128 : 64)
+                                    : (DP <= 16 ? 256 : (DP <= 32 ? 128 : (DP <= 64 ? 64 : 32)));
+    static constexpr int TPP = FQ_THREADS / PT; // threads per point when staging
+    // point rows (zero beyond dim), then one row per staging thread of a point with its share of
+    // ||p||^2 (at least two rows, so that the row count is even)
+    static constexpr int NORM_ROWS = TPP > 2 ? TPP : 2;
+    static constexpr int ROWS = DP + NORM_ROWS;
+    static constexpr int STEPS = ROWS / 2;    // MFMA steps of 2 rows
+    static constexpr int VPT = SPLIT ? 8 : DP / TPP; // values a thread carries from global memory to LDS
+    static constexpr int MT = PT / 32;        // MFMA row tiles per stage
+    static constexpr int STAGE_FLOATS = SPLIT ? 3 * KS * PT * 4 + PT : ROWS * PT;
+    static_assert(!SPLIT || (DP <= 32 && TPP == KS), "one staging thread per point and cell");
+    static constexpr size_t lds_bytes()
+    {
+        // two stages (one being multiplied, one being filled), the query buffers, exchange slots
+        return 2 * static_cast<size_t>(STAGE_FLOATS) * sizeof(float) +
+               static_cast<size_t>(FQ_WAVES) * FQ_QW * FQ_CAP * sizeof(u64) +
+               static_cast<size_t>(FQ_WAVES) * WAVE * sizeof(float) + 4 * sizeof(int);
+    }
+};
+
+// K: list length.  DP: dimension padded to 8, 16, 32, 64, 128 or 256 (padding rows are zero on
+// both sides of the product).
+template <int K, int DP, bool SPLIT>
+__global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
+{
+    using G = fused_geometry<DP, SPLIT>;
+    constexpr int PT = G::PT;
+    // Norms in the accumulator: where one staging thread carries a whole point (DP <= 16) its
+    // ||p||^2 is one row after the point rows and is read as the initial value of the
+    // accumulators, which saves the matrix step that would add it (one of 5 at DP = 8, one of 9 at
+    // DP = 16; at DP = 32 the 32 registers it takes cost as much as the 17th step).  The sum then
+    // starts from the norm instead of ending with it: same terms, another rounding order.
+    constexpr bool NORM_IN_C = SPLIT || (G::TPP == 1 && G::MT >= 2);
+    constexpr int STEPS = NORM_IN_C ? DP / 2 : G::STEPS;
+    constexpr int KB = G::KB;
+    constexpr int KS = G::KS;
+    constexpr int TPP = G::TPP;
+    constexpr int VPT = G::VPT;
+    constexpr int MT = G::MT;
+    // merge layout: S keys per query spread over LPQ lanes, R keys per lane
+    constexpr int S = K > FQ_CAP ? K : FQ_CAP;
+    constexpr int R = 4;
+    constexpr int LPQ = S / R;
+    constexpr int QPP = WAVE / LPQ;           // queries per merge pass
+    constexpr int PASSES = FQ_QW / QPP;
+
+    extern __shared__ float lds[];
+    constexpr int STAGE_FLOATS = G::STAGE_FLOATS;
+    float* const stages = lds;                                                    // [2][STAGE_FLOATS]
+    u64* const buffers = reinterpret_cast<u64*>(lds + 2 * STAGE_FLOATS);          // [waves][32][CAP]
+    float* const xchg = reinterpret_cast<float*>(buffers + FQ_WAVES * FQ_QW * FQ_CAP);  // [waves][64]
+    int* const merge_wanted = reinterpret_cast<int*>(xchg + FQ_WAVES * WAVE);           // [3]
+
+    const int dim = a.dim;
+    // this workgroup's range of points
+    const int n_begin = static_cast<int>(blockIdx.y) * a.split_points;
+    const int n = a.n < n_begin + a.split_points ? a.n : n_begin + a.split_points;
+    const size_t total_points = static_cast<size_t>(a.n);
+    const int t = static_cast<int>(threadIdx.x);
+    const int lane = t & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(t / WAVE);
+    const int half = lane / 32;               // which of the two rows of an MFMA step
+    const int ql = lane & 31;                 // query of this lane inside the wave
+    const int wave_q0 = static_cast<int>(blockIdx.x) * FQ_QB + wave * FQ_QW;
+    const int my_q = wave_q0 + ql;
+    u64* const wbuf = buffers + static_cast<size_t>(wave) * FQ_QW * FQ_CAP;
+    float* const wx = xchg + wave * WAVE;     // 32 radii, then 32 fills (as int bits)
+
+    // query fragment: step s of this lane is row 2s + half, times -2 (the stages hold the plain
+    // point values); the norm rows are multiplied by 1
+    float qf[SPLIT ? 1 : STEPS];
+    // SPLIT: the three bf16 pieces of -2q for the 8 dimensions 16*kb + 8*half .. + 7 of step kb
+    vuint4 qs[SPLIT ? 3 : 1][SPLIT ? KB : 1];
+    if constexpr (SPLIT)
+    {
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+        {
+            float val[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+            {
+                const int dd = 16 * kb + 8 * half + j;
+                val[j] = 0.0F;
+                if (dd < dim && my_q < a.q)
+                {
+                    val[j] = -2.0F * a.queries[static_cast<size_t>(dd) * a.q + my_q];
+                }
+            }
+            split_bf16x3(val, qs[0][kb], qs[1][kb], qs[2][kb]);
+        }
+        qf[0] = 0.0F;
+    }
+    else
+    {
+        qs[0][0] = vuint4{0, 0, 0, 0};
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s)
+        {
+            const int dd = 2 * s + half;
+            float val = dd >= DP ? 1.0F : 0.0F;
+            if (dd < dim && my_q < a.q)
+            {
+                val = -2.0F * a.queries[static_cast<size_t>(dd) * a.q + my_q];
+            }
+            qf[s] = val;
+        }
+    }
+
+    // rows that never change in either stage: padding dimensions, unused norm rows
+    for (int i = t; i < 2 * STAGE_FLOATS; i += FQ_THREADS)
+    {
+        lds[i] = 0.0F;
+    }
+    if (t < 3)
+    {
+        merge_wanted[t] = 0;
+    }
+    __syncthreads();
+
+    float radius = __builtin_inff(); // k-th smallest distance of my query so far
+    int fill = 0;                    // used slots of my query's buffer (same in both lanes of a query)
+    bool have_list = false;          // wave-uniform: the lists in the output arrays are valid
+    bool merged = false;             // wave-uniform: this wave has merged during the current stage
+    int stage_slot = 0;              // stage index modulo 3: the slot of merge_wanted in use
+
+    // ---- merge of all buffers of this wave into the lists --------------------------------------
+    auto merge_event = [&]() __attribute__((always_inline)) {
+        reinterpret_cast<int*>(wx)[32 + ql] = fill;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if constexpr (K > FQ_CAP)
+        {
+            // Lists longer than a buffer: the buffers are sorted in place first, 8 queries at a
+            // time, so that the passes below only pay for the merge network of the list.
+            constexpr int BR = 4;           // keys per lane
+            constexpr int BL = FQ_CAP / BR; // lanes per buffer
+#pragma unroll 1
+            for (int pass = 0; pass < FQ_QW / (WAVE / BL); ++pass)
+            {
+                const int qm = pass * (WAVE / BL) + lane / BL;
+                const int sub = lane % BL;
+                const int used = reinterpret_cast<const int*>(wx)[32 + qm];
+                u64 buf[BR];
+#pragma unroll
+                for (int r = 0; r < BR; ++r)
+                {
+                    const int i = sub * BR + r;
+                    buf[r] = i < used ? wbuf[qm * FQ_CAP + i] : PAD_KEY;
+                }
+                net_sort<BL, BR, 2, true>(buf, nullptr, sub);
+#pragma unroll
+                for (int r = 0; r < BR; ++r)
+                {
+                    wbuf[qm * FQ_CAP + sub * BR + r] = buf[r];
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+        // The list of a query is read by the lanes that wrote it in the previous merge (same
+        // pass, same positions), so plain loads and stores in program order are enough.  The list
+        // of the next pass is requested before the network of this one runs.
+        const int sub = lane % LPQ;
+        float next_dist[R];
+        std::int32_t next_label[R];
+        auto request_list = [&](int pass) __attribute__((always_inline)) {
+            const int gq = wave_q0 + pass * QPP + lane / LPQ;
+            const size_t at = (static_cast<size_t>(gq) * a.splits + blockIdx.y) * K + sub * R;
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+            {
+                next_dist[r] = __builtin_inff();
+                next_label[r] = 0x7FFFFFFF;
+                if (have_list && sub * R + r < K && gq < a.q)
+                {
+                    next_dist[r] = a.out_dist[at + r];
+                    next_label[r] = a.out_label[at + r];
+                }
+            }
+        };
+        request_list(0);
+#pragma unroll 1
+        for (int pass = 0; pass < PASSES; ++pass)
+        {
+            const int qm = pass * QPP + lane / LPQ; // query (inside the wave) of this lane group
+            const int gq = wave_q0 + qm;
+            const int used = reinterpret_cast<const int*>(wx)[32 + qm];
+            u64 buf[R];
+            u64 list[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+            {
+                const int i = sub * R + r;
+                if constexpr (K > FQ_CAP)
+                {
+                    // the sorted buffer (descending, padding first) is the tail of a descending
+                    // sequence of K keys
+                    buf[r] = i >= K - FQ_CAP ? wbuf[qm * FQ_CAP + i - (K - FQ_CAP)] : PAD_KEY;
+                }
+                else
+                {
+                    buf[r] = i < used ? wbuf[qm * FQ_CAP + (i < FQ_CAP ? i : 0)] : PAD_KEY;
+                }
+                list[r] = make_key(next_dist[r], next_label[r]);
+            }
+            if (pass + 1 < PASSES)
+            {
+                request_list(pass + 1);
+            }
+            // buffer descending, element-wise minimum with the ascending list, re-sort
+            if constexpr (K <= FQ_CAP)
+            {
+                net_sort<LPQ, R, 2, true>(buf, nullptr, sub);
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+            {
+                list[r] = buf[r] < list[r] ? buf[r] : list[r];
+            }
+            net_phase<LPQ, R, S, S / 2, false>(list, nullptr, sub);
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+            {
+                const int i = sub * R + r;
+                if (i < K && gq < a.q)
+                {
+                    const size_t at = (static_cast<size_t>(gq) * a.splits + blockIdx.y) * K + i;
+                    a.out_dist[at] = key_value(list[r]);
+                    a.out_label[at] = key_label(list[r]);
+                }
+                if (i == K - 1)
+                {
+                    wx[qm] = key_value(list[r]);
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        radius = wx[ql];
+        fill = 0;
+        have_list = true;
+        merged = true;
+    };
+
+    // position of this lane's A operands inside a stage row, for the two tiles of a pair (the
+    // second one is kept opaque so that it stays a base register of its own)
+    int tile_at[2] = {half * PT + ql, half * PT + ql + 32};
+    asm volatile("" : "+v"(tile_at[1]));
+
+    // ---- filter one 32 x 32 tile held in `acc` and append what passes ---------------------------
+    // lane holds 16 distances of query ql: rows 8*(r/4) + 4*half + r%4 of the tile
+    const int partner_addr = (lane ^ 32) << 2; // byte address of the lane that shares this lane's query
+    auto append_tile = [&](const vfloat16& acc, int tile_base) __attribute__((always_inline)) {
+        // One compare per value: its lane mask stays in scalar registers and serves the count and
+        // the predicate of the write (vector instructions take their cycles from the matrix
+        // instructions of both waves of the SIMD, scalar ones do not).
+        u64 pass[16];
+        auto compare = [&]() __attribute__((always_inline)) -> int {
+            int count = 0;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+            {
+                const bool below = acc[r] < radius;
+                pass[r] = __builtin_amdgcn_ballot_w64(below);
+                count += below ? 1 : 0;
+            }
+            return count;
+        };
+        int mine = compare();
+        int other = __builtin_amdgcn_ds_bpermute(partner_addr, mine);
+        if (__builtin_amdgcn_ballot_w64(fill + mine + other > FQ_CAP) != 0)
+        {
+            // the other waves of the workgroup would wait for this wave at the stage barrier:
+            // they are asked to merge their buffers in the meantime
+            if (lane == 0)
+            {
+                __hip_atomic_store(merge_wanted + stage_slot, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+            merge_event();
+            mine = compare();
+            other = __builtin_amdgcn_ds_bpermute(partner_addr, mine);
+        }
+        int slot = fill + (half != 0 ? other : 0);
+        const int first_point = tile_base + 4 * half;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+        {
+            if (pass[r] != 0)
+            {
+                if (__builtin_amdgcn_inverse_ballot_w64(pass[r]))
+                {
+                    wbuf[ql * FQ_CAP + slot] = make_key(acc[r], first_point + 8 * (r / 4) + (r % 4));
+                    ++slot;
+                }
+            }
+        }
+        fill += mine + other;
+    };
+    auto filter_tile = [&](const vfloat16& acc, int tile_base) __attribute__((always_inline)) {
+        // The first read of the tile is a compare the compiler sees, so that it places the wait
+        // states a matrix result needs before them; the minimum of the other 15 values is written
+        // out as v_min3 (fminf would first quieten each operand with an instruction of its own),
+        // and assembly operands are not covered by that hazard handling.
+        const u64 last_passes = __builtin_amdgcn_ballot_w64(acc[15] < radius);
+        __builtin_amdgcn_sched_barrier(0);
+        float low[5];
+#pragma unroll
+        for (int g = 0; g < 5; ++g)
+        {
+            low[g] = min3(acc[3 * g], acc[3 * g + 1], acc[3 * g + 2]);
+        }
+        const float smallest = min3(min3(low[0], low[1], low[2]), low[3], low[4]);
+        if ((last_passes | __builtin_amdgcn_ballot_w64(smallest < radius)) != 0)
+        {
+            append_tile(acc, tile_base);
+        }
+    };
+
+    // ---- staging: global -> registers -> LDS ---------------------------------------------------
+    // thread t carries dimensions (t / PT) + TPP*i of point t % PT, writes them as rows of the
+    // stage and adds up its share of ||p||^2 (the shares of a point meet inside the MFMA)
+    // SPLIT: thread t carries the 8 dimensions 8*(t % TPP) .. + 7 of point t / TPP (the threads of
+    // a point are neighbouring lanes, which add up their shares of the norm among themselves)
+    const int sp = SPLIT ? t / TPP : t % PT;
+    const int sd0 = SPLIT ? 8 * (t % TPP) : t / PT;
+    auto dim_of = [&](int i) -> int { return SPLIT ? sd0 + i : sd0 + TPP * i; };
+    float pre[VPT];
+    // Point values are read with buffer loads: a constant byte offset per value and lane (beyond
+    // the resource for dimensions dim .. DP-1, which then read as zero; the hardware checks the
+    // lane offset only) plus the scalar offset of the stage, so that a load needs no vector
+    // arithmetic.  Point matrices of 2 GiB and more take the plain loads.
+    const bool small_points = static_cast<size_t>(dim) * total_points * sizeof(float) < (1ULL << 31);
+    const auto point_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(a.points), 0,
+        small_points ? static_cast<int>(static_cast<size_t>(dim) * total_points * sizeof(float)) : 0, 0x00020000);
+    constexpr int OUTSIDE = 0x7FFFFFF0;
+    int load_off[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i)
+    {
+        const int dd = dim_of(i);
+        load_off[i] = dd < dim && small_points
+                          ? static_cast<int>((static_cast<size_t>(dd) * total_points + sp) * sizeof(float))
+                          : OUTSIDE;
+    }
+    auto fetch = [&](int base) {
+        if (small_points)
+        {
+            const int stage_off = base * static_cast<int>(sizeof(float));
+            if (base + PT <= n)
+            {
+#pragma unroll
+                for (int i = 0; i < VPT; ++i)
+                {
+                    pre[i] = __builtin_bit_cast(
+                        float, __builtin_amdgcn_raw_buffer_load_b32(point_rsrc, load_off[i], stage_off, 0));
+                }
+            }
+            else
+            {
+                // ragged last stage: points from n on read as zero
+                const bool inside = base + sp < n;
+#pragma unroll
+                for (int i = 0; i < VPT; ++i)
+                {
+                    pre[i] = __builtin_bit_cast(
+                        float, __builtin_amdgcn_raw_buffer_load_b32(point_rsrc, inside ? load_off[i] : OUTSIDE,
+                                                                    stage_off, 0));
+                }
+            }
+        }
+        else
+        {
+            const int j = base + sp;
+#pragma unroll
+            for (int i = 0; i < VPT; ++i)
+            {
+                const int dd = dim_of(i);
+                pre[i] = 0.0F;
+                if (dd < dim && j < n)
+                {
+                    pre[i] = a.points[static_cast<size_t>(dd) * total_points + j];
+                }
+            }
+        }
+    };
+    auto deposit = [&](float* stage, int base) {
+        float share = 0.0F;
+        if constexpr (SPLIT)
+        {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+            {
+                share = __builtin_fmaf(pre[i], pre[i], share);
+            }
+            vuint4 piece[3];
+            split_bf16x3(pre, piece[0], piece[1], piece[2]);
+            vuint4* const cells = reinterpret_cast<vuint4*>(stage);
+            const int ks = sd0 / 8;
+#pragma unroll
+            for (int c = 0; c < 3; ++c)
+            {
+                cells[(c * KS + ks) * PT + sp] = piece[c];
+            }
+            // the threads of a point are TPP neighbouring lanes
+            share += __builtin_bit_cast(float, lane_xor32<1>(__builtin_bit_cast(u32, share)));
+            if constexpr (TPP == 4)
+            {
+                share += __builtin_bit_cast(float, lane_xor32<2>(__builtin_bit_cast(u32, share)));
+            }
+            // points beyond the end get an infinite distance and never pass the filter
+            stage[3 * KS * PT * 4 + sp] = base + sp < n ? share : __builtin_inff();
+        }
+        else
+        {
+#pragma unroll
+            for (int i = 0; i < VPT; ++i)
+            {
+                const int dd = sd0 + TPP * i;
+                share = __builtin_fmaf(pre[i], pre[i], share);
+                // (dimensions from dim on were read as zero: their rows stay zero)
+                stage[dd * PT + sp] = pre[i];
+            }
+            // points beyond the end get an infinite distance and never pass the filter
+            // (with one staging thread per point the share is the norm, in row DP)
+            stage[(DP + sd0) * PT + sp] = base + sp < n ? share : __builtin_inff();
+        }
+    };
+
+    // all row tiles of a stage: distances, filter, append
+    auto multiply = [&](const float* stage, int base) {
+        if constexpr (SPLIT)
+        {
+            constexpr int PAIRS = MT / 2;
+            const vuint4* const cells = reinterpret_cast<const vuint4*>(stage);
+            const float* const norm_row = stage + 3 * KS * PT * 4;
+            static_for<0, PAIRS>([&](auto p_tag) {
+                constexpr int p = decltype(p_tag)::value;
+                // A operands of the two tiles: piece c of dimensions 16*kb + 8*half .. + 7
+                vuint4 af[2][3][KB];
+#pragma unroll
+                for (int tile = 0; tile < 2; ++tile)
+                {
+#pragma unroll
+                    for (int c = 0; c < 3; ++c)
+                    {
+#pragma unroll
+                        for (int kb = 0; kb < KB; ++kb)
+                        {
+                            af[tile][c][kb] = cells[(c * KS + 2 * kb + half) * PT + p * 64 + tile * 32 + ql];
+                        }
+                    }
+                }
+                // the accumulators start from the norms of the lane's 16 points
+                vfloat16 acc0;
+                vfloat16 acc1;
+                const float* norms = norm_row + p * 64 + 4 * half;
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                {
+                    const vfloat4 x = *reinterpret_cast<const vfloat4*>(norms + 8 * g);
+                    const vfloat4 y = *reinterpret_cast<const vfloat4*>(norms + 32 + 8 * g);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                    {
+                        acc0[4 * g + e] = x[e];
+                        acc1[4 * g + e] = y[e];
+                    }
+                }
+                // the six products of a step, smallest terms first
+                constexpr int order[6][2] = {{2, 0}, {1, 1}, {0, 2}, {1, 0}, {0, 1}, {0, 0}};
+                static_for<0, KB>([&](auto kb_tag) {
+                    constexpr int kb = decltype(kb_tag)::value;
+                    static_for<0, 6>([&](auto o_tag) {
+                        constexpr int ca = order[decltype(o_tag)::value][0];
+                        constexpr int cb = order[decltype(o_tag)::value][1];
+                        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(vbf16x8, af[0][ca][kb]), __builtin_bit_cast(vbf16x8, qs[cb][kb]),
+                            acc0, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(vbf16x8, af[1][ca][kb]), __builtin_bit_cast(vbf16x8, qs[cb][kb]),
+                            acc1, 0, 0, 0);
+                    });
+                });
+                filter_tile(acc0, base + p * 64);
+                filter_tile(acc1, base + p * 64 + 32);
+            });
+        }
+        else if constexpr (MT >= 2)
+        {
+            // Two row tiles at a time: two independent accumulator chains keep the matrix core
+            // issuing back to back.  The A operands of a pair sit in registers before its first
+            // MFMA; those of the next pair are requested from LDS between the MFMAs of this one
+            // (LDS instructions are overlapped with matrix instructions, vector-ALU ones are not).
+            constexpr int PAIRS = MT / 2;
+            float a[2][2][STEPS];
+            // The reads of one tile are 2*PT floats apart, which a two-address LDS read with
+            // offsets in units of 64 floats covers from one base register per tile; pairing the
+            // two tiles of a step instead needs an address computation per step.
+            const float* arow0 = stage + tile_at[0];
+            const float* arow1 = stage + tile_at[1];
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+            {
+                a[0][0][s] = arow0[2 * s * PT];
+            }
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+            {
+                a[0][1][s] = arow1[2 * s * PT];
+            }
+            // initial accumulators of a pair: zero, or the norms of the lane's 16 points
+            vfloat16 init0;
+            vfloat16 init1;
+            auto request_init = [&](int pair) __attribute__((always_inline)) {
+                if constexpr (NORM_IN_C)
+                {
+                    const float* norms = stage + DP * PT + pair * 64 + 4 * half;
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                    {
+                        const vfloat4 x = *reinterpret_cast<const vfloat4*>(norms + 8 * g);
+                        const vfloat4 y = *reinterpret_cast<const vfloat4*>(norms + 32 + 8 * g);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                        {
+                            init0[4 * g + e] = x[e];
+                            init1[4 * g + e] = y[e];
+                        }
+                    }
+                }
+                else
+                {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                    {
+                        init0[r] = 0.0F;
+                        init1[r] = 0.0F;
+                    }
+                }
+            };
+            request_init(0);
+            __builtin_amdgcn_sched_barrier(0); // keep the reads above the chain
+            static_for<0, PAIRS>([&](auto p_tag) {
+                constexpr int p = decltype(p_tag)::value;
+                constexpr int cur = p & 1;
+                vfloat16 acc0 = init0;
+                vfloat16 acc1 = init1;
+                static_for<0, STEPS>([&](auto s_tag) {
+                    constexpr int s = decltype(s_tag)::value;
+                    if constexpr (p + 1 < PAIRS)
+                    {
+                        // steps (s, s+1) of the first tile in even steps, (s-1, s) of the second
+                        // tile in odd ones
+                        constexpr int next = 64 * (p + 1);
+                        if constexpr (s % 2 == 0)
+                        {
+                            a[cur ^ 1][0][s] = arow0[2 * s * PT + next];
+                            if constexpr (s + 1 < STEPS)
+                            {
+                                a[cur ^ 1][0][s + 1] = arow0[2 * (s + 1) * PT + next];
+                            }
+                            else
+                            {
+                                a[cur ^ 1][1][s] = arow1[2 * s * PT + next];
+                            }
+                        }
+                        else
+                        {
+                            a[cur ^ 1][1][s - 1] = arow1[2 * (s - 1) * PT + next];
+                            a[cur ^ 1][1][s] = arow1[2 * s * PT + next];
+                        }
+                    }
+                    acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][0][s], qf[s], acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][1][s], qf[s], acc1, 0, 0, 0);
+                    if constexpr (NORM_IN_C && s == 0 && p + 1 < PAIRS)
+                    {
+                        request_init(p + 1); // the first step has taken this pair's
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+                filter_tile(acc0, base + p * 64);
+                filter_tile(acc1, base + p * 64 + 32);
+            });
+        }
+        else
+        {
+            vfloat16 acc0;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+            {
+                acc0[r] = 0.0F;
+            }
+            const float* arow = stage + half * PT + ql;
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+            {
+                acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(arow[2 * s * PT], qf[s], acc0, 0, 0, 0);
+            }
+            filter_tile(acc0, base);
+        }
+    };
+
+    // Stage s is multiplied while stage s+1 sits in registers and is written to the other LDS
+    // buffer afterwards; stage s+2 is requested from memory right after that.  One barrier per
+    // stage: it separates the last read of a buffer from its next fill and the fill from its
+    // first read.  A wave that had to merge in stage s raises merge_wanted[s % 3]; the others look
+    // at it before and after the barrier of that stage (the flag for stage s + 2 is cleared after the
+    // barrier of stage s: its last readers passed it before that barrier, its next writers come
+    // after the following one).
+    auto merge_if_wanted = [&]() __attribute__((always_inline)) {
+        if (!merged && __hip_atomic_load(merge_wanted + stage_slot, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_WORKGROUP) != 0)
+        {
+            merge_event();
+        }
+    };
+    fetch(n_begin);
+    // the query fragment and the first stage have arrived (nothing else is in flight yet)
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    deposit(stages, n_begin);
+    if (n_begin + PT < n)
+    {
+        fetch(n_begin + PT);
+    }
+    __syncthreads();
+    int parity = 0;
+    for (int base = n_begin; base < n; base += PT)
+    {
+        merged = false;
+        multiply(stages + parity * STAGE_FLOATS, base);
+        parity ^= 1;
+        if (base + PT < n)
+        {
+            deposit(stages + parity * STAGE_FLOATS, base + PT);
+            if (base + 2 * PT < n)
+            {
+                fetch(base + 2 * PT);
+            }
+        }
+        merge_if_wanted();
+        __syncthreads();
+        merge_if_wanted();
+        if (t == 0)
+        {
+            merge_wanted[(stage_slot + 2) % 3] = 0;
+        }
+        stage_slot = stage_slot == 2 ? 0 : stage_slot + 1;
+    }
+
+    // whatever is left in the buffers; also writes the lists of queries that never merged
+    merge_event();
+}
+
+template <int K, int DP, bool SPLIT>
+hipError_t launch_fused(const fused_args& a, hipStream_t stream)
+{
+    constexpr size_t lds_bytes = fused_geometry<DP, SPLIT>::lds_bytes();
+    if (lds_bytes > 48 * 1024)
+    {
+        const hipError_t status =
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<K, DP, SPLIT>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+        if (status != hipSuccess)
+        {
+            return status;
+        }
+    }
+    const unsigned grid = static_cast<unsigned>((a.q + FQ_QB - 1) / FQ_QB);
+    hipLaunchKernelGGL((fused_kernel<K, DP, SPLIT>), dim3(grid, static_cast<unsigned>(a.splits)),
+                       dim3(FQ_THREADS), lds_bytes, stream, a);
+    return hipGetLastError();
+}
+
+} // namespace
+} // namespace bitsknn
+
+#endif // BITSKNN_CSRC_FUSED_KERNEL_HPP_

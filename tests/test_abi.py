@@ -53,6 +53,16 @@ def test_topk_rejects_unsupported_parameters(bk, k, block, batch, msg):
     assert text == msg
 
 
+def test_fused_arithmetic_switch(bk):
+    assert bk.fused_get_arithmetic() == bk.FUSED_FP32
+    bk.fused_set_arithmetic(bk.FUSED_BF16X3)
+    assert bk.fused_get_arithmetic() == bk.FUSED_BF16X3
+    bk.fused_set_arithmetic(bk.FUSED_FP32)
+    with pytest.raises(bk.BitsKnnError, match="unknown arithmetic 7"):
+        bk.fused_set_arithmetic(7)
+    assert bk.fused_get_arithmetic() == bk.FUSED_FP32
+
+
 def test_topk_accepts_reference_parameter_lists_with_zero_rows(bk):
     # rows == 0 is a no-op that returns before any launch: every supported combination is accepted
     for block in (128, 256, 512):

@@ -257,3 +257,79 @@ def test_random_shapes_against_the_oracle(bk, dev, oracle):
             _check(oracle, p, s, k, gd, gl)
         except AssertionError as e:
             raise AssertionError((case, n, q, d, k, kind)) from e
+
+
+# ---- products from three bf16 pieces per operand (BITSKNN_FUSED_BF16X3, dimensions 9 .. 32) --------
+
+@pytest.fixture
+def bf16x3(bk):
+    bk.fused_set_arithmetic(bk.FUSED_BF16X3)
+    assert bk.fused_get_arithmetic() == bk.FUSED_BF16X3
+    yield
+    bk.fused_set_arithmetic(bk.FUSED_FP32)
+
+
+@pytest.mark.parametrize("k", [4, 8, 16, 32, 64, 128, 256])
+@pytest.mark.parametrize("d", [9, 16, 17, 32])
+def test_bf16x3_all_k_values(bk, dev, oracle, bf16x3, k, d):
+    p, s = oracle.generate(200 + k + d, 20000, 150, d)
+    gd, gl = _fused(bk, dev, p, s, k)
+    _check(oracle, p, s, k, gd, gl)
+
+
+@pytest.mark.parametrize("n,q", [(1, 1), (31, 5), (32, 33), (63, 127), (64, 128), (65, 129), (129, 3), (1000, 300), (5001, 1)])
+def test_bf16x3_ragged_counts(bk, dev, oracle, bf16x3, n, q):
+    for d in (12, 31):
+        p, s = oracle.generate(n + q + d, n, q, d)
+        for k in (4, 32):
+            gd, gl = _fused(bk, dev, p, s, k, (2, 4, 1), 1, 1)
+            _check(oracle, p, s, k, gd, gl)
+
+
+@pytest.mark.parametrize("n,q,d,k", [(20000, 150, 12, 32), (70001, 300, 16, 16), (300000, 33, 32, 4),
+                                     (9000, 1000, 24, 64)])
+def test_bf16x3_point_split_variant_with_workspace(bk, dev, oracle, bf16x3, n, q, d, k):
+    p, s = oracle.generate(n + q + d, n, q, d)
+    gd, gl = _fused(bk, dev, p, s, k, workspace="auto")
+    _check(oracle, p, s, k, gd, gl)
+    pd, pl = _fused(bk, dev, p, s, k)
+    assert np.array_equal(gd, pd) and np.array_equal(gl, pl)
+
+
+def test_bf16x3_random_shapes_against_the_oracle(bk, dev, oracle, bf16x3):
+    import torch
+    rng = np.random.default_rng(99)
+    for case in range(30):
+        d = int(rng.integers(9, 33))
+        k = int(rng.choice([4, 8, 16, 32, 64, 128, 256]))
+        n = int(rng.choice([rng.integers(1, 300), rng.integers(300, 5000), rng.integers(5000, 30000)]))
+        q = int(rng.choice([rng.integers(1, 40), rng.integers(40, 300), rng.integers(300, 600)]))
+        workspace = None if case % 2 == 0 else torch.empty(max(8, 8 * q * 64 * k), dtype=torch.uint8, device=dev)
+        p, s = oracle.generate(4000 + case, n, q, d)
+        gd, gl = _fused(bk, dev, p, s, k, (2, 4, 1), 1, 1, workspace=workspace)
+        try:
+            _check(oracle, p, s, k, gd, gl)
+        except AssertionError as e:
+            raise AssertionError((case, n, q, d, k)) from e
+
+
+def test_bf16x3_is_as_accurate_as_the_fp32_matrix_instructions(bk, dev, oracle):
+    """Error of the reported distances against the exact (fp64) ones, relative to the magnitude of
+    the cancelling terms, for both arithmetics on the same inputs: the split products must stay at
+    the level of fp32 rounding (far inside the 1e-5 bar) and within a small factor of the fp32
+    matrix instructions' own error."""
+    err = {}
+    for d in (16, 32):
+        p, s = oracle.generate(900 + d, 30000, 200, d)
+        truth = oracle.dist(s, p, "f64-partial")
+        qn = (s.astype(np.float64) ** 2).sum(1)[:, None]
+        for mode in (bk.FUSED_FP32, bk.FUSED_BF16X3):
+            bk.fused_set_arithmetic(mode)
+            try:
+                gd, gl = _fused(bk, dev, p, s, 64)
+            finally:
+                bk.fused_set_arithmetic(bk.FUSED_FP32)
+            at = np.take_along_axis(truth, gl.astype(np.int64), axis=1)
+            err[(d, mode)] = float(np.max(np.abs(gd - at) / (np.abs(at) + qn)))
+        assert err[(d, bk.FUSED_BF16X3)] < 1e-6
+        assert err[(d, bk.FUSED_BF16X3)] < 4 * err[(d, bk.FUSED_FP32)] + 1e-7
