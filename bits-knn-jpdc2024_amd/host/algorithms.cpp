@@ -447,6 +447,29 @@ private:
     knn_host::transfer_timer transfer_in_;
 };
 
+// bits-fused with the products from three bf16 pieces per operand (no counterpart in the reference):
+// the same wrapper, the library's arithmetic switched for the duration of the kernel launch
+class fused_cache_bf16x3_knn : public fused_cache_knn
+{
+public:
+    std::string id() const override { return "fused-cache-bf16x3"; }
+
+    void selection() override
+    {
+        BITSKNN_CHECK(bitsknn_fused_set_arithmetic(BITSKNN_FUSED_BF16X3));
+        try
+        {
+            fused_cache_knn::selection();
+        }
+        catch (...)
+        {
+            bitsknn_fused_set_arithmetic(BITSKNN_FUSED_FP32);
+            throw;
+        }
+        BITSKNN_CHECK(bitsknn_fused_set_arithmetic(BITSKNN_FUSED_FP32));
+    }
+};
+
 // ---------------------------------------------------------------------------------------------
 // distance-only runs (reference: include/bits/distance/dist_runner.hpp:8-15)
 // ---------------------------------------------------------------------------------------------
@@ -484,6 +507,7 @@ std::vector<std::unique_ptr<knn>> make_algorithms()
     algorithms.push_back(std::make_unique<single_query_bits>());
     algorithms.push_back(std::make_unique<partial_bitonic_regs>());
     algorithms.push_back(std::make_unique<fused_cache_knn>());
+    algorithms.push_back(std::make_unique<fused_cache_bf16x3_knn>());
     algorithms.push_back(std::make_unique<dist_runner>("cublas-dist", &make_expanded_distance));
     algorithms.push_back(std::make_unique<dist_runner>("magma-dist", &make_l2_distance));
     algorithms.push_back(std::make_unique<dist_runner>("magma-part-dist", &make_partial_l2_distance));

@@ -37,7 +37,7 @@ def test_help_lists_options_and_algorithms_on_stderr():
     p = run("--help")
     assert p.returncode == 0 and p.stdout == ""
     for token in ("--algorithm", "--items-per-thread", "--point-layout", "--deg", "--no-output",
-                  "Available algorithms:", "- bits", "- bits-prefetch", "- bits-sq", "- fused-cache",
+                  "Available algorithms:", "- bits", "- bits-prefetch", "- bits-sq", "- fused-cache", "- fused-cache-bf16x3",
                   "- magma-dist", "- magma-part-dist", "- cublas-dist", "- serial", "- parallel"):
         assert token in p.stderr
 
@@ -139,6 +139,22 @@ def test_golden_fused_checksums_end_to_end(golden):
         assert str(checksums(p)[0]) in rec["checksums"], (rec, checksums(p))
         done += 1
     assert done == 6
+
+
+@pytest.mark.gpu
+def test_golden_fused_checksums_with_bf16x3_products(golden):
+    """The reference's own checksums for d = 16 (the dimension of its fused runs that takes the
+    bf16 pieces), reproduced with the other arithmetic of the products."""
+    done = 0
+    for rec in golden:
+        if rec["family"] != "fused" or rec["d"] != 16 or (rec["n"], rec["q"]) != (131072, 8192) or rec["k"] not in (16, 32):
+            continue
+        p = run("-a", "fused-cache-bf16x3", "-n", "128k", "-q", "8k", "-d", "16", "-k", str(rec["k"]),
+                "--seed", "24", "--items-per-thread", "8,4,2", "--block-size", "1", "--deg", "1")
+        assert p.returncode == 0, p.stderr
+        assert str(checksums(p)[0]) in rec["checksums"], (rec, checksums(p))
+        done += 1
+    assert done == 2
 
 
 @pytest.mark.gpu
