@@ -374,7 +374,6 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 
     // ---- filter one 32 x 32 tile held in `acc` and append what passes ---------------------------
     // lane holds 16 distances of query ql: rows 8*(r/4) + 4*half + r%4 of the tile
-    const int partner_addr = (lane ^ 32) << 2; // byte address of the lane that shares this lane's query
     auto append_tile = [&](const vfloat16& acc, int tile_base) __attribute__((always_inline)) {
         // One compare per value: its lane mask stays in scalar registers and serves the count and
         // the predicate of the write (vector instructions take their cycles from the matrix
@@ -392,7 +391,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             return count;
         };
         int mine = compare();
-        int other = __builtin_amdgcn_ds_bpermute(partner_addr, mine);
+        int other = static_cast<int>(lane_xor32<32>(static_cast<u32>(mine)));
         if (__builtin_amdgcn_ballot_w64(fill + mine + other > FQ_CAP) != 0)
         {
             // the other waves of the workgroup would wait for this wave at the stage barrier:
@@ -403,7 +402,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             }
             merge_event();
             mine = compare();
-            other = __builtin_amdgcn_ds_bpermute(partner_addr, mine);
+            other = static_cast<int>(lane_xor32<32>(static_cast<u32>(mine)));
         }
         int slot = fill + (half != 0 ? other : 0);
         const int first_point = tile_base + 4 * half;
