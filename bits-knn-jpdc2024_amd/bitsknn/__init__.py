@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "libbitsknn.so")
 
 OK, ERR_UNSUPPORTED, ERR_INVALID, ERR_HIP = 0, 1, 2, 3
-DIST_L2, DIST_PARTIAL_L2, DIST_EXPANDED = 0, 1, 2
+DIST_L2, DIST_PARTIAL_L2, DIST_EXPANDED, DIST_PARTIAL_L2_BF16X3 = 0, 1, 2, 3
 
 # every symbol include/bitsknn.h declares
 EXPORTS = (

@@ -17,6 +17,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "dist_split.hpp"
 
 namespace bitsknn
 {
@@ -895,7 +896,8 @@ extern "C" int bitsknn_dist_f32(int op, int dim, size_t q, size_t n, const float
 {
     using namespace bitsknn;
     clear_error();
-    if (op != BITSKNN_DIST_L2 && op != BITSKNN_DIST_PARTIAL_L2 && op != BITSKNN_DIST_EXPANDED)
+    if (op != BITSKNN_DIST_L2 && op != BITSKNN_DIST_PARTIAL_L2 && op != BITSKNN_DIST_EXPANDED &&
+        op != BITSKNN_DIST_PARTIAL_L2_BF16X3)
     {
         return fail(BITSKNN_ERR_UNSUPPORTED, "Unsupported distance: %d", op);
     }
@@ -943,6 +945,15 @@ extern "C" int bitsknn_dist_f32(int op, int dim, size_t q, size_t n, const float
     }
     else
     {
+        // bf16x3 products where that kernel applies (dimensions 9 .. 64, aligned rows), else the fp32
+        // matrix instructions
+        if (op == BITSKNN_DIST_PARTIAL_L2_BF16X3 &&
+            launch_dist_split(dim, q, n, queries_dim_major, query_stride, points_dim_major, point_stride, dist,
+                              dist_row_stride, hip_stream))
+        {
+            BITSKNN_HIP_CHECK(hipGetLastError());
+            return BITSKNN_OK;
+        }
         bool launched = false;
         if (dim <= 8)
         {

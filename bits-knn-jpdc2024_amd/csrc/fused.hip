@@ -126,7 +126,8 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
         reinterpret_cast<std::uintptr_t>(workspace) % 16 == 0)
     {
         auto* matrix = static_cast<float*>(workspace);
-        const int status = bitsknn_dist_f32(BITSKNN_DIST_PARTIAL_L2, dim, static_cast<size_t>(q),
+        const bool split = g_arithmetic.load(std::memory_order_relaxed) == BITSKNN_FUSED_BF16X3;
+        const int status = bitsknn_dist_f32(split ? BITSKNN_DIST_PARTIAL_L2_BF16X3 : BITSKNN_DIST_PARTIAL_L2, dim, static_cast<size_t>(q),
                                             static_cast<size_t>(n), queries_dim_major, static_cast<size_t>(q),
                                             points_dim_major, static_cast<size_t>(n), matrix,
                                             static_cast<size_t>(n), stream);

@@ -89,6 +89,11 @@ std::unique_ptr<device_distance> make_partial_l2_distance()
     return std::make_unique<device_distance>(BITSKNN_DIST_PARTIAL_L2, "magma-part-dist");
 }
 
+std::unique_ptr<device_distance> make_partial_l2_bf16x3_distance()
+{
+    return std::make_unique<device_distance>(BITSKNN_DIST_PARTIAL_L2_BF16X3, "magma-part-dist-bf16x3");
+}
+
 std::unique_ptr<device_distance> make_expanded_distance()
 {
     return std::make_unique<device_distance>(BITSKNN_DIST_EXPANDED, "cublas-dist");
@@ -511,5 +516,7 @@ std::vector<std::unique_ptr<knn>> make_algorithms()
     algorithms.push_back(std::make_unique<dist_runner>("cublas-dist", &make_expanded_distance));
     algorithms.push_back(std::make_unique<dist_runner>("magma-dist", &make_l2_distance));
     algorithms.push_back(std::make_unique<dist_runner>("magma-part-dist", &make_partial_l2_distance));
+    algorithms.push_back(
+        std::make_unique<dist_runner>("magma-part-dist-bf16x3", &make_partial_l2_bf16x3_distance));
     return algorithms;
 }

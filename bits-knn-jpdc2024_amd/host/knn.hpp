@@ -73,6 +73,8 @@ protected:
 
 std::unique_ptr<device_distance> make_l2_distance();         // `magma-dist`
 std::unique_ptr<device_distance> make_partial_l2_distance(); // `magma-part-dist`
+// the same values with bf16x3 products (no counterpart in the reference)
+std::unique_ptr<device_distance> make_partial_l2_bf16x3_distance();
 std::unique_ptr<device_distance> make_expanded_distance();   // `cublas-dist`
 
 class knn

@@ -106,10 +106,17 @@ int bitsknn_fill_f32(float* dst, size_t count, float value, void* stream);
  * and the SGEMM + squared_length_kernel + add_norm_kernel sequence of
  * cublas_distance::compute (src/distance/cublas_distance.cu:111-186) for
  *   BITSKNN_DIST_EXPANDED    -2 q.p on fp32 MFMA, then + ||p||^2, written once
+ * No counterpart in the reference:
+ *   BITSKNN_DIST_PARTIAL_L2_BF16X3  the values of BITSKNN_DIST_PARTIAL_L2 with every fp32 operand
+ *                            cut exactly into three bf16 pieces and a product taken as the fp32
+ *                            sum of six bf16 matrix products (what is left out is below 2^-23 of
+ *                            a product); for dimensions 33 .. 64 and matrix rows that start on
+ *                            16-byte boundaries, otherwise the same as BITSKNN_DIST_PARTIAL_L2
  */
 #define BITSKNN_DIST_L2 0
 #define BITSKNN_DIST_PARTIAL_L2 1
 #define BITSKNN_DIST_EXPANDED 2
+#define BITSKNN_DIST_PARTIAL_L2_BF16X3 3
 int bitsknn_dist_f32(int op, int dim, size_t q, size_t n, const float* queries_dim_major,
                      size_t query_stride, const float* points_dim_major, size_t point_stride,
                      float* dist, size_t dist_row_stride, void* stream);

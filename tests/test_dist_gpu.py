@@ -220,3 +220,40 @@ def test_random_shapes_and_strides_against_the_oracle(bk, dev, oracle):
             exp = oracle.dist(s, p, "partial")
             scale = (p.astype(np.float64) ** 2).sum(1)[None, :] * 2 + (s.astype(np.float64) ** 2).sum(1)[:, None]
             assert np.max(np.abs(got - exp) / np.maximum(scale, 1e-30)) < 1e-5, what
+
+
+# ---- BITSKNN_DIST_PARTIAL_L2_BF16X3: products from three bf16 pieces per operand (dimensions 33 .. 64) ----
+
+@pytest.mark.parametrize("n,q,d", [(1000, 37, 33), (4097, 130, 40), (257, 129, 64), (5000, 200, 48), (129, 5, 63),
+                                   (16385, 129, 64), (70000, 300, 50), (32, 32, 16), (1024, 32, 32), (300, 7, 100)])
+def test_bf16x3_distances(bk, dev, oracle, n, q, d):
+    """Same bar as the fp32 matrix instructions (1e-5 of the cancelling terms, measured: a few
+    1e-7), including the dimensions and shapes for which the operation falls back to them."""
+    p, s = oracle.generate(77, n, q, d)
+    got = _gpu_dist(bk, dev, s, p, bk.DIST_PARTIAL_L2_BF16X3)
+    fp32 = _gpu_dist(bk, dev, s, p, bk.DIST_PARTIAL_L2)
+    truth = oracle.dist(s, p, "f64-partial")
+    scale = (p.astype(np.float64) ** 2).sum(1)[None, :] * 2 + (s.astype(np.float64) ** 2).sum(1)[:, None]
+    err = np.max(np.abs(got - truth) / scale)
+    err32 = np.max(np.abs(fp32 - truth) / scale)
+    assert err < 1e-6 and err < 4 * err32 + 1e-7
+    if d <= 32 or d > 64:
+        assert np.array_equal(got, fp32)
+
+
+def test_bf16x3_distances_views_and_ragged_ends(bk, dev, oracle):
+    """Padded and offset views: aligned rows take the bf16x3 kernel (whole and ragged last tiles,
+    rows beyond the last query of a wave), unaligned ones the fp32 kernels; nothing outside the
+    view is written."""
+    import torch
+    for case, (n, q, opad, off) in enumerate([(1003, 45, 1, 0), (1003, 45, 5, 4), (2050, 130, 2, 0), (64, 33, 0, 0),
+                                              (16384 + 37, 100, 3, 0), (999, 45, 0, 1)]):
+        d = 33 + 7 * case
+        p, s = oracle.generate(17 + case, n, q, d)
+        out = torch.full((q, n + opad + off), -7.0, device=dev)
+        bk.distances(_dm(s, dev), _dm(p, dev), bk.DIST_PARTIAL_L2_BF16X3, out=out[:, off:off + n])
+        torch.cuda.synchronize()
+        assert (out[:, :off] == -7).all() and (out[:, off + n:] == -7).all()
+        exp = oracle.dist(s, p, "partial")
+        scale = (p.astype(np.float64) ** 2).sum(1)[None, :] * 2 + (s.astype(np.float64) ** 2).sum(1)[:, None]
+        assert np.max(np.abs(out[:, off:off + n].cpu().numpy() - exp) / scale) < 1e-5, (n, q, d, opad, off)

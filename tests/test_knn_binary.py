@@ -38,7 +38,7 @@ def test_help_lists_options_and_algorithms_on_stderr():
     assert p.returncode == 0 and p.stdout == ""
     for token in ("--algorithm", "--items-per-thread", "--point-layout", "--deg", "--no-output",
                   "Available algorithms:", "- bits", "- bits-prefetch", "- bits-sq", "- fused-cache", "- fused-cache-bf16x3",
-                  "- magma-dist", "- magma-part-dist", "- cublas-dist", "- serial", "- parallel"):
+                  "- magma-dist", "- magma-part-dist", "- magma-part-dist-bf16x3", "- cublas-dist", "- serial", "- parallel"):
         assert token in p.stderr
 
 
