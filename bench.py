@@ -103,6 +103,7 @@ def gemm_knn(bitsknn, torch, dev, q=4096, n=1 << 20, d=64, k=64, runs=5):
         return start.elapsed_time(end) / 1e3 / runs
 
     t_dist = timed(lambda: bitsknn.distances(queries, points, bitsknn.DIST_PARTIAL_L2, out=dist))
+    t_split = timed(lambda: bitsknn.distances(queries, points, bitsknn.DIST_PARTIAL_L2_BF16X3, out=dist))
     t_topk = timed(lambda: bitsknn.topk_bits(dist, k, 256, 8, out_dist=out_d, out_label=out_l))
     tflops = 2.0 * q * n * d / t_dist / 1e12
     return {"workload": f"GEMM distance + bits, {n} points x {q} queries, d={d}, k={k}",
@@ -110,6 +111,12 @@ def gemm_knn(bitsknn, torch, dev, q=4096, n=1 << 20, d=64, k=64, runs=5):
             "distance_roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_F32_PEAK_TFLOPS,
                                   "unit": "TFLOP/s", "frac": tflops / MFMA_F32_PEAK_TFLOPS,
                                   "store_GBps": 4.0 * q * n / t_dist / 1e9},
+            "distance_bf16x3": {"arithmetic": "three bf16 pieces per fp32 operand, six bf16 matrix products per "
+                                              "product, fp32 accumulation",
+                                "ms": t_split * 1e3, "pairs_per_s": q * n / t_split,
+                                "roofline": {"bound": "hbm", "achieved": (4.0 * q * n + 4.0 * (q + n) * d) / t_split / 1e9,
+                                             "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                             "frac": (4.0 * q * n + 4.0 * (q + n) * d) / t_split / 1e9 / HBM_PEAK_GBS}},
             "selection_ms": t_topk * 1e3, "selection_elements_per_s": q * n / t_topk,
             "selection_hbm_frac": (4.0 * q * n + 8.0 * q * k) / t_topk / 1e9 / HBM_PEAK_GBS}
 
