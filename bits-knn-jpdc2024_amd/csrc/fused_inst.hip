@@ -13,15 +13,17 @@ namespace bitsknn
 #define BITSKNN_CAT(a, b) a##b
 #define BITSKNN_CAT_EXPANDED(a, b) BITSKNN_CAT2(a, b)
 
-// split: the products of dimensions 9 .. 32 from three bf16 pieces per operand (below 9 the fp32
+// split: the products of dimensions 9 .. 64 from three bf16 pieces per operand (below 9 the fp32
 // matrix instructions are as fast)
 hipError_t BITSKNN_CAT_EXPANDED(launch_fused_k_, BITSKNN_FUSED_K)(const fused_args& a, bool split,
                                                                   hipStream_t stream)
 {
     constexpr int K = BITSKNN_FUSED_K;
-    if (split && a.dim > 8 && a.dim <= 32)
+    if (split && a.dim > 8 && a.dim <= 64)
     {
-        return a.dim <= 16 ? launch_fused<K, 16, true>(a, stream) : launch_fused<K, 32, true>(a, stream);
+        return a.dim <= 16   ? launch_fused<K, 16, true>(a, stream)
+               : a.dim <= 32 ? launch_fused<K, 32, true>(a, stream)
+                             : launch_fused<K, 64, true>(a, stream);
     }
     if (a.dim <= 8)
     {

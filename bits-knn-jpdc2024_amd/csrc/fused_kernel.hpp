@@ -61,7 +61,7 @@ __device__ __forceinline__ float min3(float a, float b, float c)
 // SPLIT = false: fp32 matrix instructions; a stage is (DP + norm rows) x PT floats, PT points per
 // stage so that it stays below 20 KB for DP <= 128.
 //
-// SPLIT = true (DP <= 32): every fp32 value x is cut into three bf16 pieces x = x1 + x2 + x3
+// SPLIT = true (DP <= 64): every fp32 value x is cut into three bf16 pieces x = x1 + x2 + x3
 // (exactly: 8 + 8 + 8 significant bits) and a product x*y is the sum of the bf16 products
 // x3*y1 + x2*y2 + x1*y3 + x2*y1 + x1*y2 + x1*y1 accumulated in fp32 (what is left out is below
 // 2^-23 of the product, the size of one fp32 rounding).  The bf16 matrix path runs at 16 times
@@ -74,7 +74,7 @@ struct fused_geometry
     static constexpr int DK = DP < 16 ? 16 : DP;       // SPLIT: dimensions padded to whole matrix steps
     static constexpr int KB = DK / 16;                 // SPLIT: matrix steps of 16 dimensions
     static constexpr int KS = DK / 8;                  // SPLIT: cells of 8 dimensions per point and piece
-    static constexpr int PT = SPLIT ? (DK <= 16 ? 128 : 64)
+    static constexpr int PT = SPLIT ? (DK <= 16 ? 128 : (DK <= 32 ? 64 : 32))
                                     : (DP <= 16 ? 256 : (DP <= 32 ? 128 : (DP <= 64 ? 64 : 32)));
     static constexpr int TPP = FQ_THREADS / PT; // threads per point when staging
     // point rows (zero beyond dim), then one row per staging thread of a point with its share of
@@ -85,7 +85,7 @@ struct fused_geometry
     static constexpr int VPT = SPLIT ? 8 : DP / TPP; // values a thread carries from global memory to LDS
     static constexpr int MT = PT / 32;        // MFMA row tiles per stage
     static constexpr int STAGE_FLOATS = SPLIT ? 3 * KS * PT * 4 + PT : ROWS * PT;
-    static_assert(!SPLIT || (DP <= 32 && TPP == KS), "one staging thread per point and cell");
+    static_assert(!SPLIT || (DP <= 64 && TPP == KS), "one staging thread per point and cell");
     static constexpr size_t lds_bytes()
     {
         // two stages (one being multiplied, one being filled), the query buffers, exchange slots
@@ -484,9 +484,13 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             }
             // the threads of a point are TPP neighbouring lanes
             share += __builtin_bit_cast(float, lane_xor32<1>(__builtin_bit_cast(u32, share)));
-            if constexpr (TPP == 4)
+            if constexpr (TPP >= 4)
             {
                 share += __builtin_bit_cast(float, lane_xor32<2>(__builtin_bit_cast(u32, share)));
+            }
+            if constexpr (TPP == 8)
+            {
+                share += __builtin_bit_cast(float, lane_xor32<4>(__builtin_bit_cast(u32, share)));
             }
             // points beyond the end get an infinite distance and never pass the filter
             stage[3 * KS * PT * 4 + sp] = base + sp < n ? share : __builtin_inff();
@@ -565,6 +569,43 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 filter_tile(acc0, base + p * 64);
                 filter_tile(acc1, base + p * 64 + 32);
             });
+            if constexpr (MT == 1)
+            {
+                // 64 dimensions: a stage is one tile
+                vuint4 af[3][KB];
+#pragma unroll
+                for (int c = 0; c < 3; ++c)
+                {
+#pragma unroll
+                    for (int kb = 0; kb < KB; ++kb)
+                    {
+                        af[c][kb] = cells[(c * KS + 2 * kb + half) * PT + ql];
+                    }
+                }
+                vfloat16 acc;
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                {
+                    const vfloat4 x = *reinterpret_cast<const vfloat4*>(norm_row + 4 * half + 8 * g);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                    {
+                        acc[4 * g + e] = x[e];
+                    }
+                }
+                constexpr int order[6][2] = {{2, 0}, {1, 1}, {0, 2}, {1, 0}, {0, 1}, {0, 0}};
+                static_for<0, KB>([&](auto kb_tag) {
+                    constexpr int kb = decltype(kb_tag)::value;
+                    static_for<0, 6>([&](auto o_tag) {
+                        constexpr int ca = order[decltype(o_tag)::value][0];
+                        constexpr int cb = order[decltype(o_tag)::value][1];
+                        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(vbf16x8, af[ca][kb]), __builtin_bit_cast(vbf16x8, qs[cb][kb]), acc, 0,
+                            0, 0);
+                    });
+                });
+                filter_tile(acc, base);
+            }
         }
         else if constexpr (MT >= 2)
         {

@@ -142,14 +142,14 @@ int bitsknn_fused_l2_topk_f32(const float* queries_dim_major, const float* point
                               int dim_mult, void* stream);
 
 /*
- * Arithmetic of the products q.p inside the bits-fused kernels for dim <= 32 (process-wide, read
+ * Arithmetic of the products q.p inside the bits-fused kernels for 9 <= dim <= 64 (process-wide, read
  * at every call):
  *   BITSKNN_FUSED_FP32    fp32 matrix instructions (v_mfma_f32_32x32x2_f32).
  *   BITSKNN_FUSED_BF16X3  every fp32 operand is cut exactly into three bf16 pieces and a product
  *                         is the fp32 sum of six bf16 products on the bf16 matrix path
  *                         (v_mfma_f32_32x32x16_bf16); what is left out is below 2^-23 of a
  *                         product, the size of one fp32 rounding.
- * Larger dimensions always use BITSKNN_FUSED_FP32.  No counterpart in the reference, whose fused
+ * Other dimensions always use BITSKNN_FUSED_FP32.  No counterpart in the reference, whose fused
  * kernel multiplies on the fp32 vector unit (fused_cache_kernel_structs.cuh:457-522).
  * bitsknn_fused_set_arithmetic returns BITSKNN_ERR_INVALID for another value.
  */

@@ -259,7 +259,7 @@ def test_random_shapes_against_the_oracle(bk, dev, oracle):
             raise AssertionError((case, n, q, d, k, kind)) from e
 
 
-# ---- products from three bf16 pieces per operand (BITSKNN_FUSED_BF16X3, dimensions 9 .. 32) --------
+# ---- products from three bf16 pieces per operand (BITSKNN_FUSED_BF16X3, dimensions 9 .. 64) --------
 
 @pytest.fixture
 def bf16x3(bk):
@@ -270,7 +270,7 @@ def bf16x3(bk):
 
 
 @pytest.mark.parametrize("k", [4, 8, 16, 32, 64, 128, 256])
-@pytest.mark.parametrize("d", [9, 16, 17, 32])
+@pytest.mark.parametrize("d", [9, 16, 17, 32, 33, 64])
 def test_bf16x3_all_k_values(bk, dev, oracle, bf16x3, k, d):
     p, s = oracle.generate(200 + k + d, 20000, 150, d)
     gd, gl = _fused(bk, dev, p, s, k)
@@ -279,7 +279,7 @@ def test_bf16x3_all_k_values(bk, dev, oracle, bf16x3, k, d):
 
 @pytest.mark.parametrize("n,q", [(1, 1), (31, 5), (32, 33), (63, 127), (64, 128), (65, 129), (129, 3), (1000, 300), (5001, 1)])
 def test_bf16x3_ragged_counts(bk, dev, oracle, bf16x3, n, q):
-    for d in (12, 31):
+    for d in (12, 31, 50):
         p, s = oracle.generate(n + q + d, n, q, d)
         for k in (4, 32):
             gd, gl = _fused(bk, dev, p, s, k, (2, 4, 1), 1, 1)
@@ -287,7 +287,7 @@ def test_bf16x3_ragged_counts(bk, dev, oracle, bf16x3, n, q):
 
 
 @pytest.mark.parametrize("n,q,d,k", [(20000, 150, 12, 32), (70001, 300, 16, 16), (300000, 33, 32, 4),
-                                     (9000, 1000, 24, 64)])
+                                     (9000, 1000, 24, 64), (30000, 100, 64, 32)])
 def test_bf16x3_point_split_variant_with_workspace(bk, dev, oracle, bf16x3, n, q, d, k):
     p, s = oracle.generate(n + q + d, n, q, d)
     gd, gl = _fused(bk, dev, p, s, k, workspace="auto")
@@ -300,7 +300,7 @@ def test_bf16x3_random_shapes_against_the_oracle(bk, dev, oracle, bf16x3):
     import torch
     rng = np.random.default_rng(99)
     for case in range(30):
-        d = int(rng.integers(9, 33))
+        d = int(rng.integers(9, 65))
         k = int(rng.choice([4, 8, 16, 32, 64, 128, 256]))
         n = int(rng.choice([rng.integers(1, 300), rng.integers(300, 5000), rng.integers(5000, 30000)]))
         q = int(rng.choice([rng.integers(1, 40), rng.integers(40, 300), rng.integers(300, 600)]))
@@ -319,7 +319,7 @@ def test_bf16x3_is_as_accurate_as_the_fp32_matrix_instructions(bk, dev, oracle):
     the level of fp32 rounding (far inside the 1e-5 bar) and within a small factor of the fp32
     matrix instructions' own error."""
     err = {}
-    for d in (16, 32):
+    for d in (16, 32, 64):
         p, s = oracle.generate(900 + d, 30000, 200, d)
         truth = oracle.dist(s, p, "f64-partial")
         qn = (s.astype(np.float64) ** 2).sum(1)[:, None]
