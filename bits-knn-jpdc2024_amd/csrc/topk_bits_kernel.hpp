@@ -152,15 +152,17 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     const u32 full_end =
         n > static_cast<u32>(NL) ? static_cast<u32>(NL) + ((n - static_cast<u32>(NL)) / CHUNK) * CHUNK
                                  : static_cast<u32>(NL);
-    // The chunks after the first NL values are visited from both ends of the row inwards
-    // (first, last, second, last but one, ...): whichever end of a sorted row holds the small
-    // values, the radius is tight after two chunks, where a front-to-back pass over a descending
-    // row would let every value through the filter.  The result does not depend on the order.
+    // The chunks after the first NL values are visited from both ends of the row inwards, the
+    // back first (last, first, last but one, second, ...): whichever end of a sorted row holds the
+    // small values, the radius is tight after the first NL values (ascending rows) or after the
+    // last chunk (descending rows), where a front-to-back pass over a descending row would let
+    // every value through the filter.  The result does not depend on the order.
     const u32 chunk_count = n > static_cast<u32>(NL) ? (n - static_cast<u32>(NL) + CHUNK - 1) / CHUNK : 0;
     u32 left = chunk_count;            // chunks not yet visited
-    u32 chunk = NL;                    // the next chunk to visit
-    // distance to the chunk after it: alternating in sign and shrinking by one chunk per visit
-    std::int32_t jump = chunk_count > 0 ? static_cast<std::int32_t>((chunk_count - 1) * CHUNK) : 0;
+    // distance from the chunk being visited to the next one: alternating in sign and shrinking by
+    // one chunk per visit
+    std::int32_t jump = chunk_count > 0 ? -static_cast<std::int32_t>((chunk_count - 1) * CHUNK) : 0;
+    u32 chunk = static_cast<u32>(NL) + static_cast<u32>(-jump); // the next chunk to visit
 
     // the first NL values go straight to the buffer: column c into slot c
 #pragma unroll
