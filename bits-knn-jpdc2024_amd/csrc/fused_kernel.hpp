@@ -120,6 +120,10 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     constexpr int LPQ = S / R;
     constexpr int QPP = WAVE / LPQ;           // queries per merge pass
     constexpr int PASSES = FQ_QW / QPP;
+    // Whether the waves of a workgroup merge together (below): pays for the long merges of long
+    // lists (k = 256: 65 -> 52 ms); for k <= 32 the two looks at the flag per stage cost more (1 %
+    // each) than the short merges they overlap.
+    constexpr bool JOIN_MERGES = K > FQ_CAP;
 
     extern __shared__ float lds[];
     constexpr int STAGE_FLOATS = G::STAGE_FLOATS;
@@ -352,7 +356,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         {
             // the other waves of the workgroup would wait for this wave at the stage barrier:
             // they are asked to merge their buffers in the meantime
-            if (lane == 0)
+            if (JOIN_MERGES && lane == 0)
             {
                 __hip_atomic_store(merge_wanted + stage_slot, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
@@ -759,14 +763,21 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 fetch(base + 2 * PT);
             }
         }
-        merge_if_wanted();
-        __syncthreads();
-        merge_if_wanted();
-        if (t == 0)
+        if constexpr (JOIN_MERGES)
         {
-            merge_wanted[(stage_slot + 2) % 3] = 0;
+            merge_if_wanted();
+            __syncthreads();
+            merge_if_wanted();
+            if (t == 0)
+            {
+                merge_wanted[(stage_slot + 2) % 3] = 0;
+            }
+            stage_slot = stage_slot == 2 ? 0 : stage_slot + 1;
         }
-        stage_slot = stage_slot == 2 ? 0 : stage_slot + 1;
+        else
+        {
+            __syncthreads();
+        }
     }
 
     // whatever is left in the buffers; also writes the lists of queries that never merged
