@@ -161,8 +161,13 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     u32 left = chunk_count;            // chunks not yet visited
     // distance from the chunk being visited to the next one: alternating in sign and shrinking by
     // one chunk per visit
-    std::int32_t jump = chunk_count > 0 ? -static_cast<std::int32_t>((chunk_count - 1) * CHUNK) : 0;
-    u32 chunk = static_cast<u32>(NL) + static_cast<u32>(-jump); // the next chunk to visit
+    // (Lists of 512 entries and more start at the front instead -- first, last, second, ... --:
+    // measured on uniform rows of 2^20 values they lose 0.4 % at k = 512 and 1.5 % at k = 2048 of
+    // the HBM roofline with the back first, more than a merge per sorted row is worth there.)
+    constexpr bool BACK_FIRST = NL < 512;
+    const std::int32_t span = chunk_count > 0 ? static_cast<std::int32_t>((chunk_count - 1) * CHUNK) : 0;
+    std::int32_t jump = BACK_FIRST ? -span : span;
+    u32 chunk = static_cast<u32>(NL) + (BACK_FIRST ? static_cast<u32>(span) : 0U); // the next chunk to visit
 
     // the first NL values go straight to the buffer: column c into slot c
 #pragma unroll
