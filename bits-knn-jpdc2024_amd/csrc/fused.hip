@@ -12,7 +12,7 @@ namespace bitsknn
 namespace
 {
 
-// arithmetic of the products for d <= 32 (bitsknn_fused_set_arithmetic)
+// arithmetic of the products for 9 <= d <= 64 (bitsknn_fused_set_arithmetic)
 std::atomic<int> g_arithmetic{BITSKNN_FUSED_FP32};
 
 bool in_list(int v, std::initializer_list<int> values)
@@ -26,14 +26,6 @@ bool in_list(int v, std::initializer_list<int> values)
     }
     return false;
 }
-
-} // namespace
-} // namespace bitsknn
-
-namespace bitsknn
-{
-namespace
-{
 
 // Number of point ranges for a problem: enough workgroups for two per compute unit, ranges of at
 // least 4096 points and a multiple of 256, at most 64 ranges.
