@@ -105,12 +105,14 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     constexpr int E = 4 * L;         // values per thread and iteration
     constexpr u32 CHUNK = BS * E;    // values per workgroup and iteration
     static_assert(E <= 32, "one pass bit per value in a 32-bit lane mask");
+    constexpr u32 SAMPLE_PAIRS = 2;  // pieces per thread and end of the row that the sample looks at
 
     __shared__ u64 buffer[2 * NL];   // candidates; the second half is exchange space of the merges
     __shared__ u64 s_radius;
     __shared__ int s_fill[W];
     __shared__ int s_flag;  // some wave wants a merge
     __shared__ int s_more;  // some wave still has values to process after this merge
+    __shared__ u32 s_sample[W];
 
     const int t = static_cast<int>(threadIdx.x);
     const int lane = t & (WAVE - 1);
@@ -169,6 +171,46 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     std::int32_t jump = BACK_FIRST ? -span : span;
     u32 chunk = static_cast<u32>(NL) + (BACK_FIRST ? static_cast<u32>(span) : 0U); // the next chunk to visit
 
+    // ---- radius from a sample.  Every thread looks at up to SAMPLE_PAIRS pairs of 16-byte pieces
+    // of the row, one at its front and one at its back (at most a sixteenth of the row in all), and
+    // keeps its two smallest values; every wave takes the c-th smallest of its 128, c = ceil(k / W).
+    // At least k values of the row are then not above the largest of these W values, so nothing
+    // above it can belong to the result: it serves as radius until the list itself has a smaller
+    // one.  This replaces the first merges of a row, which each only halve the radius and which
+    // all rows of a launch do at the same time.
+    if constexpr (VEC)
+    {
+        const u32 c = (a.k + W - 1) / W;
+        const u32 fit = n / (128U * BS);
+        const u32 pairs = fit < SAMPLE_PAIRS ? fit : SAMPLE_PAIRS;
+        u32 wave_bound = 0xFFFFFFFFU;
+        if (c <= 2 * WAVE && pairs > 0)
+        {
+            const u32 back = (n - pairs * 4 * BS) & ~3U;
+            float lo = __builtin_inff();
+            float lo2 = __builtin_inff();
+            for (u32 p = 0; p < pairs; ++p)
+            {
+                const u32 col = (p * BS + static_cast<u32>(t)) * 4;
+                const vfloat4 x[2] = {*reinterpret_cast<const vfloat4*>(row + col),
+                                      *reinterpret_cast<const vfloat4*>(row + back + col)};
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                {
+                    const float value = fminf(x[i / 4][i % 4], __builtin_inff()); // NaN -> +inf
+                    lo2 = __builtin_amdgcn_fmed3f(value, lo, lo2);
+                    lo = fminf(value, lo);
+                }
+            }
+            u64 two[2] = {static_cast<u64>(float_key(lo)) << 32U, static_cast<u64>(float_key(lo2)) << 32U};
+            net_sort<WAVE, 2, 2, false>(two, nullptr, lane);
+            const u32 pick = static_cast<u32>(((c - 1) & 1U) != 0 ? two[1] >> 32U : two[0] >> 32U);
+            wave_bound = static_cast<u32>(
+                __builtin_amdgcn_readlane(static_cast<int>(pick), static_cast<int>((c - 1) >> 1U)));
+        }
+        s_sample[wave] = wave_bound;
+    }
+
     // the first NL values go straight to the buffer: column c into slot c
 #pragma unroll
     for (int r = 0; r < IPT; ++r)
@@ -188,6 +230,21 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
 
     float radius = __builtin_inff();
     u64 radius_key = PAD_KEY;
+    if constexpr (VEC)
+    {
+        u32 bound = 0;
+#pragma unroll
+        for (int w = 0; w < W; ++w)
+        {
+            bound = s_sample[w] > bound ? s_sample[w] : bound;
+        }
+        // values up to the bound pass: the radius is the next key after it with the lowest label
+        if (bound < float_key(__builtin_inff()))
+        {
+            radius_key = static_cast<u64>(bound + 1) << 32U;
+            radius = key_float(bound + 1);
+        }
+    }
     u32 cur_chunk = 0; // first column of the chunk held in v[]
 
     float v[E];
@@ -311,22 +368,24 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
         // ---- rendezvous: every wave arrives here when it needs a merge, saw the flag, or ran
         // out of values
         const bool more_work = pending || left > 0;
-        if (lane == 0)
+        // (wave-uniform values, stored by every lane: a branch on the lane next to a loop exit
+        // makes the compiler treat the loop state as differing between lanes, which turns the
+        // streaming loop into an exec-masked one with its counters in vector registers)
+        s_fill[wave] = fill;
+        if (more_work)
         {
-            s_fill[wave] = fill;
-            if (more_work)
-            {
-                s_more = 1;
-            }
+            s_more = 1;
         }
         __syncthreads();
+        // (the same in every lane; said explicitly so that the loops stay wave-uniform)
         int total = 0;
 #pragma unroll
         for (int w = 0; w < W; ++w)
         {
             total += s_fill[w];
         }
-        const bool more = s_more != 0;
+        total = __builtin_amdgcn_readfirstlane(total);
+        const bool more = __builtin_amdgcn_readfirstlane(s_more) != 0;
         if (total > 0)
         {
             merge_buffer<BS, IPT>(topk, buffer, s_fill, t);
@@ -337,7 +396,9 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
                 s_flag = 0;
                 s_more = 0;
             }
-            radius_key = broadcast_radius<IPT>(topk, a.k, &s_radius, t);
+            // (the radius from the sample stays until the list has a smaller one)
+            const u64 list_radius = broadcast_radius<IPT>(topk, a.k, &s_radius, t);
+            radius_key = list_radius < radius_key ? list_radius : radius_key;
             radius = key_value(radius_key);
         }
         else
@@ -362,10 +423,7 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
             if (end > CAP)
             {
                 fill = CAP;
-                if (lane == 0)
-                {
-                    s_flag = 1;
-                }
+                s_flag = 1;
                 continue;
             }
             fill = end;
@@ -388,7 +446,7 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
             {
                 load_chunk(v, chunk);
             }
-            const int flag = *static_cast<volatile int*>(&s_flag);
+            const int flag = __hip_atomic_load(&s_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             cur_chunk = chunk;
             left -= 1;
             chunk += static_cast<u32>(jump);
@@ -450,10 +508,7 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
                     slot_base = fill;
                     pending = true;
                     fill = CAP;
-                    if (lane == 0)
-                    {
-                        s_flag = 1;
-                    }
+                    s_flag = 1;
                     break;
                 }
                 fill = running;

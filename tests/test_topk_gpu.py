@@ -91,6 +91,43 @@ def test_hard_inputs(bk, dev, oracle, kind, k):
         _check(bk, dev, oracle, m, k, block=block, batch=16)
 
 
+def test_rows_long_enough_for_the_sampled_radius(bk, dev, oracle):
+    """Rows of at least 128 x block size values start from a radius that the kernel takes from a
+    sample of both ends of the row; the result must not depend on it."""
+    rng = np.random.default_rng(5)
+    rows, cols = 7, 70000
+    m = oracle.uniform_matrix(321, rows, cols, -3.0, 3.0)
+    m[0, :3000] = np.inf                      # nothing finite in the sampled parts
+    m[0, -3000:] = np.inf
+    m[1, :] = np.inf                          # fewer finite values than k, none of them sampled
+    m[1, 30000:30040] = rng.random(40, dtype=np.float32)
+    m[2, :4096] = -7.0                        # more equal values than k inside the sample
+    m[3, 20000:20300] = -7.0                  # the smallest values tie and lie outside the sample
+    m[4] = np.round(m[4] * 8) / 8             # few distinct values
+    m[5, :2048] = np.sort(m[5, :2048])        # sampled parts sorted towards the middle
+    m[5, -2048:] = np.sort(m[5, -2048:])[::-1]
+    m[6, 1::2] = -0.0                         # both zeros, everywhere
+    m[6, 0::2] = 0.0
+    for block in (128, 256, 512):
+        for k in (1, 5, 100, 127, 128, 129, 256, 257, 512, 1024):
+            if k // block > 16:
+                continue
+            gd, gl = _run(bk, dev, m, k, block=block, batch=8)
+            ed, el = oracle.topk(m, k)
+            assert np.array_equal(gd, ed) and np.array_equal(gl, el), (block, k)
+    # explicit labels with the extreme values on tied entries, and label offsets
+    labels = np.stack([rng.permutation(cols) for _ in range(rows)]).astype(np.int32)
+    labels[4, :4] = [np.iinfo(np.int32).max, np.iinfo(np.int32).min, -1, 0]
+    offsets = (np.arange(rows) * 1000003).astype(np.int32)
+    short, short_labels = np.ascontiguousarray(m[:, :66000]), np.ascontiguousarray(labels[:, :66000])
+    for matrix, k, block, batch, lab, off in ((short, 300, 128, 8, short_labels, None),
+                                              (m, 64, 256, 4, None, offsets),
+                                              (m, 512, 512, 3, labels, offsets)):
+        gd, gl = _run(bk, dev, matrix, k, block=block, batch=batch, labels=lab, offsets=off)
+        ed, el = oracle.topk(matrix, k, labels=lab, label_offsets=off)
+        assert np.array_equal(gd, ed) and np.array_equal(gl, el), (k, block)
+
+
 def test_negative_values_and_infinities(bk, dev, oracle):
     m = oracle.uniform_matrix(3, 4, 20000, -5.0, 5.0)
     m[0, 17] = -np.inf
