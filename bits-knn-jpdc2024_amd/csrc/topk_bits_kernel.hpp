@@ -19,7 +19,9 @@
 //    go through LDS (two alternating regions, one barrier per exchange);
 //  * the chunks of a row are visited from both ends inwards, so that sorted rows of either
 //    direction tighten the radius at once, and for small batches the next chunk is requested
-//    before the current one is filtered.
+//    before the current one is filtered;
+//  * long rows start from a radius taken from a sample of both row ends instead of from +inf,
+//    which saves the first merges (they only halve the radius each).
 // Because waves drift apart, the filter compares full keys when a value equals the radius, so
 // that "equal values by lower label" holds no matter which wave saw which value first.
 
