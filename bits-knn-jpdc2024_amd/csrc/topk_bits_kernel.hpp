@@ -18,8 +18,8 @@
 //  * exchange distances below 64 lanes stay inside a wave, only distances of 64 lanes and more
 //    go through LDS (two alternating regions, one barrier per exchange);
 //  * the chunks of a row are visited from both ends inwards, so that sorted rows of either
-//    direction tighten the radius at once, and for small batches the next chunk is requested
-//    before the current one is filtered;
+//    direction tighten the radius at once, and for up to 16 values per thread the next chunk
+//    is requested before the current one is filtered;
 //  * long rows start from a radius taken from a sample of both row ends instead of from +inf,
 //    which saves the first merges (they only halve the radius each).
 // Because waves drift apart, the filter compares full keys when a value equals the radius, so
@@ -293,9 +293,9 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
             }
         }
     };
-    // Software pipelining for small batches: the next chunk is requested before the current one
+    // Software pipelining for up to 4 loads per thread: the next chunk is requested before the current one
     // is filtered, at the price of E more registers and E moves per chunk.
-    constexpr bool PIPE = L <= 2;
+    constexpr bool PIPE = L <= 4;
     float ahead[E];
 #pragma unroll
     for (int j = 0; j < E; ++j)
