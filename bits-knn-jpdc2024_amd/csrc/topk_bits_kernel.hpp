@@ -18,8 +18,8 @@
 //  * exchange distances below 64 lanes stay inside a wave, only distances of 64 lanes and more
 //    go through LDS (two alternating regions, one barrier per exchange);
 //  * the chunks of a row are visited from both ends inwards, so that sorted rows of either
-//    direction tighten the radius at once, and for up to 16 values per thread the next chunk
-//    is requested before the current one is filtered;
+//    direction tighten the radius at once, and for small batches the next chunk is requested
+//    before the current one is filtered;
 //  * long rows start from a radius taken from a sample of both row ends instead of from +inf,
 //    which saves the first merges (they only halve the radius each).
 // Because waves drift apart, the filter compares full keys when a value equals the radius, so
@@ -107,7 +107,11 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     constexpr int E = 4 * L;         // values per thread and iteration
     constexpr u32 CHUNK = BS * E;    // values per workgroup and iteration
     static_assert(E <= 32, "one pass bit per value in a 32-bit lane mask");
-    constexpr u32 SAMPLE_PAIRS = 2;  // pieces per thread and end of the row that the sample looks at
+    // The sample that gives the first radius: smallest values kept per thread (the wave's pick
+    // should not lie above the middle of what its lanes keep, and a wave picks up to 64 * IPT),
+    // and 16-byte pieces per thread and end of the row (4 values looked at per value kept).
+    constexpr int SAMPLE_KEEP = IPT <= 1 ? 2 : (IPT == 2 ? 4 : 8);
+    constexpr u32 SAMPLE_PAIRS = SAMPLE_KEEP;
 
     __shared__ u64 buffer[2 * NL];   // candidates; the second half is exchange space of the merges
     __shared__ u64 s_radius;
@@ -175,22 +179,26 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
 
     // ---- radius from a sample.  Every thread looks at up to SAMPLE_PAIRS pairs of 16-byte pieces
     // of the row, one at its front and one at its back (at most a sixteenth of the row in all), and
-    // keeps its two smallest values; every wave takes the c-th smallest of its 128, c = ceil(k / W).
-    // At least k values of the row are then not above the largest of these W values, so nothing
-    // above it can belong to the result: it serves as radius until the list itself has a smaller
-    // one.  This replaces the first merges of a row, which each only halve the radius and which
-    // all rows of a launch do at the same time.
+    // keeps its SAMPLE_KEEP smallest values; every wave takes the c-th smallest of its
+    // 64 * SAMPLE_KEEP, c = ceil(k / W).  At least k values of the row are then not above the
+    // largest of these W values, so nothing above it can belong to the result: it serves as
+    // radius until the list itself has a smaller one.  This replaces the first merges of a row,
+    // which each only halve the radius and which all rows of a launch do at the same time.
     if constexpr (VEC)
     {
         const u32 c = (a.k + W - 1) / W;
         const u32 fit = n / (128U * BS);
         const u32 pairs = fit < SAMPLE_PAIRS ? fit : SAMPLE_PAIRS;
         u32 wave_bound = 0xFFFFFFFFU;
-        if (c <= 2 * WAVE && pairs > 0)
+        if (c <= WAVE * SAMPLE_KEEP && pairs > 0)
         {
             const u32 back = (n - pairs * 4 * BS) & ~3U;
-            float lo = __builtin_inff();
-            float lo2 = __builtin_inff();
+            float lo[SAMPLE_KEEP]; // ascending
+#pragma unroll
+            for (int j = 0; j < SAMPLE_KEEP; ++j)
+            {
+                lo[j] = __builtin_inff();
+            }
             for (u32 p = 0; p < pairs; ++p)
             {
                 const u32 col = (p * BS + static_cast<u32>(t)) * 4;
@@ -200,15 +208,30 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
                 for (int i = 0; i < 8; ++i)
                 {
                     const float value = fminf(x[i / 4][i % 4], __builtin_inff()); // NaN -> +inf
-                    lo2 = __builtin_amdgcn_fmed3f(value, lo, lo2);
-                    lo = fminf(value, lo);
+#pragma unroll
+                    for (int j = SAMPLE_KEEP - 1; j > 0; --j)
+                    {
+                        lo[j] = __builtin_amdgcn_fmed3f(value, lo[j - 1], lo[j]);
+                    }
+                    lo[0] = fminf(value, lo[0]);
                 }
             }
-            u64 two[2] = {static_cast<u64>(float_key(lo)) << 32U, static_cast<u64>(float_key(lo2)) << 32U};
-            net_sort<WAVE, 2, 2, false>(two, nullptr, lane);
-            const u32 pick = static_cast<u32>(((c - 1) & 1U) != 0 ? two[1] >> 32U : two[0] >> 32U);
-            wave_bound = static_cast<u32>(
-                __builtin_amdgcn_readlane(static_cast<int>(pick), static_cast<int>((c - 1) >> 1U)));
+            u64 keys[SAMPLE_KEEP];
+#pragma unroll
+            for (int j = 0; j < SAMPLE_KEEP; ++j)
+            {
+                keys[j] = static_cast<u64>(float_key(lo[j])) << 32U;
+            }
+            net_sort<WAVE, SAMPLE_KEEP, 2, false>(keys, nullptr, lane);
+            // sorted position c - 1 is entry (c - 1) % SAMPLE_KEEP of lane (c - 1) / SAMPLE_KEEP
+            u32 pick = 0;
+#pragma unroll
+            for (int j = 0; j < SAMPLE_KEEP; ++j)
+            {
+                pick = (c - 1) % SAMPLE_KEEP == static_cast<u32>(j) ? static_cast<u32>(keys[j] >> 32U) : pick;
+            }
+            wave_bound = static_cast<u32>(__builtin_amdgcn_readlane(
+                static_cast<int>(pick), static_cast<int>((c - 1) / SAMPLE_KEEP)));
         }
         s_sample[wave] = wave_bound;
     }
@@ -293,9 +316,9 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
             }
         }
     };
-    // Software pipelining for up to 4 loads per thread: the next chunk is requested before the current one
+    // Software pipelining for small batches: the next chunk is requested before the current one
     // is filtered, at the price of E more registers and E moves per chunk.
-    constexpr bool PIPE = L <= 4;
+    constexpr bool PIPE = L <= 2;
     float ahead[E];
 #pragma unroll
     for (int j = 0; j < E; ++j)
