@@ -156,27 +156,6 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
         topk[r] = PAD_KEY;
     }
 
-    const u32 first = n < static_cast<u32>(NL) ? n : static_cast<u32>(NL);
-    const u32 full_end =
-        n > static_cast<u32>(NL) ? static_cast<u32>(NL) + ((n - static_cast<u32>(NL)) / CHUNK) * CHUNK
-                                 : static_cast<u32>(NL);
-    // The chunks after the first NL values are visited from both ends of the row inwards, the
-    // back first (last, first, last but one, second, ...): whichever end of a sorted row holds the
-    // small values, the radius is tight after the first NL values (ascending rows) or after the
-    // last chunk (descending rows), where a front-to-back pass over a descending row would let
-    // every value through the filter.  The result does not depend on the order.
-    const u32 chunk_count = n > static_cast<u32>(NL) ? (n - static_cast<u32>(NL) + CHUNK - 1) / CHUNK : 0;
-    u32 left = chunk_count;            // chunks not yet visited
-    // distance from the chunk being visited to the next one: alternating in sign and shrinking by
-    // one chunk per visit
-    // (Lists of 512 entries and more start at the front instead -- first, last, second, ... --:
-    // measured on uniform rows of 2^20 values they lose 0.4 % at k = 512 and 1.5 % at k = 2048 of
-    // the HBM roofline with the back first, more than a merge per sorted row is worth there.)
-    constexpr bool BACK_FIRST = NL < 512;
-    const std::int32_t span = chunk_count > 0 ? static_cast<std::int32_t>((chunk_count - 1) * CHUNK) : 0;
-    std::int32_t jump = BACK_FIRST ? -span : span;
-    u32 chunk = static_cast<u32>(NL) + (BACK_FIRST ? static_cast<u32>(span) : 0U); // the next chunk to visit
-
     // ---- radius from a sample.  Every thread looks at up to SAMPLE_PAIRS pairs of 16-byte pieces
     // of the row, one at its front and one at its back (at most a sixteenth of the row in all), and
     // keeps its SAMPLE_KEEP smallest values; every wave takes the c-th smallest of its
@@ -236,16 +215,6 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
         s_sample[wave] = wave_bound;
     }
 
-    // the first NL values go straight to the buffer: column c into slot c
-#pragma unroll
-    for (int r = 0; r < IPT; ++r)
-    {
-        const u32 col = static_cast<u32>(r * BS + t);
-        if (col < first)
-        {
-            buffer[col] = make_key(row[col], label_of(col));
-        }
-    }
     if (t == 0)
     {
         s_flag = 0;
@@ -255,6 +224,7 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
 
     float radius = __builtin_inff();
     u64 radius_key = PAD_KEY;
+    bool sampled = false;
     if constexpr (VEC)
     {
         u32 bound = 0;
@@ -264,10 +234,47 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
             bound = s_sample[w] > bound ? s_sample[w] : bound;
         }
         // values up to the bound pass: the radius is the next key after it with the lowest label
+        bound = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(bound)));
         if (bound < float_key(__builtin_inff()))
         {
             radius_key = static_cast<u64>(bound + 1) << 32U;
             radius = key_float(bound + 1);
+            sampled = true;
+        }
+    }
+
+    // Without a radius from the sample the first NL values go straight to the buffer and the
+    // first merge sorts them; with one, they are filtered like the rest of the row (`head` = 0),
+    // which saves that merge.
+    const u32 head = sampled ? 0U : static_cast<u32>(NL);
+    const u32 first = n < head ? n : head;
+    const u32 full_end = n > head ? head + ((n - head) / CHUNK) * CHUNK : head;
+    // The chunks after the head are visited from both ends of the row inwards, the
+    // back first (last, first, last but one, second, ...): whichever end of a sorted row holds the
+    // small values, the radius is tight after the first NL values (ascending rows) or after the
+    // last chunk (descending rows), where a front-to-back pass over a descending row would let
+    // every value through the filter.  The result does not depend on the order.
+    const u32 chunk_count = n > head ? (n - head + CHUNK - 1) / CHUNK : 0;
+    u32 left = chunk_count;            // chunks not yet visited
+    // distance from the chunk being visited to the next one: alternating in sign and shrinking by
+    // one chunk per visit
+    // (Lists of 512 entries and more start at the front instead -- first, last, second, ... --:
+    // measured on uniform rows of 2^20 values they lose 0.4 % at k = 512 and 1.5 % at k = 2048 of
+    // the HBM roofline with the back first, more than a merge per sorted row is worth there.)
+    constexpr bool BACK_FIRST = NL < 512;
+    const std::int32_t span = chunk_count > 0 ? static_cast<std::int32_t>((chunk_count - 1) * CHUNK) : 0;
+    std::int32_t jump = BACK_FIRST ? -span : span;
+    u32 chunk = head + (BACK_FIRST ? static_cast<u32>(span) : 0U); // the next chunk to visit
+
+    // the head goes straight to the buffer: column c into slot c (the barrier at the top of the
+    // main loop orders these writes before the merge that reads them)
+#pragma unroll
+    for (int r = 0; r < IPT; ++r)
+    {
+        const u32 col = static_cast<u32>(r * BS + t);
+        if (col < first)
+        {
+            buffer[col] = make_key(row[col], label_of(col));
         }
     }
     u32 cur_chunk = 0; // first column of the chunk held in v[]
