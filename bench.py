@@ -34,7 +34,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 matrix peak
 # HBM bytes per launch of the top-k kernel from two counter passes (FETCH_SIZE, WRITE_SIZE, each
 # scaled by what the counter reads for a plain 1 GiB copy), keyed by (rows, cols, k).  Measured
 # under a profiler, so it cannot be taken live; other workloads report null.
-MEASURED_TRAFFIC_BYTES = {(1024, 1 << 20, 32): 4295307731}
+MEASURED_TRAFFIC_BYTES = {(1024, 1 << 20, 32): 4295326899}
 
 
 def fused_headline(bitsknn, torch, dev, q=65536, n=1 << 20, d=32, k=32, runs=3):
