@@ -95,7 +95,7 @@ def test_rows_long_enough_for_the_sampled_radius(bk, dev, oracle):
     """Rows of at least 128 x block size values start from a radius that the kernel takes from a
     sample of both ends of the row; the result must not depend on it."""
     rng = np.random.default_rng(5)
-    rows, cols = 7, 70000
+    rows, cols = 8, 70000
     m = oracle.uniform_matrix(321, rows, cols, -3.0, 3.0)
     m[0, :3000] = np.inf                      # nothing finite in the sampled parts
     m[0, -3000:] = np.inf
@@ -108,6 +108,7 @@ def test_rows_long_enough_for_the_sampled_radius(bk, dev, oracle):
     m[5, -2048:] = np.sort(m[5, -2048:])[::-1]
     m[6, 1::2] = -0.0                         # both zeros, everywhere
     m[6, 0::2] = 0.0
+    m[7] = (rng.permutation(cols).astype(np.uint32) + 1).view(np.float32)  # subnormal values only
     for block in (128, 256, 512):
         for k in (1, 5, 100, 127, 128, 129, 256, 257, 512, 1024):
             if k // block > 16:
