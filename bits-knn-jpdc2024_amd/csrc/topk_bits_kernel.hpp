@@ -163,7 +163,6 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     // largest of these W values, so nothing above it can belong to the result: it serves as
     // radius until the list itself has a smaller one.  This replaces the first merges of a row,
     // which each only halve the radius and which all rows of a launch do at the same time.
-    if constexpr (VEC)
     {
         const u32 c = (a.k + W - 1) / W;
         const u32 fit = n / (128U * BS);
@@ -171,7 +170,7 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
         u32 wave_bound = 0xFFFFFFFFU;
         if (c <= WAVE * SAMPLE_KEEP && pairs > 0)
         {
-            const u32 back = (n - pairs * 4 * BS) & ~3U;
+            const u32 back = VEC ? (n - pairs * 4 * BS) & ~3U : n - pairs * 4 * BS;
             float lo[SAMPLE_KEEP]; // ascending
 #pragma unroll
             for (int j = 0; j < SAMPLE_KEEP; ++j)
@@ -181,8 +180,21 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
             for (u32 p = 0; p < pairs; ++p)
             {
                 const u32 col = (p * BS + static_cast<u32>(t)) * 4;
-                const vfloat4 x[2] = {*reinterpret_cast<const vfloat4*>(row + col),
-                                      *reinterpret_cast<const vfloat4*>(row + back + col)};
+                vfloat4 x[2];
+                if constexpr (VEC)
+                {
+                    x[0] = *reinterpret_cast<const vfloat4*>(row + col);
+                    x[1] = *reinterpret_cast<const vfloat4*>(row + back + col);
+                }
+                else
+                {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                    {
+                        x[0][i] = row[col + i];
+                        x[1][i] = row[back + col + i];
+                    }
+                }
 #pragma unroll
                 for (int i = 0; i < 8; ++i)
                 {
@@ -225,7 +237,6 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     float radius = __builtin_inff();
     u64 radius_key = PAD_KEY;
     bool sampled = false;
-    if constexpr (VEC)
     {
         u32 bound = 0;
 #pragma unroll

@@ -116,6 +116,15 @@ def test_rows_long_enough_for_the_sampled_radius(bk, dev, oracle):
             gd, gl = _run(bk, dev, m, k, block=block, batch=8)
             ed, el = oracle.topk(m, k)
             assert np.array_equal(gd, ed) and np.array_equal(gl, el), (block, k)
+    # rows that do not start on a 16-byte boundary take 4-byte loads, the sample included
+    import torch
+    t = torch.from_numpy(m).to(dev)
+    for view, ref in ((t[:, 1:], m[:, 1:]), (t[:, 2:69999], m[:, 2:69999])):
+        for block, k in ((128, 100), (256, 256), (512, 2048)):
+            od, ol = bk.topk_bits(view, k, block, 8)
+            torch.cuda.synchronize()
+            ed, el = oracle.topk(np.ascontiguousarray(ref), k)
+            assert np.array_equal(od.cpu().numpy(), ed) and np.array_equal(ol.cpu().numpy(), el), (block, k)
     # explicit labels with the extreme values on tied entries, and label offsets
     labels = np.stack([rng.permutation(cols) for _ in range(rows)]).astype(np.int32)
     labels[4, :4] = [np.iinfo(np.int32).max, np.iinfo(np.int32).min, -1, 0]
