@@ -49,18 +49,14 @@ def fused_headline(bitsknn, torch, dev, q=65536, n=1 << 20, d=32, k=32, runs=3):
     out_l = torch.empty((q, k), dtype=torch.int32, device=dev)
 
     def timed(arithmetic):
-        bitsknn.fused_set_arithmetic(arithmetic)
-        try:
-            bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l)
-            torch.cuda.synchronize()
-            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            start.record()
-            for _ in range(runs):
-                bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l)
-            end.record()
-            torch.cuda.synchronize()
-        finally:
-            bitsknn.fused_set_arithmetic(bitsknn.FUSED_FP32)
+        bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l, arithmetic=arithmetic)
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(runs):
+            bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l, arithmetic=arithmetic)
+        end.record()
+        torch.cuda.synchronize()
         return start.elapsed_time(end) / 1e3 / runs
 
     seconds = timed(bitsknn.FUSED_FP32)

@@ -27,8 +27,7 @@ EXPORTS = (
     "bitsknn_fused_l2_topk_f32",
     "bitsknn_fused_workspace_bytes",
     "bitsknn_fused_l2_topk_f32_ws",
-    "bitsknn_fused_set_arithmetic",
-    "bitsknn_fused_get_arithmetic",
+    "bitsknn_fused_l2_topk_f32_ex",
 )
 
 
@@ -74,10 +73,10 @@ def lib():
         L.bitsknn_fused_l2_topk_f32.argtypes = [vp, vp, ctypes.c_int, i32, i32, vp, vp, ctypes.c_int,
                                                 ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                 ctypes.c_int, ctypes.c_int, vp]
-        L.bitsknn_fused_set_arithmetic.restype = ctypes.c_int
-        L.bitsknn_fused_set_arithmetic.argtypes = [ctypes.c_int]
-        L.bitsknn_fused_get_arithmetic.restype = ctypes.c_int
-        L.bitsknn_fused_get_arithmetic.argtypes = []
+        L.bitsknn_fused_l2_topk_f32_ex.restype = ctypes.c_int
+        L.bitsknn_fused_l2_topk_f32_ex.argtypes = [vp, vp, ctypes.c_int, i32, i32, vp, vp, ctypes.c_int,
+                                                   ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                   ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, sz, vp]
         L.bitsknn_fused_workspace_bytes.restype = ctypes.c_size_t
         L.bitsknn_fused_workspace_bytes.argtypes = [i32, i32, ctypes.c_int]
         L.bitsknn_fused_l2_topk_f32_ws.restype = ctypes.c_int
@@ -179,11 +178,16 @@ def distances(queries_dm, points_dm, op=DIST_L2, out=None):
     return out
 
 
+FUSED_FP32, FUSED_BF16X3 = 0, 1
+
+
 def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1, dim_mult=1,
-                  out_dist=None, out_label=None, workspace=None):
+                  out_dist=None, out_label=None, workspace=None, arithmetic=None):
     """bits-fused: top-k of ||p||^2 - 2 q.p without materialising the distance matrix.
     workspace: None -> the plain entry point; "auto" -> allocate what
-    bitsknn_fused_workspace_bytes asks for; or a uint8 device tensor."""
+    bitsknn_fused_workspace_bytes asks for; or a uint8 device tensor.
+    arithmetic: None -> the entry points with fp32 matrix instructions; FUSED_FP32 / FUSED_BF16X3
+    -> bitsknn_fused_l2_topk_f32_ex with that arithmetic."""
     import torch
     d, q = queries_dm.shape
     d2, n = points_dm.shape
@@ -192,32 +196,20 @@ def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1,
         out_dist = torch.empty((q, k), dtype=torch.float32, device=queries_dm.device)
     if out_label is None:
         out_label = torch.empty((q, k), dtype=torch.int32, device=queries_dm.device)
-    if workspace is None:
-        _check(lib().bitsknn_fused_l2_topk_f32(_ptr(queries_dm), _ptr(points_dm), d, q, n,
-                                               _ptr(out_dist), _ptr(out_label), k, params[0],
-                                               params[1], params[2], block_query_dim, dim_mult,
-                                               _stream()))
-        return out_dist, out_label
     if isinstance(workspace, str):
         workspace = torch.empty(max(1, fused_workspace_bytes(q, n, k)), dtype=torch.uint8,
                                 device=queries_dm.device)
-    _check(lib().bitsknn_fused_l2_topk_f32_ws(_ptr(queries_dm), _ptr(points_dm), d, q, n,
-                                              _ptr(out_dist), _ptr(out_label), k, params[0],
-                                              params[1], params[2], block_query_dim, dim_mult,
-                                              _ptr(workspace), workspace.numel(), _stream()))
+    head = (_ptr(queries_dm), _ptr(points_dm), d, q, n, _ptr(out_dist), _ptr(out_label), k,
+            params[0], params[1], params[2], block_query_dim, dim_mult)
+    if arithmetic is not None:
+        _check(lib().bitsknn_fused_l2_topk_f32_ex(*head, int(arithmetic), _ptr(workspace),
+                                                  workspace.numel() if workspace is not None else 0,
+                                                  _stream()))
+    elif workspace is None:
+        _check(lib().bitsknn_fused_l2_topk_f32(*head, _stream()))
+    else:
+        _check(lib().bitsknn_fused_l2_topk_f32_ws(*head, _ptr(workspace), workspace.numel(), _stream()))
     return out_dist, out_label
-
-
-FUSED_FP32, FUSED_BF16X3 = 0, 1
-
-
-def fused_set_arithmetic(arithmetic):
-    """Arithmetic of the products in the fused kernels for dim <= 32 (process-wide)."""
-    _check(lib().bitsknn_fused_set_arithmetic(int(arithmetic)))
-
-
-def fused_get_arithmetic():
-    return int(lib().bitsknn_fused_get_arithmetic())
 
 
 def fused_workspace_bytes(q, n, k):

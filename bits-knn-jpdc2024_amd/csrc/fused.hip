@@ -1,7 +1,5 @@
-// C-ABI entry points of bits-fused: parameter validation, the choice between the fused kernel, its
-// point-split form and the two-pass form, and dispatch to the kernels instantiated per list length
-// in fused_inst.hip.
-#include <atomic>
+// C-ABI entry points of bits-fused: parameter validation, the choice between the fused kernel and
+// its point-split form, and dispatch to the kernels instantiated per list length in fused_inst.hip.
 #include <initializer_list>
 
 #include "common.hpp"
@@ -11,9 +9,6 @@ namespace bitsknn
 {
 namespace
 {
-
-// arithmetic of the products for 9 <= d <= 64 (bitsknn_fused_set_arithmetic)
-std::atomic<int> g_arithmetic{BITSKNN_FUSED_FP32};
 
 bool in_list(int v, std::initializer_list<int> values)
 {
@@ -40,28 +35,25 @@ int choose_splits(int q, int n)
     return splits;
 }
 
-// Long lists (k >= 128): the 32-slot buffers of the fused kernel make every merge pay for the whole
-// list, and its time grows with k.  When the caller's workspace can hold the
-// q x n distance matrix (at most 16 GiB), the entry point with a workspace therefore computes the
-// matrix there with the MFMA distance kernel and selects with the bits kernel: two passes whose
-// time does not depend on k.  The matrix never leaves the workspace.
-constexpr int TWO_PASS_MIN_K = 128;
-constexpr size_t TWO_PASS_MAX_BYTES = 16ULL << 30;
-
-size_t two_pass_bytes(std::int32_t q, std::int32_t n, int k)
+// bytes of the partial lists [q][splits][k]: distances, then labels
+size_t partial_list_bytes(std::int32_t q, int splits, int k)
 {
-    const size_t bytes = static_cast<size_t>(q) * static_cast<size_t>(n) * sizeof(float);
-    return k >= TWO_PASS_MIN_K && bytes <= TWO_PASS_MAX_BYTES ? bytes : 0;
+    return static_cast<size_t>(q) * static_cast<size_t>(splits) * static_cast<size_t>(k) * 8;
 }
 
+// use_workspace: the points may be cut into ranges whose partial lists go to `workspace`; a
+// workspace too small for the ranges the problem would like gets as many as fit (a power of two,
+// down to the single fused kernel that needs none).
 int fused_impl(const float* queries_dim_major, const float* points_dim_major, int dim, std::int32_t q,
                std::int32_t n, float* out_dist, std::int32_t* out_label, int k, int query_reg,
-               int db_reg, int dim_reg, int block_query_dim, int dim_mult, void* workspace,
-               size_t workspace_bytes, bool use_workspace, void* stream)
+               int db_reg, int dim_reg, int block_query_dim, int dim_mult, int arithmetic,
+               void* workspace, size_t workspace_bytes, bool use_workspace, void* stream)
 {
     clear_error();
-    // the reference's nested dispatch, outermost first (fused_cache_knn.cu:72-144); the tuning
-    // parameters are validated like there although the MFMA tiling does not depend on them
+    // the reference's nested dispatch, outermost first (fused_cache_knn.cu:72-144).  Its tuning
+    // parameters describe a register tiling for the fp32 vector unit; they are validated like
+    // there and have no effect on the tiling for the matrix cores, which is fixed by the
+    // instruction shape (32 queries per wave) and by the dimension (points per stage)
     if (!in_list(query_reg, {2, 4, 8, 16}))
     {
         return fail(BITSKNN_ERR_UNSUPPORTED, "Unsupported queries_reg value: %d", query_reg);
@@ -95,6 +87,10 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     {
         return fail(BITSKNN_ERR_UNSUPPORTED, "Unsupported dimension: %d (at most 256)", dim);
     }
+    if (arithmetic != BITSKNN_FUSED_FP32 && arithmetic != BITSKNN_FUSED_BF16X3)
+    {
+        return fail(BITSKNN_ERR_INVALID, "bitsknn_fused_l2_topk_f32: unknown arithmetic %d", arithmetic);
+    }
     if (q <= 0)
     {
         return BITSKNN_OK;
@@ -113,34 +109,15 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
         return fail(BITSKNN_ERR_INVALID, "bitsknn_fused_l2_topk_f32: too many queries: %d", q);
     }
 
-    const size_t matrix_bytes = use_workspace ? two_pass_bytes(q, n, k) : 0;
-    if (matrix_bytes != 0 && workspace != nullptr && workspace_bytes >= matrix_bytes &&
-        reinterpret_cast<std::uintptr_t>(workspace) % 16 == 0)
+    int splits = use_workspace && workspace != nullptr &&
+                         reinterpret_cast<std::uintptr_t>(workspace) % 4 == 0
+                     ? choose_splits(q, n)
+                     : 1;
+    while (splits > 1 && partial_list_bytes(q, splits, k) > workspace_bytes)
     {
-        auto* matrix = static_cast<float*>(workspace);
-        const bool split = g_arithmetic.load(std::memory_order_relaxed) == BITSKNN_FUSED_BF16X3;
-        const int status = bitsknn_dist_f32(split ? BITSKNN_DIST_PARTIAL_L2_BF16X3 : BITSKNN_DIST_PARTIAL_L2, dim, static_cast<size_t>(q),
-                                            static_cast<size_t>(n), queries_dim_major, static_cast<size_t>(q),
-                                            points_dim_major, static_cast<size_t>(n), matrix,
-                                            static_cast<size_t>(n), stream);
-        if (status != BITSKNN_OK)
-        {
-            return status;
-        }
-        return bitsknn_topk_bits_f32(matrix, static_cast<size_t>(n), nullptr, 0, nullptr, static_cast<size_t>(q),
-                                     static_cast<size_t>(n), out_dist, out_label, static_cast<size_t>(k),
-                                     static_cast<std::uint32_t>(k), 512, 3, 0,
-                                     stream);
+        splits /= 2;
     }
-
-    int splits = use_workspace ? choose_splits(q, n) : 1;
     const size_t pairs = static_cast<size_t>(q) * static_cast<size_t>(splits) * static_cast<size_t>(k);
-    if (splits > 1 && (workspace == nullptr || workspace_bytes < pairs * 8))
-    {
-        return fail(BITSKNN_ERR_INVALID,
-                    "bitsknn_fused_l2_topk_f32_ws: workspace of %zu bytes is too small, %zu needed",
-                    workspace_bytes, pairs * 8);
-    }
     fused_args a{queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, 1, 0};
     if (splits > 1)
     {
@@ -152,7 +129,7 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     a.split_points = ((n + splits - 1) / splits + 255) / 256 * 256;
 
     auto* hip_stream = static_cast<hipStream_t>(stream);
-    const bool split = g_arithmetic.load(std::memory_order_relaxed) == BITSKNN_FUSED_BF16X3;
+    const bool split = arithmetic == BITSKNN_FUSED_BF16X3;
     hipError_t status = hipSuccess;
     switch (k)
     {
@@ -200,24 +177,8 @@ extern "C" int bitsknn_fused_l2_topk_f32(const float* queries_dim_major,
                                          int dim_mult, void* stream)
 {
     return bitsknn::fused_impl(queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, k,
-                               query_reg, db_reg, dim_reg, block_query_dim, dim_mult, nullptr, 0, false,
-                               stream);
-}
-
-extern "C" int bitsknn_fused_set_arithmetic(int arithmetic)
-{
-    bitsknn::clear_error();
-    if (arithmetic != BITSKNN_FUSED_FP32 && arithmetic != BITSKNN_FUSED_BF16X3)
-    {
-        return bitsknn::fail(BITSKNN_ERR_INVALID, "bitsknn_fused_set_arithmetic: unknown arithmetic %d", arithmetic);
-    }
-    bitsknn::g_arithmetic.store(arithmetic, std::memory_order_relaxed);
-    return BITSKNN_OK;
-}
-
-extern "C" int bitsknn_fused_get_arithmetic(void)
-{
-    return bitsknn::g_arithmetic.load(std::memory_order_relaxed);
+                               query_reg, db_reg, dim_reg, block_query_dim, dim_mult, BITSKNN_FUSED_FP32,
+                               nullptr, 0, false, stream);
 }
 
 extern "C" size_t bitsknn_fused_workspace_bytes(int32_t q, int32_t n, int k)
@@ -226,13 +187,8 @@ extern "C" size_t bitsknn_fused_workspace_bytes(int32_t q, int32_t n, int k)
     {
         return 0;
     }
-    const size_t matrix_bytes = bitsknn::two_pass_bytes(q, n, k);
-    if (matrix_bytes != 0)
-    {
-        return matrix_bytes;
-    }
     const int splits = bitsknn::choose_splits(q, n);
-    return splits > 1 ? static_cast<size_t>(q) * static_cast<size_t>(splits) * static_cast<size_t>(k) * 8 : 0;
+    return splits > 1 ? bitsknn::partial_list_bytes(q, splits, k) : 0;
 }
 
 extern "C" int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major,
@@ -243,6 +199,18 @@ extern "C" int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major,
                                             size_t workspace_bytes, void* stream)
 {
     return bitsknn::fused_impl(queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, k,
-                               query_reg, db_reg, dim_reg, block_query_dim, dim_mult, workspace,
-                               workspace_bytes, true, stream);
+                               query_reg, db_reg, dim_reg, block_query_dim, dim_mult, BITSKNN_FUSED_FP32,
+                               workspace, workspace_bytes, true, stream);
+}
+
+extern "C" int bitsknn_fused_l2_topk_f32_ex(const float* queries_dim_major,
+                                            const float* points_dim_major, int dim, int32_t q,
+                                            int32_t n, float* out_dist, int32_t* out_label, int k,
+                                            int query_reg, int db_reg, int dim_reg,
+                                            int block_query_dim, int dim_mult, int arithmetic,
+                                            void* workspace, size_t workspace_bytes, void* stream)
+{
+    return bitsknn::fused_impl(queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, k,
+                               query_reg, db_reg, dim_reg, block_query_dim, dim_mult, arithmetic, workspace,
+                               workspace_bytes, workspace != nullptr, stream);
 }

@@ -407,7 +407,13 @@ private:
 class fused_cache_knn : public device_knn
 {
 public:
-    std::string id() const override { return "fused-cache"; }
+    // arithmetic: BITSKNN_FUSED_FP32 (the reference's id) or BITSKNN_FUSED_BF16X3
+    explicit fused_cache_knn(int arithmetic = BITSKNN_FUSED_FP32) : arithmetic_(arithmetic) {}
+
+    std::string id() const override
+    {
+        return arithmetic_ == BITSKNN_FUSED_BF16X3 ? "fused-cache-bf16x3" : "fused-cache";
+    }
 
     void initialize(const knn_args& args) override
     {
@@ -419,6 +425,7 @@ public:
         const auto queries = to_dim_major(args_.queries, query_count(), dim(), args_.queries_layout);
         points_ = device_buffer<float>{points.size()};
         queries_ = device_buffer<float>{queries.size()};
+        // partial lists of the point ranges when the queries alone do not fill the GPU
         workspace_ = device_buffer<unsigned char>{bitsknn_fused_workspace_bytes(
             static_cast<std::int32_t>(query_count()), static_cast<std::int32_t>(point_count()),
             static_cast<int>(k()))};
@@ -433,45 +440,48 @@ public:
 
     void selection() override
     {
-        BITSKNN_CHECK(bitsknn_fused_l2_topk_f32_ws(
+        BITSKNN_CHECK(bitsknn_fused_l2_topk_f32_ex(
             queries_.data(), points_.data(), static_cast<int>(dim()), static_cast<std::int32_t>(query_count()),
             static_cast<std::int32_t>(point_count()), out_dist_.data(), out_label_.data(),
             static_cast<int>(k()), static_cast<int>(args_.items_per_thread[0]),
             static_cast<int>(args_.items_per_thread[1]), static_cast<int>(args_.items_per_thread[2]),
-            static_cast<int>(args_.selection_block_size), static_cast<int>(args_.deg),
-            workspace_.data(), workspace_.size(), nullptr));
+            static_cast<int>(args_.selection_block_size), static_cast<int>(args_.deg), arithmetic_,
+            workspace_.size() != 0 ? workspace_.data() : nullptr, workspace_.size(), nullptr));
         sync_default_stream();
     }
 
     float transfer_in_seconds() const override { return transfer_in_.seconds(); }
 
 private:
+    int arithmetic_;
     device_buffer<float> points_;
     device_buffer<float> queries_;
-    device_buffer<unsigned char> workspace_; // partial lists when the points are split into ranges
+    device_buffer<unsigned char> workspace_;
     knn_host::transfer_timer transfer_in_;
 };
 
-// bits-fused with the products from three bf16 pieces per operand (no counterpart in the reference):
-// the same wrapper, the library's arithmetic switched for the duration of the kernel launch
-class fused_cache_bf16x3_knn : public fused_cache_knn
+// `fused-cache-2pass` (no counterpart among the reference's ids; the same two phases as its runs
+// of bits-prefetch next to fused-cache, scripts/run-fused.sh): the partial distances
+// ||p||^2 - 2 q.p go to a q x n matrix in the `distances` phase (matrix instructions) and the bits
+// kernel selects from it in the `selection` phase.  Unlike the fused kernel its time does not grow
+// with k, at the price of the matrix.
+class two_pass_knn : public device_knn
 {
 public:
-    std::string id() const override { return "fused-cache-bf16x3"; }
+    std::string id() const override { return "fused-cache-2pass"; }
+
+    void initialize(const knn_args& args) override
+    {
+        set_dist_impl(make_partial_l2_distance());
+        device_knn::initialize(args);
+    }
 
     void selection() override
     {
-        BITSKNN_CHECK(bitsknn_fused_set_arithmetic(BITSKNN_FUSED_BF16X3));
-        try
-        {
-            fused_cache_knn::selection();
-        }
-        catch (...)
-        {
-            bitsknn_fused_set_arithmetic(BITSKNN_FUSED_FP32);
-            throw;
-        }
-        BITSKNN_CHECK(bitsknn_fused_set_arithmetic(BITSKNN_FUSED_FP32));
+        BITSKNN_CHECK(bitsknn_topk_bits_f32(
+            in_dist_gpu(), point_count(), nullptr, 0, nullptr, query_count(), point_count(),
+            out_dist_.data(), out_label_.data(), k(), static_cast<std::uint32_t>(k()), 512, 3, 0, nullptr));
+        sync_default_stream();
     }
 };
 
@@ -511,8 +521,9 @@ std::vector<std::unique_ptr<knn>> make_algorithms()
     algorithms.push_back(std::make_unique<bits_knn>(true));
     algorithms.push_back(std::make_unique<single_query_bits>());
     algorithms.push_back(std::make_unique<partial_bitonic_regs>());
-    algorithms.push_back(std::make_unique<fused_cache_knn>());
-    algorithms.push_back(std::make_unique<fused_cache_bf16x3_knn>());
+    algorithms.push_back(std::make_unique<fused_cache_knn>(BITSKNN_FUSED_FP32));
+    algorithms.push_back(std::make_unique<fused_cache_knn>(BITSKNN_FUSED_BF16X3));
+    algorithms.push_back(std::make_unique<two_pass_knn>());
     algorithms.push_back(std::make_unique<dist_runner>("cublas-dist", &make_expanded_distance));
     algorithms.push_back(std::make_unique<dist_runner>("magma-dist", &make_l2_distance));
     algorithms.push_back(std::make_unique<dist_runner>("magma-part-dist", &make_partial_l2_distance));

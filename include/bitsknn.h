@@ -134,7 +134,10 @@ int bitsknn_dist_f32(int op, int dim, size_t q, size_t n, const float* queries_d
  *  query_reg, db_reg, dim_reg, block_query_dim, dim_mult
  *                             the reference's tuning parameters; validated against its lists
  *                             ({2,4,8,16}, {4,8,16}, {1,2,4}, {1,2,4}, {1,2,4}) with its
- *                             messages; dim must be >= dim_mult*dim_reg as there
+ *                             messages; dim must be >= dim_mult*dim_reg as there.  Accepted for
+ *                             compatibility only: they describe a register tiling for the fp32
+ *                             vector unit and do not change the matrix-core kernel, so a sweep
+ *                             over them measures the same kernel every time
  */
 int bitsknn_fused_l2_topk_f32(const float* queries_dim_major, const float* points_dim_major,
                               int dim, int32_t q, int32_t n, float* out_dist, int32_t* out_label,
@@ -142,45 +145,49 @@ int bitsknn_fused_l2_topk_f32(const float* queries_dim_major, const float* point
                               int dim_mult, void* stream);
 
 /*
- * Arithmetic of the products q.p inside the bits-fused kernels for 9 <= dim <= 64 (process-wide, read
- * at every call):
- *   BITSKNN_FUSED_FP32    fp32 matrix instructions (v_mfma_f32_32x32x2_f32).
- *   BITSKNN_FUSED_BF16X3  every fp32 operand is cut exactly into three bf16 pieces and a product
- *                         is the fp32 sum of six bf16 products on the bf16 matrix path
- *                         (v_mfma_f32_32x32x16_bf16); what is left out is below 2^-23 of a
- *                         product, the size of one fp32 rounding.
- * Other dimensions always use BITSKNN_FUSED_FP32.  No counterpart in the reference, whose fused
- * kernel multiplies on the fp32 vector unit (fused_cache_kernel_structs.cuh:457-522).
- * bitsknn_fused_set_arithmetic returns BITSKNN_ERR_INVALID for another value.
- */
-#define BITSKNN_FUSED_FP32 0
-#define BITSKNN_FUSED_BF16X3 1
-int bitsknn_fused_set_arithmetic(int arithmetic);
-int bitsknn_fused_get_arithmetic(void);
-
-/*
- * bits-fused with a caller-provided workspace.  Same neighbours as bitsknn_fused_l2_topk_f32.
- * When there are too few queries to fill the GPU with one workgroup per 128 queries, the points
- * are cut into ranges that are searched by separate workgroups; their partial lists go to the
+ * bits-fused with a caller-provided workspace.  Same neighbours as bitsknn_fused_l2_topk_f32, and
+ * still the fused kernel: no distance is written to memory.  When there are too few queries to
+ * fill the GPU with one workgroup per 128 queries, the points are cut into ranges that are
+ * searched by separate workgroups; their partial lists (k pairs per query and range) go to the
  * workspace and one bits pass (explicit labels) selects the final k.
- * For k >= 128, when the q x n distance matrix fits 16 GiB, bitsknn_fused_workspace_bytes asks for
- * room for that matrix and the call runs the MFMA distance kernel into the workspace followed by
- * the bits kernel (the fused kernel's 32-slot buffers make its time grow with k; the two passes
- * do not).  A smaller workspace, or bitsknn_fused_l2_topk_f32, keeps the single fused kernel.
  *
  * No counterpart in the reference, whose fused kernel always runs one thread block per query tile
  * (src/topk/singlepass/fused_cache_knn.cu:60-69); the host wrapper that owns the device memory
  * (fused_cache_knn::initialize, fused_cache_knn.cu:149-195) is where the workspace is allocated.
  *
- * bitsknn_fused_workspace_bytes returns the size the call wants (0: workspace unused).
- * Errors as for bitsknn_fused_l2_topk_f32, plus BITSKNN_ERR_INVALID for a workspace too small
- * for the partial lists.
+ * bitsknn_fused_workspace_bytes returns the size the call wants: 8*q*ranges*k bytes, at most 64
+ * ranges; 0 when the queries fill the GPU by themselves.  A smaller workspace (4-byte aligned) is
+ * not an error: the call uses as many ranges as fit, down to the single kernel without any.
+ * Errors as for bitsknn_fused_l2_topk_f32.
  */
 size_t bitsknn_fused_workspace_bytes(int32_t q, int32_t n, int k);
 int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major, const float* points_dim_major,
                                  int dim, int32_t q, int32_t n, float* out_dist, int32_t* out_label,
                                  int k, int query_reg, int db_reg, int dim_reg, int block_query_dim,
                                  int dim_mult, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * bits-fused with the arithmetic of the products q.p chosen per call (nothing process-wide is
+ * read); workspace may be NULL (then as bitsknn_fused_l2_topk_f32) or as for
+ * bitsknn_fused_l2_topk_f32_ws.
+ *   BITSKNN_FUSED_FP32    fp32 matrix instructions (v_mfma_f32_32x32x2_f32); what the two entry
+ *                         points above use.
+ *   BITSKNN_FUSED_BF16X3  for 9 <= dim <= 64: every fp32 operand is cut exactly into three bf16
+ *                         pieces and a product is the fp32 sum of six bf16 products on the bf16
+ *                         matrix path (v_mfma_f32_32x32x16_bf16); what is left out is below 2^-23
+ *                         of a product, the size of one fp32 rounding.  Other dimensions use
+ *                         BITSKNN_FUSED_FP32.
+ * No counterpart in the reference, whose fused kernel multiplies on the fp32 vector unit
+ * (include/bits/topk/singlepass/fused_cache_kernel_structs.cuh:457-522).
+ * BITSKNN_ERR_INVALID for another value of `arithmetic`.
+ */
+#define BITSKNN_FUSED_FP32 0
+#define BITSKNN_FUSED_BF16X3 1
+int bitsknn_fused_l2_topk_f32_ex(const float* queries_dim_major, const float* points_dim_major,
+                                 int dim, int32_t q, int32_t n, float* out_dist, int32_t* out_label,
+                                 int k, int query_reg, int db_reg, int dim_reg, int block_query_dim,
+                                 int dim_mult, int arithmetic, void* workspace, size_t workspace_bytes,
+                                 void* stream);
 
 #ifdef __cplusplus
 }

@@ -53,14 +53,52 @@ def test_topk_rejects_unsupported_parameters(bk, k, block, batch, msg):
     assert text == msg
 
 
-def test_fused_arithmetic_switch(bk):
-    assert bk.fused_get_arithmetic() == bk.FUSED_FP32
-    bk.fused_set_arithmetic(bk.FUSED_BF16X3)
-    assert bk.fused_get_arithmetic() == bk.FUSED_BF16X3
-    bk.fused_set_arithmetic(bk.FUSED_FP32)
-    with pytest.raises(bk.BitsKnnError, match="unknown arithmetic 7"):
-        bk.fused_set_arithmetic(7)
-    assert bk.fused_get_arithmetic() == bk.FUSED_FP32
+def _fused_ex_status(bk, k, arithmetic, params=(8, 4, 2)):
+    # validation only: q = 0 returns before any pointer is looked at or any HIP call is made
+    L = bk.lib()
+    st = L.bitsknn_fused_l2_topk_f32_ex(None, None, 8, 0, 0, None, None, k, params[0], params[1], params[2],
+                                        1, 1, arithmetic, None, 0, None)
+    return st, L.bitsknn_last_error().decode()
+
+
+def test_fused_arithmetic_is_a_call_argument(bk):
+    assert _fused_ex_status(bk, 32, bk.FUSED_FP32) == (bk.OK, "")
+    assert _fused_ex_status(bk, 32, bk.FUSED_BF16X3) == (bk.OK, "")
+    st, text = _fused_ex_status(bk, 32, 7)
+    assert st == bk.ERR_INVALID and "unknown arithmetic 7" in text
+    st, text = _fused_ex_status(bk, 5, bk.FUSED_BF16X3)
+    assert st == bk.ERR_UNSUPPORTED and text == "Unsupported k value: 5"
+    # nothing process-wide is left behind by a call: the library exports no mode setter
+    assert not hasattr(bk, "fused_set_arithmetic")
+    with pytest.raises(AttributeError):
+        bk.lib().bitsknn_fused_set_arithmetic
+
+
+def test_two_threads_with_different_arithmetics(bk):
+    """Two host threads validate calls with different arithmetics and different mistakes at the
+    same time: every thread sees its own status and its own (thread-local) message."""
+    import threading
+    failures = []
+
+    def worker(arithmetic, bad_k, rounds=2000):
+        for i in range(rounds):
+            if i % 2 == 0:
+                got = _fused_ex_status(bk, 32, arithmetic)
+                want = (bk.OK, "")
+            else:
+                got = _fused_ex_status(bk, bad_k, arithmetic)
+                want = (bk.ERR_UNSUPPORTED, "Unsupported k value: %d" % bad_k)
+            if got != want:
+                failures.append((arithmetic, i, got))
+                return
+
+    threads = [threading.Thread(target=worker, args=(bk.FUSED_FP32, 5)),
+               threading.Thread(target=worker, args=(bk.FUSED_BF16X3, 7))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not failures, failures[:3]
 
 
 def test_topk_accepts_reference_parameter_lists_with_zero_rows(bk):
