@@ -215,7 +215,7 @@ def test_long_lists_stay_in_the_fused_kernel(bk, dev, oracle, k):
     matrix), and with or without it the result is the fused kernel's."""
     n, q, d = 20000, 300, 24
     points, queries = oracle.generate(77, n, q, d)
-    assert bk.fused_workspace_bytes(q, n, k) <= 8 * q * 64 * k < q * n * 4
+    assert 0 < bk.fused_workspace_bytes(q, n, k) <= 8 * q * 64 * k and bk.fused_workspace_bytes(q, n, k) < q * n * 4
     gd, gl = _fused(bk, dev, points, queries, k, workspace="auto")
     _check(oracle, points, queries, k, gd, gl)
     fd, fl = _fused(bk, dev, points, queries, k)
