@@ -28,6 +28,8 @@ EXPORTS = (
     "bitsknn_fused_workspace_bytes",
     "bitsknn_fused_l2_topk_f32_ws",
     "bitsknn_fused_l2_topk_f32_ex",
+    "bitsknn_fused_static_scratch_bytes",
+    "bitsknn_fused_l2_topk_f32_static",
 )
 
 
@@ -83,6 +85,10 @@ def lib():
         L.bitsknn_fused_l2_topk_f32_ws.argtypes = [vp, vp, ctypes.c_int, i32, i32, vp, vp, ctypes.c_int,
                                                    ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                    ctypes.c_int, ctypes.c_int, vp, sz, vp]
+        L.bitsknn_fused_static_scratch_bytes.restype = ctypes.c_size_t
+        L.bitsknn_fused_static_scratch_bytes.argtypes = []
+        L.bitsknn_fused_l2_topk_f32_static.restype = ctypes.c_int
+        L.bitsknn_fused_l2_topk_f32_static.argtypes = L.bitsknn_fused_l2_topk_f32.argtypes
         _lib = L
     return _lib
 
@@ -185,7 +191,8 @@ def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1,
                   out_dist=None, out_label=None, workspace=None, arithmetic=None):
     """bits-fused: top-k of ||p||^2 - 2 q.p without materialising the distance matrix.
     workspace: None -> the plain entry point; "auto" -> allocate what
-    bitsknn_fused_workspace_bytes asks for; or a uint8 device tensor.
+    bitsknn_fused_workspace_bytes asks for; "static" -> the entry point that uses the library's own
+    scratch memory and allocates nothing; or a uint8 device tensor.
     arithmetic: None -> the entry points with fp32 matrix instructions; FUSED_FP32 / FUSED_BF16X3
     -> bitsknn_fused_l2_topk_f32_ex with that arithmetic."""
     import torch
@@ -196,12 +203,15 @@ def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1,
         out_dist = torch.empty((q, k), dtype=torch.float32, device=queries_dm.device)
     if out_label is None:
         out_label = torch.empty((q, k), dtype=torch.int32, device=queries_dm.device)
-    if isinstance(workspace, str):
+    if isinstance(workspace, str) and workspace == "auto":
         workspace = torch.empty(max(1, fused_workspace_bytes(q, n, k)), dtype=torch.uint8,
                                 device=queries_dm.device)
     head = (_ptr(queries_dm), _ptr(points_dm), d, q, n, _ptr(out_dist), _ptr(out_label), k,
             params[0], params[1], params[2], block_query_dim, dim_mult)
-    if arithmetic is not None:
+    if isinstance(workspace, str) and workspace == "static":
+        assert arithmetic is None
+        _check(lib().bitsknn_fused_l2_topk_f32_static(*head, _stream()))
+    elif arithmetic is not None:
         _check(lib().bitsknn_fused_l2_topk_f32_ex(*head, int(arithmetic), _ptr(workspace),
                                                   workspace.numel() if workspace is not None else 0,
                                                   _stream()))
@@ -214,3 +224,7 @@ def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1,
 
 def fused_workspace_bytes(q, n, k):
     return int(lib().bitsknn_fused_workspace_bytes(q, n, k))
+
+
+def fused_static_scratch_bytes():
+    return int(lib().bitsknn_fused_static_scratch_bytes())

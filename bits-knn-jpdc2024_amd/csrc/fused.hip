@@ -1,6 +1,7 @@
 // C-ABI entry points of bits-fused: parameter validation, the choice between the fused kernel and
 // its point-split form, and dispatch to the kernels instantiated per list length in fused_inst.hip.
 #include <initializer_list>
+#include <mutex>
 
 #include "common.hpp"
 #include "fused_args.hpp"
@@ -9,6 +10,50 @@ namespace bitsknn
 {
 namespace
 {
+
+// Scratch memory of bitsknn_fused_l2_topk_f32_static: the partial lists of the point ranges.
+// Every GPU the library runs on holds its own copy of the array until the process ends.  In host
+// code the array's name is only a handle for hipGetSymbolAddress; the device address it returns
+// (one per device) is what kernels, copies and fills get.
+constexpr size_t STATIC_SCRATCH_BYTES = 32ULL << 20;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[MAX_DEVICES] = {}; // device address of `scratch` on each device, once known
+
+// Device address of the current device's copy of `scratch`, looked up on the first call per
+// device; nullptr (with the error recorded) when a runtime call fails.
+void* static_scratch()
+{
+    int device = -1;
+    hipError_t status = hipGetDevice(&device);
+    if (status == hipSuccess && (device < 0 || device >= MAX_DEVICES))
+    {
+        fail(BITSKNN_ERR_INVALID, "bitsknn_fused_l2_topk_f32_static: device %d is not supported (at most %d)",
+             device, MAX_DEVICES);
+        return nullptr;
+    }
+    if (status == hipSuccess)
+    {
+        const std::lock_guard<std::mutex> lock{g_scratch_mutex};
+        if (g_scratch_ptr[device] == nullptr)
+        {
+            void* ptr = nullptr;
+            status = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+            if (status == hipSuccess)
+            {
+                g_scratch_ptr[device] = ptr;
+            }
+        }
+        if (status == hipSuccess)
+        {
+            return g_scratch_ptr[device];
+        }
+    }
+    fail(BITSKNN_ERR_HIP, "%s:%d %s: %s", __FILE__, __LINE__, hipGetErrorName(status), hipGetErrorString(status));
+    return nullptr;
+}
 
 bool in_list(int v, std::initializer_list<int> values)
 {
@@ -213,4 +258,45 @@ extern "C" int bitsknn_fused_l2_topk_f32_ex(const float* queries_dim_major,
     return bitsknn::fused_impl(queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, k,
                                query_reg, db_reg, dim_reg, block_query_dim, dim_mult, arithmetic, workspace,
                                workspace_bytes, workspace != nullptr, stream);
+}
+
+extern "C" size_t bitsknn_fused_static_scratch_bytes(void) { return bitsknn::STATIC_SCRATCH_BYTES; }
+
+extern "C" int bitsknn_fused_l2_topk_f32_static(const float* queries_dim_major,
+                                                const float* points_dim_major, int dim, int32_t q,
+                                                int32_t n, float* out_dist, int32_t* out_label, int k,
+                                                int query_reg, int db_reg, int dim_reg,
+                                                int block_query_dim, int dim_mult, void* stream)
+{
+    using namespace bitsknn;
+    // parameter errors first, with the messages of the other entry points (no queries: validation only)
+    const int valid = fused_impl(queries_dim_major, points_dim_major, dim, 0, n, out_dist, out_label, k,
+                                 query_reg, db_reg, dim_reg, block_query_dim, dim_mult, BITSKNN_FUSED_FP32,
+                                 nullptr, 0, false, stream);
+    if (valid != BITSKNN_OK)
+    {
+        return valid;
+    }
+    const size_t need = bitsknn_fused_workspace_bytes(q, n, k);
+    if (need > STATIC_SCRATCH_BYTES)
+    {
+        return fail(BITSKNN_ERR_INVALID,
+                    "bitsknn_fused_l2_topk_f32_static: the partial lists of this problem take %zu bytes, the "
+                    "library's own scratch memory holds %zu (use bitsknn_fused_l2_topk_f32_ws)",
+                    need, STATIC_SCRATCH_BYTES);
+    }
+    void* workspace = nullptr;
+    if (need != 0 && q > 0)
+    {
+        workspace = static_scratch();
+        if (workspace == nullptr)
+        {
+            return BITSKNN_ERR_HIP;
+        }
+    }
+    // The kernels write every entry of the partial lists they read back (ranges without points
+    // included), so nothing in the scratch memory has to be cleared between calls.
+    return fused_impl(queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, k, query_reg,
+                      db_reg, dim_reg, block_query_dim, dim_mult, BITSKNN_FUSED_FP32, workspace,
+                      workspace != nullptr ? STATIC_SCRATCH_BYTES : 0, workspace != nullptr, stream);
 }

@@ -189,6 +189,27 @@ int bitsknn_fused_l2_topk_f32_ex(const float* queries_dim_major, const float* po
                                  int dim_mult, int arithmetic, void* workspace, size_t workspace_bytes,
                                  void* stream);
 
+/*
+ * bitsknn_fused_l2_topk_f32_ws for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc): the partial lists go to
+ * scratch memory inside the library, a static device array of bitsknn_fused_static_scratch_bytes()
+ * = 32 MiB that every GPU the library runs on holds until the process ends.  The call allocates
+ * and frees nothing (its first call on a device looks up the array's address on that device).
+ * Same results as bitsknn_fused_l2_topk_f32_ws with the workspace it asks for, bit for bit.
+ *
+ * No counterpart in the reference.
+ *
+ * Errors as for bitsknn_fused_l2_topk_f32, plus BITSKNN_ERR_INVALID when
+ * bitsknn_fused_workspace_bytes(q, n, k) exceeds the scratch memory (nothing is launched then).
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
+ * streams or threads) race on it and must be serialised by the caller.
+ */
+size_t bitsknn_fused_static_scratch_bytes(void);
+int bitsknn_fused_l2_topk_f32_static(const float* queries_dim_major, const float* points_dim_major,
+                                     int dim, int32_t q, int32_t n, float* out_dist,
+                                     int32_t* out_label, int k, int query_reg, int db_reg, int dim_reg,
+                                     int block_query_dim, int dim_mult, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
