@@ -1,123 +1,203 @@
 #!/usr/bin/env python3
 """Benchmark of the k-NN hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--k 32] [--block-size 256]
-                    [--items-per-thread 8] [--sweep] [--no-fused] [--no-cpu-baseline]
-                    [--copy-calibration]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only LEG,...] [--skip LEG,...]
+                    [--k 32] [--block-size 256] [--items-per-thread 8] [--prefetch]
+                    [--fused-d D] [--fused-k K] [--no-verify]
 
 A step is one bits top-k pass (through the C ABI) over a resident 1024 x 1,048,576 fp32 matrix
 of i.i.d. uniform [0,1) values (4 GiB, generated on the device).  The printed JSON line follows
 the reference's throughput convention: elements/s = rows*cols / mean step time
 (reference scripts/plot-kselection.py:161).  `roofline` prices the top-k kernel against HBM
 bandwidth with its algorithmic bytes (4 B read per matrix element + 8 B written per output pair)
-over the kernel's mean duration measured with events on the launch stream.  `cpu_baseline` times
-the CPU restatement of the reference's parallel top-k (reference src/topk/parallel_knn.cpp:30-65)
-on the host cores, on a bounded sample.  `fused` reports the second headline figure, bits-fused
-queries/s at n = 2^20 points, q = 65,536 queries, d = 32, k = 32, priced against the fp32 MFMA peak
-with 2*q*n*d flops.
+over the kernel's mean duration measured with events on the launch stream.
+
+The same line carries the other workloads of the path, each leg with the fraction of the roofline
+that bounds it (`frac`) and `verified`: after a leg's timed launches a sample of its rows or
+queries is compared with the CPU oracle (top-k: values and labels bit for bit; distances: k-th
+neighbour distance within 1e-5 of the scale of its terms and recall >= 0.999), so that a launch
+which did not do its work cannot produce a figure.
+
+  headline     the step described above (`value`, `roofline`)
+  calibration  a plain streaming read of the same matrix with the same row-per-workgroup mapping
+               (the read rate this machine reaches) and 1 GiB device copies (known traffic for
+               scaling byte counters read under a profiler)
+  sweep        the 4 GiB matrix at k in {16,32,128,512,2048} x block size {128,256,512}, plus the
+               configuration the shipped optima file names for each k
+  hard         16,384 x 65,536 rows sorted ascending / descending / drawn from 256 values, k = 32, 256
+  gemm         ||p||^2 - 2 q.p on fp32 MFMA for 1,048,576 points x 4,096 queries, d = 64 (a 16 GiB
+               matrix), then bits top-k (k = 64) on it
+  fused        bits-fused, 1,048,576 points x 65,536 queries, d in {8,16,32} x k in {4,16,32}, priced
+               against the fp32 MFMA peak with 2*q*n*d flops; `fused` itself is the d = 32, k = 32
+               case (queries/s), `fused.grid` the nine cases
+  cpu          `cpu_baseline`: the CPU restatement of the reference's parallel top-k (reference
+               src/topk/parallel_knn.cpp:30-65) on the host cores and of its serial top-k
+               (src/topk/serial_knn.cpp:35-43) on one core, on a 1024 x 65,536 matrix
 """
 import argparse
+import hashlib
 import json
 import os
+import re
 import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.join(ROOT, "bits-knn-jpdc2024_amd")
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "bits-knn-jpdc2024_amd"))
+sys.path.insert(0, PKG)
 
 HBM_PEAK_GBS = 8000.0       # MI355X published peak
 MFMA_F32_PEAK_TFLOPS = 157.3  # dense fp32 matrix peak
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 matrix peak
+LEGS = ("headline", "calibration", "sweep", "hard", "gemm", "fused", "cpu")
+REL = 1e-5
+MIN_RECALL = 0.999
+
+# the sources the top-k kernel is built from; the profiled traffic figure is only quoted while
+# they are the ones that were profiled
+TOPK_SOURCES = ("csrc/topk_bits_kernel.hpp", "csrc/bitonic_net.hpp", "csrc/common.hpp",
+                "csrc/topk_bits_inst.hip", "csrc/topk_bits.hip")
+TOPK_PROFILE = os.path.join(ROOT, "profiles", "bits_topk_1024x1048576_k32.md")
 
 
-# HBM bytes per launch of the top-k kernel from two counter passes (FETCH_SIZE, WRITE_SIZE, each
-# scaled by what the counter reads for a plain 1 GiB copy), keyed by (rows, cols, k).  Measured
-# under a profiler, so it cannot be taken live; other workloads report null.
-MEASURED_TRAFFIC_BYTES = {(1024, 1 << 20, 32): 4295326899}
+def topk_sources_sha256():
+    digest = hashlib.sha256()
+    for name in TOPK_SOURCES:
+        with open(os.path.join(PKG, name), "rb") as handle:
+            digest.update(handle.read())
+    return digest.hexdigest()
 
 
-def fused_headline(bitsknn, torch, dev, q=65536, n=1 << 20, d=32, k=32, runs=3):
-    """Config 5's headline case with both arithmetics of the products: fp32 matrix instructions
-    (the figure quoted against the fp32 MFMA peak) and three bf16 pieces per operand, six bf16
-    matrix products per fp32 product (quoted against the bf16 MFMA peak with six times the flops)."""
-    gen = torch.Generator(device=dev)
-    gen.manual_seed(24)
-    points = torch.rand((d, n), device=dev, generator=gen)
-    queries = torch.rand((d, q), device=dev, generator=gen)
-    out_d = torch.empty((q, k), dtype=torch.float32, device=dev)
-    out_l = torch.empty((q, k), dtype=torch.int32, device=dev)
-
-    def timed(arithmetic):
-        bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l, arithmetic=arithmetic)
-        torch.cuda.synchronize()
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        for _ in range(runs):
-            bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l, arithmetic=arithmetic)
-        end.record()
-        torch.cuda.synchronize()
-        return start.elapsed_time(end) / 1e3 / runs
-
-    seconds = timed(bitsknn.FUSED_FP32)
-    tflops = 2.0 * q * n * d / seconds / 1e12
-    split_seconds = timed(bitsknn.FUSED_BF16X3)
-    split_tflops = 6 * 2.0 * q * n * d / split_seconds / 1e12
-    return {"workload": f"bits-fused, {n} points x {q} queries, d={d}, k={k}, fp32 uniform[0,1)",
-            "arithmetic": "fp32 matrix instructions",
-            "queries_per_s": q / seconds, "ms": seconds * 1e3, "pairs_per_s": q * n / seconds,
-            "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_F32_PEAK_TFLOPS,
-                         "unit": "TFLOP/s", "frac": tflops / MFMA_F32_PEAK_TFLOPS},
-            "bf16x3": {"arithmetic": "three bf16 pieces per fp32 operand, six bf16 matrix products per product, "
-                                     "fp32 accumulation",
-                       "queries_per_s": q / split_seconds, "ms": split_seconds * 1e3,
-                       "pairs_per_s": q * n / split_seconds,
-                       "roofline": {"bound": "mfma", "achieved": split_tflops, "peak": MFMA_BF16_PEAK_TFLOPS,
-                                    "unit": "TFLOP/s", "frac": split_tflops / MFMA_BF16_PEAK_TFLOPS}}}
+def profiled_traffic(rows, cols, k):
+    """HBM bytes per launch of the headline kernel from the two counter passes recorded in the
+    profile summary, or None when the summary is for another workload or for other kernel sources
+    than the ones in the tree (the figure cannot be taken live: counters need a profiler)."""
+    try:
+        with open(TOPK_PROFILE) as handle:
+            text = handle.read()
+    except OSError:
+        return None
+    fields = dict(re.findall(r"^(\w+) = (\S+)$", text, flags=re.M))
+    if (fields.get("workload") != f"{rows}x{cols}_k{k}" or
+            fields.get("kernel_sources_sha256") != topk_sources_sha256()):
+        return None
+    return int(fields["traffic_bytes_per_launch"])
 
 
-def gemm_knn(bitsknn, torch, dev, q=4096, n=1 << 20, d=64, k=64, runs=5):
-    """Config 4: ||p||^2 - 2 q.p on MFMA into a q x n matrix (16 GiB), then bits top-k on it."""
-    gen = torch.Generator(device=dev)
-    gen.manual_seed(24)
-    points = torch.rand((d, n), device=dev, generator=gen)
-    queries = torch.rand((d, q), device=dev, generator=gen)
-    dist = torch.empty((q, n), dtype=torch.float32, device=dev)
-    out_d = torch.empty((q, k), dtype=torch.float32, device=dev)
-    out_l = torch.empty((q, k), dtype=torch.int32, device=dev)
+class Timer:
+    """Mean duration of launches on the current stream, from events around every launch."""
 
-    def timed(fn):
-        for _ in range(2):
+    def __init__(self, torch):
+        self.torch = torch
+
+    def run(self, fn, steps, warmup):
+        torch = self.torch
+        for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        for _ in range(runs):
+        starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        t0 = time.perf_counter()
+        for i in range(steps):
+            starts[i].record()
             fn()
-        end.record()
+            ends[i].record()
         torch.cuda.synchronize()
-        return start.elapsed_time(end) / 1e3 / runs
-
-    t_dist = timed(lambda: bitsknn.distances(queries, points, bitsknn.DIST_PARTIAL_L2, out=dist))
-    t_split = timed(lambda: bitsknn.distances(queries, points, bitsknn.DIST_PARTIAL_L2_BF16X3, out=dist))
-    t_topk = timed(lambda: bitsknn.topk_bits(dist, k, 256, 8, out_dist=out_d, out_label=out_l))
-    tflops = 2.0 * q * n * d / t_dist / 1e12
-    return {"workload": f"GEMM distance + bits, {n} points x {q} queries, d={d}, k={k}",
-            "distance_ms": t_dist * 1e3, "pairs_per_s": q * n / t_dist,
-            "distance_roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_F32_PEAK_TFLOPS,
-                                  "unit": "TFLOP/s", "frac": tflops / MFMA_F32_PEAK_TFLOPS,
-                                  "store_GBps": 4.0 * q * n / t_dist / 1e9},
-            "distance_bf16x3": {"arithmetic": "three bf16 pieces per fp32 operand, six bf16 matrix products per "
-                                              "product, fp32 accumulation",
-                                "ms": t_split * 1e3, "pairs_per_s": q * n / t_split,
-                                "roofline": {"bound": "hbm", "achieved": (4.0 * q * n + 4.0 * (q + n) * d) / t_split / 1e9,
-                                             "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                             "frac": (4.0 * q * n + 4.0 * (q + n) * d) / t_split / 1e9 / HBM_PEAK_GBS}},
-            "selection_ms": t_topk * 1e3, "selection_elements_per_s": q * n / t_topk,
-            "selection_hbm_frac": (4.0 * q * n + 8.0 * q * k) / t_topk / 1e9 / HBM_PEAK_GBS}
+        wall = time.perf_counter() - t0
+        kernel_ms = sum(s.elapsed_time(e) for s, e in zip(starts, ends)) / steps
+        return wall / steps, kernel_ms / 1e3
 
 
-def hard_inputs(bitsknn, torch, dev, rows=16384, cols=65536, runs=5):
+def sample_indices(count, samples):
+    step = max(1, count // samples)
+    return list(range(step // 2, count, step))[:samples]
+
+
+def verify_topk(oracle, cache, matrix, sample, k, out_d, out_l):
+    """Bit-exact comparison of the sampled rows with the oracle's top-k of the same rows."""
+    import numpy as np
+    key = (id(matrix), k)
+    if key not in cache:
+        host = cache.setdefault((id(matrix), "rows"), matrix[sample].cpu().numpy())
+        cache[key] = oracle.topk(host, k)
+    exp_d, exp_l = cache[key]
+    got_d = out_d[sample].cpu().numpy()
+    got_l = out_l[sample].cpu().numpy()
+    return bool(np.array_equal(got_d.view(np.uint32), exp_d.view(np.uint32)) and np.array_equal(got_l, exp_l))
+
+
+def verify_neighbours(np, points, queries, exp_d, exp_l, got_d, got_l, k):
+    """k-th neighbour distance within REL of the scale of its terms (|value| + ||q||^2) and recall
+    >= MIN_RECALL against the oracle's lists of partial distances; a reported point outside the
+    oracle's list counts when its exact distance is within the tolerance of the k-th distance
+    (neighbours closer together than fp32 resolves).  Also returns the error of the completed
+    k-th distance (value + ||q||^2) relative to itself, for the record."""
+    qn = (queries.astype(np.float64) ** 2).sum(1)
+    kth_e = exp_d[:, k - 1].astype(np.float64)
+    kth_g = got_d[:, k - 1].astype(np.float64)
+    scale = np.abs(kth_e) + qn
+    err_scale = float(np.max(np.abs(kth_g - kth_e) / scale))
+    err_completed = float(np.max(np.abs(kth_g - kth_e) / np.maximum(kth_e + qn, 1e-30)))
+    hits = 0
+    for row in range(queries.shape[0]):
+        want = set(exp_l[row].tolist())
+        for label in got_l[row].tolist():
+            if label in want:
+                hits += 1
+                continue
+            p = points[label].astype(np.float64)
+            exact = float((p * p).sum() - 2.0 * (p * queries[row].astype(np.float64)).sum())
+            hits += exact <= kth_e[row] + REL * scale[row]
+    recall = hits / (queries.shape[0] * k)
+    ascending = bool(np.all(got_d[:, 1:] >= got_d[:, :-1]))
+    ok = err_scale <= REL and recall >= MIN_RECALL and ascending
+    return ok, {"kth_err_of_scale": err_scale, "kth_err_of_completed_distance": err_completed, "recall": recall}
+
+
+def leg_calibration(bitsknn, torch, timer, matrix, steps):
+    rows, cols = matrix.shape
+    out = torch.empty(rows, dtype=torch.float32, device=matrix.device)
+    _, seconds = timer.run(lambda: bitsknn.stream_read(matrix, out), steps, 3)
+    verified = bool(torch.equal(out, matrix.min(dim=1).values))
+    gbs = 4.0 * rows * cols / seconds / 1e9
+    src = torch.empty(1 << 28, dtype=torch.float32, device=matrix.device).fill_(1.0)
+    dst = torch.empty_like(src)
+    _, copy_s = timer.run(lambda: dst.copy_(src), 3, 1)
+    return {"streaming_read": {"workload": f"row minima of the {rows}x{cols} matrix, 256 threads per row, "
+                                           "two 16-byte non-temporal loads in flight per thread",
+                               "GBps": gbs, "frac": gbs / HBM_PEAK_GBS, "ms": seconds * 1e3, "verified": verified},
+            "device_copy": {"bytes_read_per_copy": 1 << 30, "bytes_written_per_copy": 1 << 30, "copies": 4,
+                            "GBps_read_plus_written": 2.0 * (1 << 30) / copy_s / 1e9}}
+
+
+def leg_sweep(bitsknn, torch, timer, oracle, matrix, batch, steps, check):
+    from bitsknn import tuning
+    rows, cols = matrix.shape
+    cache = {}
+    sample = sample_indices(rows, 8)
+    out = []
+    for k in (16, 32, 128, 512, 2048):
+        out_d = torch.empty((rows, k), dtype=torch.float32, device=matrix.device)
+        out_l = torch.empty((rows, k), dtype=torch.int32, device=matrix.device)
+        tuned_block, _, tuned_batch, _, _ = tuning.config_algorithm("bits", rows, k)
+        cases = [(block, batch, False) for block in (128, 256, 512) if k // block <= 16]
+        cases.append((tuned_block, tuned_batch, True))
+        for block, items, tuned in cases:
+            out_d.fill_(-1.0)
+            s, ks = timer.run(lambda: bitsknn.topk_bits(matrix, k, block, items, out_dist=out_d, out_label=out_l),
+                              steps, 3)
+            entry = {"k": k, "block": block, "items_per_thread": items, "elements_per_s": rows * cols / s,
+                     "kernel_ms": ks * 1e3, "frac": (4.0 * rows * cols + 8.0 * rows * k) / ks / 1e9 / HBM_PEAK_GBS}
+            if tuned:
+                entry["tuned"] = True
+            if check:
+                entry["verified"] = verify_topk(oracle, cache, matrix, sample, k, out_d, out_l)
+            out.append(entry)
+    return out
+
+
+def leg_hard(bitsknn, torch, timer, oracle, dev, steps, check, rows=16384, cols=65536):
     """Config 3: rows sorted ascending, descending, or drawn from 256 distinct values."""
     gen = torch.Generator(device=dev)
     gen.manual_seed(24)
@@ -125,53 +205,160 @@ def hard_inputs(bitsknn, torch, dev, rows=16384, cols=65536, runs=5):
     asc = torch.sort(base, dim=1).values
     inputs = {"ascending": asc, "descending": torch.flip(asc, dims=[1]).contiguous(),
               "256-values": torch.floor(base * 256) / 256}
+    del base
+    sample = sample_indices(rows, 32)
     out = []
     for name, matrix in inputs.items():
+        cache = {}
         for k in (32, 256):
-            out_d = torch.empty((rows, k), dtype=torch.float32, device=dev)
+            out_d = torch.full((rows, k), -1.0, dtype=torch.float32, device=dev)
             out_l = torch.empty((rows, k), dtype=torch.int32, device=dev)
             # block 128 with batches of 8: the best single choice over the six cases on this shape
-            _, kernel_s = topk_pass(bitsknn, torch, matrix, k, 128, 8, False, out_d, out_l, runs, 2)
-            out.append({"rows": name, "k": k, "block": 128, "items_per_thread": 8, "elements_per_s": rows * cols / kernel_s,
-                        "hbm_frac": (4.0 * rows * cols + 8.0 * rows * k) / kernel_s / 1e9 / HBM_PEAK_GBS})
+            _, ks = timer.run(lambda: bitsknn.topk_bits(matrix, k, 128, 8, out_dist=out_d, out_label=out_l),
+                              steps, 2)
+            entry = {"rows": name, "k": k, "block": 128, "items_per_thread": 8,
+                     "elements_per_s": rows * cols / ks, "kernel_ms": ks * 1e3,
+                     "frac": (4.0 * rows * cols + 8.0 * rows * k) / ks / 1e9 / HBM_PEAK_GBS}
+            if check:
+                entry["verified"] = verify_topk(oracle, cache, matrix, sample, k, out_d, out_l)
+            out.append(entry)
     return out
 
 
-def copy_calibration(torch, dev, gib=1, reps=3):
-    """A plain device-to-device copy of known size, so that byte counters read under a profiler
-    can be scaled (bytes read = bytes written = gib GiB per copy)."""
-    src = torch.empty(gib << 28, dtype=torch.float32, device=dev).fill_(1.0)
-    dst = torch.empty_like(src)
-    torch.cuda.synchronize()
-    for _ in range(reps):
-        dst.copy_(src)
-    torch.cuda.synchronize()
-    return {"bytes_read_per_copy": gib << 30, "bytes_written_per_copy": gib << 30, "copies": reps}
-
-
-def topk_pass(bitsknn, torch, matrix, k, block, batch, prefetch, out_d, out_l, steps, warmup):
-    for _ in range(warmup):
-        bitsknn.topk_bits(matrix, k, block, batch, prefetch, out_dist=out_d, out_label=out_l)
-    torch.cuda.synchronize()
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    t0 = time.perf_counter()
-    for i in range(steps):
-        starts[i].record()
-        bitsknn.topk_bits(matrix, k, block, batch, prefetch, out_dist=out_d, out_label=out_l)
-        ends[i].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    kernel_ms = sum(s.elapsed_time(e) for s, e in zip(starts, ends)) / steps
-    return wall / steps, kernel_ms / 1e3
-
-
-def cpu_baseline(rows, cols, k, budget_s=12.0):
-    """Reference CPU path (OpenMP heap per row) restated in oracle/, on config 1's matrix."""
+def leg_gemm(bitsknn, torch, timer, oracle, dev, steps, check, q=4096, n=1 << 20, d=64, k=64):
+    """Config 4: ||p||^2 - 2 q.p on MFMA into a q x n matrix (16 GiB), then bits top-k on it."""
     import numpy as np
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(24)
+    points = torch.rand((d, n), device=dev, generator=gen)
+    queries = torch.rand((d, q), device=dev, generator=gen)
+    dist = torch.empty((q, n), dtype=torch.float32, device=dev)
+    out_d = torch.full((q, k), -1.0, dtype=torch.float32, device=dev)
+    out_l = torch.empty((q, k), dtype=torch.int32, device=dev)
+    _, t_split = timer.run(lambda: bitsknn.distances(queries, points, bitsknn.DIST_PARTIAL_L2_BF16X3, out=dist),
+                           steps, 2)
+    dist.fill_(-1.0)
+    _, t_dist = timer.run(lambda: bitsknn.distances(queries, points, bitsknn.DIST_PARTIAL_L2, out=dist), steps, 2)
+    _, t_topk = timer.run(lambda: bitsknn.topk_bits(dist, k, 256, 8, out_dist=out_d, out_label=out_l), steps, 2)
+    tflops = 2.0 * q * n * d / t_dist / 1e12
+    bytes_dist = 4.0 * q * n + 4.0 * (q + n) * d
+    result = {"workload": f"GEMM distance + bits, {n} points x {q} queries, d={d}, k={k}",
+              "distance_ms": t_dist * 1e3, "pairs_per_s": q * n / t_dist,
+              "frac": tflops / MFMA_F32_PEAK_TFLOPS,
+              "distance_roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_F32_PEAK_TFLOPS,
+                                    "unit": "TFLOP/s", "frac": tflops / MFMA_F32_PEAK_TFLOPS,
+                                    "store_GBps": 4.0 * q * n / t_dist / 1e9,
+                                    "hbm_frac": bytes_dist / t_dist / 1e9 / HBM_PEAK_GBS},
+              "distance_bf16x3": {"arithmetic": "three bf16 pieces per fp32 operand, six bf16 matrix products per "
+                                                "product, fp32 accumulation",
+                                  "ms": t_split * 1e3, "pairs_per_s": q * n / t_split,
+                                  "roofline": {"bound": "hbm", "achieved": bytes_dist / t_split / 1e9,
+                                               "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                               "frac": bytes_dist / t_split / 1e9 / HBM_PEAK_GBS}},
+              "selection_ms": t_topk * 1e3, "selection_elements_per_s": q * n / t_topk,
+              "selection_frac": (4.0 * q * n + 8.0 * q * k) / t_topk / 1e9 / HBM_PEAK_GBS}
+    if check:
+        sample = sample_indices(q, 16)
+        points_h = np.ascontiguousarray(points.cpu().numpy().T)
+        queries_h = np.ascontiguousarray(queries[:, sample].cpu().numpy().T)
+        part = oracle.dist(queries_h, points_h, "partial")
+        got_rows = dist[sample].cpu().numpy()
+        qn = (queries_h.astype(np.float64) ** 2).sum(1)[:, None]
+        matrix_err = float(np.max(np.abs(got_rows.astype(np.float64) - part) / (np.abs(part) + qn)))
+        # the selection is exact on the matrix it was given ...
+        sel_d, sel_l = oracle.topk(got_rows, k)
+        got_d = out_d[sample].cpu().numpy()
+        got_l = out_l[sample].cpu().numpy()
+        exact = bool(np.array_equal(got_d.view(np.uint32), sel_d.view(np.uint32)) and np.array_equal(got_l, sel_l))
+        # ... and the neighbours are the reference arithmetic's
+        exp_d, exp_l = oracle.topk(part, k)
+        ok, detail = verify_neighbours(np, points_h, queries_h, exp_d, exp_l, got_d, got_l, k)
+        detail["matrix_err_of_scale"] = matrix_err
+        detail["selection_bit_exact_on_the_matrix"] = exact
+        result["verified"] = bool(ok and exact and matrix_err <= REL)
+        result["verification"] = detail
+    return result
+
+
+def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=65536, n=1 << 20):
+    """Config 5: bits-fused at d x k; the d = 32, k = 32 case also with bf16x3 products."""
+    import numpy as np
+    grid = []
+    headline = None
+    sample = sample_indices(q, 64)
+    for d in dims:
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(24 + d)
+        points = torch.rand((d, n), device=dev, generator=gen)
+        queries = torch.rand((d, q), device=dev, generator=gen)
+        part = None
+        for k in ks:
+            out_d = torch.full((q, k), -1.0, dtype=torch.float32, device=dev)
+            out_l = torch.empty((q, k), dtype=torch.int32, device=dev)
+            _, seconds = timer.run(lambda: bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l),
+                                   steps, 1)
+            tflops = 2.0 * q * n * d / seconds / 1e12
+            entry = {"d": d, "k": k, "ms": seconds * 1e3, "queries_per_s": q / seconds,
+                     "pairs_per_s": q * n / seconds, "frac": tflops / MFMA_F32_PEAK_TFLOPS}
+            if check:
+                if part is None:
+                    points_h = np.ascontiguousarray(points.cpu().numpy().T)
+                    queries_h = np.ascontiguousarray(queries[:, sample].cpu().numpy().T)
+                    part = oracle.dist(queries_h, points_h, "partial")
+                exp_d, exp_l = oracle.topk(part, k)
+                ok, detail = verify_neighbours(np, points_h, queries_h, exp_d, exp_l, out_d[sample].cpu().numpy(),
+                                               out_l[sample].cpu().numpy(), k)
+                entry["verified"] = bool(ok)
+                entry["verification"] = detail
+            grid.append(entry)
+            if d == 32 and k == 32:
+                headline = {"workload": f"bits-fused, {n} points x {q} queries, d={d}, k={k}, fp32 uniform[0,1)",
+                            "arithmetic": "fp32 matrix instructions",
+                            "queries_per_s": q / seconds, "ms": seconds * 1e3, "pairs_per_s": q * n / seconds,
+                            "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_F32_PEAK_TFLOPS,
+                                         "unit": "TFLOP/s", "frac": tflops / MFMA_F32_PEAK_TFLOPS}}
+                if check:
+                    headline["verified"] = entry["verified"]
+                out_d.fill_(-1.0)
+                _, split_s = timer.run(
+                    lambda: bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l,
+                                                  arithmetic=bitsknn.FUSED_BF16X3), steps, 1)
+                split_tflops = 6 * 2.0 * q * n * d / split_s / 1e12
+                headline["bf16x3"] = {
+                    "arithmetic": "three bf16 pieces per fp32 operand, six bf16 matrix products per product, "
+                                  "fp32 accumulation",
+                    "queries_per_s": q / split_s, "ms": split_s * 1e3, "pairs_per_s": q * n / split_s,
+                    "roofline": {"bound": "mfma", "achieved": split_tflops, "peak": MFMA_BF16_PEAK_TFLOPS,
+                                 "unit": "TFLOP/s", "frac": split_tflops / MFMA_BF16_PEAK_TFLOPS}}
+                if check:
+                    ok, detail = verify_neighbours(np, points_h, queries_h, exp_d, exp_l,
+                                                   out_d[sample].cpu().numpy(), out_l[sample].cpu().numpy(), k)
+                    headline["bf16x3"]["verified"] = bool(ok)
+        del points, queries
+    result = headline if headline is not None else {"workload": "bits-fused, restricted grid"}
+    result["grid"] = grid
+    return result
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as handle:
+            for line in handle:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def leg_cpu(rows, cols, k, budget_s=8.0):
+    """The reference's CPU paths restated in oracle/, on config 1's matrix: the OpenMP heap per row
+    on the host cores this job may use, and the full sort of every row on one core."""
     from oracle import binding as oracle
     m = oracle.uniform_matrix(24, rows, cols)
-    threads = min(16, os.cpu_count() or 1)
+    # the cores this job may use: the OpenMP setting of the environment when there is one (a GPU
+    # box hands a job a share of its cores), else every core of the host
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1)
     reps, spent = 0, 0.0
     oracle.topk_parallel(m, k, threads)  # warm
     while spent < budget_s and reps < 50:
@@ -179,9 +366,16 @@ def cpu_baseline(rows, cols, k, budget_s=12.0):
         _, _, used = oracle.topk_parallel(m, k, threads)
         spent += time.perf_counter() - t0
         reps += 1
+    t0 = time.perf_counter()
+    oracle.topk_serial(m, k)
+    serial_s = time.perf_counter() - t0
     return {"value": rows * cols * reps / spent, "unit": "elements/s", "cores": used, "kind": "port",
             "sample": f"{reps} passes of parallel_knn::selection restated (OpenMP heap) over a "
-                      f"{rows}x{cols} fp32 uniform matrix, k={k}"}
+                      f"{rows}x{cols} fp32 uniform matrix, k={k} (the GPU figure is for {rows}x1048576)",
+            "cpu_model": cpu_model(), "host_cpus": os.cpu_count(),
+            "serial": {"value": rows * cols / serial_s, "unit": "elements/s", "cores": 1,
+                       "sample": f"one pass of serial_knn::selection restated (std::sort of every row) over "
+                                 f"the same {rows}x{cols} matrix"}}
 
 
 def main():
@@ -195,104 +389,84 @@ def main():
     ap.add_argument("--prefetch", action="store_true", help="the bits-prefetch variant")
     ap.add_argument("--rows", type=int, default=1024)
     ap.add_argument("--cols", type=int, default=1 << 20)
-    ap.add_argument("--sweep", action="store_true", help="also time k x block-size combinations")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-fused", action="store_true", help="skip the bits-fused headline figure")
-    ap.add_argument("--no-topk", action="store_true", help="skip the top-k leg (profiling other kernels)")
-    ap.add_argument("--gemm-knn", action="store_true",
-                    help="also time config 4: MFMA distance matrix (16 GiB) + bits top-k")
-    ap.add_argument("--hard-inputs", action="store_true",
-                    help="also time config 3: 16384 x 65536 sorted / heavily tied rows, k = 32, 256")
-    ap.add_argument("--copy-calibration", action="store_true",
-                    help="also run plain 1 GiB device copies (reference traffic for byte counters)")
+    ap.add_argument("--only", default="", help="comma-separated legs to run: " + ", ".join(LEGS))
+    ap.add_argument("--skip", default="", help="comma-separated legs to leave out")
+    ap.add_argument("--fused-d", type=int, default=0, help="restrict the fused grid to this dimension")
+    ap.add_argument("--fused-k", type=int, default=0, help="restrict the fused grid to this list length")
+    ap.add_argument("--no-verify", action="store_true", help="leave out the comparison with the oracle")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (--gpus 1); multi-GPU figures are not "
               "part of it", file=sys.stderr)
         sys.exit(2)
+    legs = set(x for x in args.only.split(",") if x) or set(LEGS)
+    legs -= set(x for x in args.skip.split(",") if x)
+    unknown = legs - set(LEGS)
+    if unknown:
+        print(f"bench.py: unknown legs {sorted(unknown)}; known: {', '.join(LEGS)}", file=sys.stderr)
+        sys.exit(2)
 
     import torch
     import bitsknn
     bitsknn.lib()
+    check = not args.no_verify
+    oracle = None
+    if check:
+        from oracle import binding as oracle  # the checker of every leg, never the thing measured
+        oracle.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    timer = Timer(torch)
     rows, cols = args.rows, args.cols
-    prefetch = args.prefetch
-    if args.no_topk:
-        result = {"metric": "bits top-k selected-from elements/s (rows*cols / step time)", "value": None,
-                  "unit": "elements/s", "n_gpus": 1, "config": {"workload": "top-k leg skipped"}}
-        if not args.no_fused:
-            result["fused"] = fused_headline(bitsknn, torch, dev, runs=max(1, args.steps))
-        if args.gemm_knn:
-            result["gemm_knn"] = gemm_knn(bitsknn, torch, dev)
-        print(json.dumps(result))
-        return
-    gen = torch.Generator(device=dev)
-    gen.manual_seed(24)
-    matrix = torch.rand((rows, cols), device=dev, generator=gen)
+    few = max(3, args.steps // 4)
 
-    def run(k, block, batch, steps, warmup):
-        out_d = torch.empty((rows, k), dtype=torch.float32, device=dev)
-        out_l = torch.empty((rows, k), dtype=torch.int32, device=dev)
-        return topk_pass(bitsknn, torch, matrix, k, block, batch, prefetch, out_d, out_l, steps, warmup)
+    result = {"metric": "bits top-k selected-from elements/s (rows*cols / step time)", "value": None,
+              "unit": "elements/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None,
+              "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+              "data": "synthetic",
+              "config": {"workload": f"bits top-k, fp32 matrix {rows}x{cols} uniform[0,1) resident in HBM, "
+                                     f"k={args.k}, block {args.block_size}, items/thread {args.items_per_thread}, "
+                                     f"prefetch {int(args.prefetch)}"}}
 
-    step_s, kernel_s = run(args.k, args.block_size, args.items_per_thread, args.steps, args.warmup)
-    bytes_alg = 4.0 * rows * cols + 8.0 * rows * args.k
-    achieved = bytes_alg / kernel_s / 1e9
-
-    result = {
-        "metric": "bits top-k selected-from elements/s (rows*cols / step time)",
-        "value": rows * cols / step_s,
-        "unit": "elements/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": step_s * 1e3,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic",
-        "config": {"workload": f"bits top-k, fp32 matrix {rows}x{cols} uniform[0,1) resident in HBM, "
-                               f"k={args.k}, block {args.block_size}, items/thread {args.items_per_thread}, "
-                               f"prefetch {int(prefetch)}"},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((rows, cols, args.k)),
-                     "kernel_ms": kernel_s * 1e3, "algorithmic_bytes": bytes_alg},
-    }
-
-    if args.sweep:
-        from bitsknn import tuning
-        sweep = []
-        for k in (16, 32, 128, 512, 2048):
-            for block in (128, 256, 512):
-                if k // block > 16:
-                    continue
-                s, ks = run(k, block, args.items_per_thread, max(5, args.steps // 2), 3)
-                sweep.append({"k": k, "block": block, "items_per_thread": args.items_per_thread,
-                              "elements_per_s": rows * cols / s,
-                              "hbm_frac": (4.0 * rows * cols + 8.0 * rows * k) / ks / 1e9 / HBM_PEAK_GBS})
-            # the configuration the shipped optima file names for this problem
-            block, _, batch, _, _ = tuning.config_algorithm("bits", rows, k)
-            s, ks = run(k, block, batch, max(5, args.steps // 2), 3)
-            sweep.append({"k": k, "block": block, "items_per_thread": batch, "tuned": True,
-                          "elements_per_s": rows * cols / s,
-                          "hbm_frac": (4.0 * rows * cols + 8.0 * rows * k) / ks / 1e9 / HBM_PEAK_GBS})
-        result["sweep"] = sweep
-
-    del matrix
-    torch.cuda.empty_cache()
-    if args.copy_calibration:
-        result["copy_calibration"] = copy_calibration(torch, dev)
-    if not args.no_fused:
-        result["fused"] = fused_headline(bitsknn, torch, dev)
-    if args.gemm_knn:
-        result["gemm_knn"] = gemm_knn(bitsknn, torch, dev)
-    if args.hard_inputs:
-        result["hard_inputs"] = hard_inputs(bitsknn, torch, dev)
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(1024, 65536, 32)
+    if legs & {"headline", "calibration", "sweep"}:
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(24)
+        matrix = torch.rand((rows, cols), device=dev, generator=gen)
+        if "headline" in legs:
+            k = args.k
+            out_d = torch.full((rows, k), -1.0, dtype=torch.float32, device=dev)
+            out_l = torch.empty((rows, k), dtype=torch.int32, device=dev)
+            step_s, kernel_s = timer.run(
+                lambda: bitsknn.topk_bits(matrix, k, args.block_size, args.items_per_thread, args.prefetch,
+                                          out_dist=out_d, out_label=out_l), args.steps, args.warmup)
+            bytes_alg = 4.0 * rows * cols + 8.0 * rows * k
+            achieved = bytes_alg / kernel_s / 1e9
+            result["value"] = rows * cols / step_s
+            result["ms_per_step"] = step_s * 1e3
+            result["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                  "frac": achieved / HBM_PEAK_GBS, "traffic": profiled_traffic(rows, cols, k),
+                                  "kernel_ms": kernel_s * 1e3, "algorithmic_bytes": bytes_alg}
+            if check:
+                result["verified"] = verify_topk(oracle, {}, matrix, sample_indices(rows, 8), k, out_d, out_l)
+        if "calibration" in legs:
+            result["calibration"] = leg_calibration(bitsknn, torch, timer, matrix, few)
+        if "sweep" in legs:
+            result["sweep"] = leg_sweep(bitsknn, torch, timer, oracle, matrix, args.items_per_thread, few, check)
+        del matrix
+        torch.cuda.empty_cache()
+    if "hard" in legs:
+        result["hard_inputs"] = leg_hard(bitsknn, torch, timer, oracle, dev, few, check)
+        torch.cuda.empty_cache()
+    if "gemm" in legs:
+        result["gemm_knn"] = leg_gemm(bitsknn, torch, timer, oracle, dev, few, check)
+        torch.cuda.empty_cache()
+    if "fused" in legs:
+        dims = (args.fused_d,) if args.fused_d else (8, 16, 32)
+        ks = (args.fused_k,) if args.fused_k else (4, 16, 32)
+        result["fused"] = leg_fused(bitsknn, torch, timer, oracle, dev, max(2, args.steps // 10), check, dims, ks)
+        torch.cuda.empty_cache()
+    if "cpu" in legs:
+        result["cpu_baseline"] = leg_cpu(1024, 65536, 32)
     print(json.dumps(result))
 
 

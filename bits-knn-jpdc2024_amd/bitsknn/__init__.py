@@ -23,6 +23,7 @@ EXPORTS = (
     "bitsknn_topk_partial_bitonic_f32",
     "bitsknn_label_offsets",
     "bitsknn_fill_f32",
+    "bitsknn_stream_read_f32",
     "bitsknn_dist_f32",
     "bitsknn_fused_l2_topk_f32",
     "bitsknn_fused_workspace_bytes",
@@ -69,6 +70,8 @@ def lib():
         L.bitsknn_label_offsets.argtypes = [vp, sz, sz, sz, vp]
         L.bitsknn_fill_f32.restype = ctypes.c_int
         L.bitsknn_fill_f32.argtypes = [vp, sz, ctypes.c_float, vp]
+        L.bitsknn_stream_read_f32.restype = ctypes.c_int
+        L.bitsknn_stream_read_f32.argtypes = [vp, sz, sz, sz, vp, vp]
         L.bitsknn_dist_f32.restype = ctypes.c_int
         L.bitsknn_dist_f32.argtypes = [ctypes.c_int, ctypes.c_int, sz, sz, vp, sz, vp, sz, vp, sz, vp]
         L.bitsknn_fused_l2_topk_f32.restype = ctypes.c_int
@@ -168,6 +171,16 @@ def label_offsets(rows, parts, cols_per_part, device="cuda"):
 def fill(t, value):
     _check(lib().bitsknn_fill_f32(_ptr(t), t.numel(), float(value), _stream()))
     return t
+
+
+def stream_read(matrix, out=None):
+    """Row minima by a plain streaming read (calibration of the achievable read rate)."""
+    import torch
+    rows, cols = matrix.shape
+    if out is None:
+        out = torch.empty(rows, dtype=torch.float32, device=matrix.device)
+    _check(lib().bitsknn_stream_read_f32(_ptr(matrix), _row_stride(matrix), rows, cols, _ptr(out), _stream()))
+    return out
 
 
 def distances(queries_dm, points_dm, op=DIST_L2, out=None):

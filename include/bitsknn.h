@@ -93,6 +93,16 @@ int bitsknn_label_offsets(int32_t* offsets, size_t rows, size_t parts, size_t co
 int bitsknn_fill_f32(float* dst, size_t count, float value, void* stream);
 
 /*
+ * Calibration: the minimum of every row of a rows x cols fp32 matrix by a plain streaming read with
+ * the row-per-workgroup mapping and the 16-byte non-temporal loads of the top-k kernel and no
+ * other work.  Its rate is the read rate such a kernel can reach on the machine at hand, the
+ * yardstick next to the published HBM peak.  No counterpart in the reference.
+ * Rows must start on 16-byte boundaries (BITSKNN_ERR_INVALID otherwise).
+ */
+int bitsknn_stream_read_f32(const float* in, size_t in_row_stride, size_t rows, size_t cols,
+                            float* row_min, void* stream);
+
+/*
  * Distance matrix dist[i*dist_row_stride + j] between query i and point j, inputs dim-major
  * (component t of vector v at base[t*stride + v]), as the reference uploads them
  * (src/distance/magma_distance.cu:13-71).
