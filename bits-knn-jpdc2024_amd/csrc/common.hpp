@@ -40,7 +40,8 @@ void clear_error();
 // A (value, label) pair is held as one unsigned 64-bit key whose integer order is the
 // lexicographic order (value ascending as IEEE floats, then label ascending as int32).  A
 // sorting network over such keys is a total order, so equal values always come out by lower
-// label.  -0.0 is folded onto +0.0 (they compare equal as floats); NaNs sort after +inf.
+// label.  -0.0 is folded onto +0.0 (they compare equal as floats); a NaN of either sign takes the
+// key of +inf, so that every path treats it as +inf (and writes it back as +inf).
 
 __host__ __device__ __forceinline__ u32 float_key(float v)
 {
@@ -49,7 +50,7 @@ __host__ __device__ __forceinline__ u32 float_key(float v)
         float f;
         u32 u;
     } c;
-    c.f = v + 0.0F; // -0.0 -> +0.0
+    c.f = fminf(v + 0.0F, __builtin_inff()); // -0.0 -> +0.0, NaN -> +inf
     const u32 b = c.u;
     return b ^ (static_cast<u32>(static_cast<std::int32_t>(b) >> 31) | 0x80000000U);
 }

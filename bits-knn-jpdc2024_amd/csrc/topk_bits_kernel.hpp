@@ -372,10 +372,11 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     };
 
     // exact filter: below the radius key (an equal value is decided by its label; the +inf
-    // padding of a ragged tail never passes)
+    // padding of a ragged tail never passes).  A NaN counts as +inf: it is neither below nor above
+    // the radius and its key decides, which can only succeed while the radius is +inf.
     auto passes = [&](float value, int j) -> bool {
         bool pass = value < radius;
-        if (value == radius)
+        if (!(value < radius) && !(value > radius))
         {
             const u32 col = column_of(cur_chunk, j);
             pass = col < n && make_key(value, label_of(col)) < radius_key;
@@ -504,11 +505,14 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
                 }
             }
 
+            // NaN-propagating minimum (v_minimum3_f32): a lane that holds a NaN of any kind gets a NaN
+            // here and takes the look at every value below (the NaN-ignoring minimum would need
+            // every operand quietened first, and loses values after a signalling NaN otherwise)
             float smallest = v[0];
 #pragma unroll
             for (int j = 1; j < E; ++j)
             {
-                smallest = fminf(smallest, v[j]);
+                smallest = __builtin_elementwise_minimum(smallest, v[j]);
             }
             // A value equal to the radius passes only with a label below the radius key's.  With
             // implicit labels every label of this chunk is at least that of its first column, so
@@ -516,13 +520,14 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
             // values have one in every chunk).
             const bool no_ties =
                 lrow == nullptr && static_cast<std::int32_t>(cur_chunk + label_offset) >= key_label(radius_key);
-            if (__builtin_amdgcn_ballot_w64(no_ties ? smallest < radius : smallest <= radius) != 0)
+            // (negated compares: true for a NaN)
+            if (__builtin_amdgcn_ballot_w64(no_ties ? !(smallest >= radius) : !(smallest > radius)) != 0)
             {
                 int running = fill;
 #pragma unroll
                 for (int j = 0; j < E; ++j)
                 {
-                    if (__builtin_amdgcn_ballot_w64(v[j] <= radius) != 0)
+                    if (__builtin_amdgcn_ballot_w64(!(v[j] > radius)) != 0)
                     {
                         const bool pass = passes(v[j], j);
                         const u64 mask = __builtin_amdgcn_ballot_w64(pass);

@@ -42,3 +42,13 @@ def dev():
     if not torch.cuda.is_available():
         pytest.fail("GPU test selected but no GPU is visible")
     return torch.device("cuda:0")
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """The largest k-th-neighbour distance errors the floating-point parity checks met (pytest -s)."""
+    try:
+        import parity
+    except ImportError:
+        return
+    for key, seen in sorted(parity.margins.items()):
+        print("\nparity margin %s: %s" % (key, ", ".join("%s %.3g" % kv for kv in sorted(seen.items()))))

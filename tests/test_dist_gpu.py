@@ -1,12 +1,15 @@
 """Parity of the distance kernels (through the C ABI) with the CPU oracle.
 
 Bars: BITSKNN_DIST_L2 bit-exact (sequential fused multiply-add, the reference's default
-distance); the MFMA kernels within 1e-5 relative of the oracle's partial distance measured
-against the magnitude of the terms (||p||^2 and 2|q.p| cancel), and the completed distance
-within the reference test's own tolerances (tests/distance/dist_test.hpp:93-115, 164-186).
+distance); the MFMA kernels within 1e-5 of the oracle's partial distance relative to the
+magnitude of the terms that cancel in it (||p||^2 and 2|q.p|), the k-th neighbour distance of
+every query to the contract's bar (tests/parity.py), and the completed distance within the
+reference test's own tolerances (tests/distance/dist_test.hpp:93-115, 164-186).
 """
 import numpy as np
 import pytest
+
+from parity import assert_kth_distance
 
 pytestmark = pytest.mark.gpu
 
@@ -59,10 +62,14 @@ def test_mfma_distances(bk, dev, oracle, n, q, d, op):
     got = _gpu_dist(bk, dev, s, p, bk.DIST_PARTIAL_L2 if op == "partial" else bk.DIST_EXPANDED)
     exp = oracle.dist(s, p, "partial")
     truth = oracle.dist(s, p, "f64-partial")
-    # scale of the cancelling terms: ||p||^2 + 2|q.p| <= ||p||^2 + ||q||^2 + ||p||^2
-    scale = (p.astype(np.float64) ** 2).sum(1)[None, :] * 2 + (s.astype(np.float64) ** 2).sum(1)[:, None]
+    # the terms that cancel in an entry: ||p||^2 and 2|q.p| (exact values)
+    p64, s64 = p.astype(np.float64), s.astype(np.float64)
+    scale = (p64 ** 2).sum(1)[None, :] + 2.0 * np.abs(s64 @ p64.T)
     assert np.max(np.abs(got - exp) / scale) < 1e-5
     assert np.max(np.abs(got - truth) / scale) < 1e-5
+    # the k-th neighbour distance of every query (k = 16, or all points when there are fewer)
+    kk = min(16, n)
+    assert_kth_distance(s, np.sort(exp, axis=1)[:, kk - 1], np.sort(got, axis=1)[:, kk - 1], d, (n, q, d, op))
     # the reference's own check: add ||q||^2 on the CPU, compare with the plain triple loop at 1e-3
     full = got.astype(np.float64) + (s.astype(np.float64) ** 2).sum(1)[:, None]
     ref_full = oracle.dist(s, p, "f64")
@@ -95,10 +102,8 @@ def test_knn_through_both_distances_meets_the_recall_bar(bk, dev, oracle):
     gd, gl = gd.cpu().numpy(), gl.cpu().numpy()
     recall = np.mean([len(set(a) & set(b)) / k for a, b in zip(gl, el)])
     assert recall >= 0.999, recall
-    qn = (s.astype(np.float64) ** 2).sum(1)
-    full_g = gd[:, -1].astype(np.float64) + qn
-    full_e = ed[:, -1].astype(np.float64) + qn
-    assert np.max(np.abs(full_g - full_e) / full_e) < 1e-5
+    completed, _, _ = assert_kth_distance(s, ed[:, -1], gd[:, -1], d, "gemm + bits")
+    assert completed < 1e-5
     # and the top-k of the device matrix itself is bit-exact
     od, ol = oracle.topk(dist.cpu().numpy(), k)
     assert np.array_equal(gd, od) and np.array_equal(gl, ol)

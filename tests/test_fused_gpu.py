@@ -2,18 +2,18 @@
 
 The distances come from fp32 MFMA, so they are not bit-identical to the reference's sequential
 fused multiply-adds.  Bar (the stated tolerance of this path): the k-th neighbour distance within
-1e-5 relative -- measured on the partial distance ||p||^2 - 2 q.p that the reference outputs,
-relative to the magnitude of the quantities it is the difference of (|value| + ||q||^2) -- and
-recall@k >= 0.999 against the oracle's neighbour sets.  Structure is checked exactly: ascending
-order, distinct in-range labels, and every reported distance equal (to the same tolerance) to the
-oracle's distance of the reported label.
+1e-5 relative of the oracle's -- of the completed distance (value + ||q||^2) for dim >= 16, of the
+reported partial distance below that, see tests/parity.py -- and recall@k >= 0.999 against the
+oracle's neighbour sets.  Structure is checked exactly: ascending order, distinct in-range labels,
+and every reported distance equal to the oracle's distance of the reported label (to 1e-5 of the
+magnitude of the terms that cancel in it).
 """
 import numpy as np
 import pytest
 
-pytestmark = pytest.mark.gpu
+from parity import REL, assert_kth_distance
 
-REL = 1e-5
+pytestmark = pytest.mark.gpu
 
 
 def _dm(a, dev):
@@ -46,8 +46,7 @@ def _check(oracle, points, queries, k, gd, gl, min_recall=0.999):
     scale = np.abs(ref_at) + qn
     assert np.max(np.abs(gd[:, :kk] - ref_at) / scale) <= REL
     # k-th neighbour distance and recall
-    scale_k = np.abs(ed[:, kk - 1]) + qn[:, 0]
-    assert np.max(np.abs(gd[:, kk - 1] - ed[:, kk - 1]) / scale_k) <= REL
+    assert_kth_distance(queries, ed[:, kk - 1], gd[:, kk - 1], points.shape[1], (n, queries.shape[0], k))
     recall = np.mean([len(set(a[:kk]) & set(b[:kk])) / kk for a, b in zip(gl, el)])
     if recall < min_recall:
         # Neighbours closer together than fp32 resolves (many points on a line, say): which of

@@ -158,6 +158,43 @@ def test_negative_zero_is_returned_as_positive_zero(bk, dev, oracle):
     assert gd[0, 0] == 0.0 and gd[0, 1] == 0.0 and not np.signbit(gd[0, 0])
 
 
+def test_nans_count_as_plus_infinity(bk, dev, oracle):
+    """A NaN of either sign is treated as +inf everywhere (first values of a row, streamed part,
+    sampled row ends) and is written back as +inf: the result equals the oracle's on the matrix
+    with every NaN replaced by +inf, ties by lower label included."""
+    pos_nan = np.array([0x7FC00000], dtype=np.uint32).view(np.float32)[0]
+    neg_nan = np.array([0xFFC00000], dtype=np.uint32).view(np.float32)[0]   # what 0/0 gives on x86
+    sig_nan = np.array([0x7F800001], dtype=np.uint32).view(np.float32)[0]
+    rng = np.random.default_rng(8)
+    for cols in (3000, 70000):                      # without and with a sampled first radius
+        m = oracle.uniform_matrix(900 + cols, 6, cols, -2.0, 2.0)
+        m[0, :40:3] = neg_nan                       # among the first values of the row
+        m[0, 5] = pos_nan
+        m[1, cols // 2:cols // 2 + 50:2] = neg_nan  # in the streamed part
+        m[1, cols - 7:] = pos_nan                   # at the very end (sampled when the row is long)
+        m[2, rng.permutation(cols)[:cols // 3]] = neg_nan   # a third of the row
+        m[2, rng.permutation(cols)[:cols // 5]] = sig_nan
+        m[3, :] = neg_nan                           # nothing but NaNs ...
+        m[3, 100:110] = np.arange(10, dtype=np.float32)     # ... and ten numbers
+        m[4, :] = pos_nan                           # NaNs, infinities and five numbers: fewer than k
+        m[4, 1::2] = np.inf
+        m[4, [7, 77, 777, 1777, 2777]] = [3.0, -1.0, 2.0, 0.0, 1.0]
+        m[5, :] = neg_nan                           # nothing at all
+        want = np.where(np.isnan(m), np.float32(np.inf), m)
+        for block, batch in ((128, 3), (256, 8), (512, 16)):
+            for k in (1, 16, 40, 256, 1024):
+                gd, gl = _run(bk, dev, m, k, block=block, batch=batch)
+                ed, el = oracle.topk(want, k)
+                assert not np.isnan(gd).any()
+                assert np.array_equal(gd, ed) and np.array_equal(gl, el), (cols, block, batch, k)
+    # the unfiltered baseline builds the same keys
+    import torch
+    gd, gl = bk.topk_partial_bitonic(torch.from_numpy(m).to(dev), 64, 256)
+    torch.cuda.synchronize()
+    ed, el = oracle.topk(want, 64)
+    assert np.array_equal(gd.cpu().numpy(), ed) and np.array_equal(gl.cpu().numpy(), el)
+
+
 def test_k_larger_than_row(bk, dev, oracle):
     m = oracle.uniform_matrix(8, 3, 20)
     _check(bk, dev, oracle, m, 32, block=128, batch=1)
