@@ -22,7 +22,8 @@ which did not do its work cannot produce a figure.
   calibration  a plain streaming read of the same matrix with the same row-per-workgroup mapping
                (the read rate this machine reaches) and 1 GiB device copies (known traffic for
                scaling byte counters read under a profiler)
-  sweep        the 4 GiB matrix at k in {16,32,128,512,2048} x block size {128,256,512}, plus the
+  sweep        the 4 GiB matrix at k in {16,32,128,512,2048} x block size {128,256,512} with 2048
+               values of a row in flight per iteration (16 / 8 / 4 values per thread), plus the
                configuration the shipped optima file names for each k
   hard         16,384 x 65,536 rows sorted ascending / descending / drawn from 256 values, k = 32, 256
   gemm         ||p||^2 - 2 q.p on fp32 MFMA for 1,048,576 points x 4,096 queries, d = 64 (a 16 GiB
@@ -51,6 +52,9 @@ HBM_PEAK_GBS = 8000.0       # MI355X published peak
 MFMA_F32_PEAK_TFLOPS = 157.3  # dense fp32 matrix peak
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 matrix peak
 LEGS = ("headline", "calibration", "sweep", "hard", "gemm", "fused", "cpu")
+# values per thread in the block-size sweep: the same 2048 values of a row in flight per iteration
+# whatever the workgroup size (fewer waves per row need more loads each)
+SWEEP_ITEMS = {128: 16, 256: 8, 512: 4}
 REL = 1e-5
 MIN_RECALL = 0.999
 
@@ -171,7 +175,7 @@ def leg_calibration(bitsknn, torch, timer, matrix, steps):
                             "GBps_read_plus_written": 2.0 * (1 << 30) / copy_s / 1e9}}
 
 
-def leg_sweep(bitsknn, torch, timer, oracle, matrix, batch, steps, check):
+def leg_sweep(bitsknn, torch, timer, oracle, matrix, steps, check):
     from bitsknn import tuning
     rows, cols = matrix.shape
     cache = {}
@@ -181,7 +185,7 @@ def leg_sweep(bitsknn, torch, timer, oracle, matrix, batch, steps, check):
         out_d = torch.empty((rows, k), dtype=torch.float32, device=matrix.device)
         out_l = torch.empty((rows, k), dtype=torch.int32, device=matrix.device)
         tuned_block, _, tuned_batch, _, _ = tuning.config_algorithm("bits", rows, k)
-        cases = [(block, batch, False) for block in (128, 256, 512) if k // block <= 16]
+        cases = [(block, SWEEP_ITEMS[block], False) for block in (128, 256, 512) if k // block <= 16]
         cases.append((tuned_block, tuned_batch, True))
         for block, items, tuned in cases:
             out_d.fill_(-1.0)
@@ -195,6 +199,10 @@ def leg_sweep(bitsknn, torch, timer, oracle, matrix, batch, steps, check):
                 entry["verified"] = verify_topk(oracle, cache, matrix, sample, k, out_d, out_l)
             out.append(entry)
     return out
+
+
+# workgroup size and values per thread of the hard-input leg: the best single choice over its six cases
+HARD_CONFIG = (128, 16)
 
 
 def leg_hard(bitsknn, torch, timer, oracle, dev, steps, check, rows=16384, cols=65536):
@@ -213,10 +221,10 @@ def leg_hard(bitsknn, torch, timer, oracle, dev, steps, check, rows=16384, cols=
         for k in (32, 256):
             out_d = torch.full((rows, k), -1.0, dtype=torch.float32, device=dev)
             out_l = torch.empty((rows, k), dtype=torch.int32, device=dev)
-            # block 128 with batches of 8: the best single choice over the six cases on this shape
-            _, ks = timer.run(lambda: bitsknn.topk_bits(matrix, k, 128, 8, out_dist=out_d, out_label=out_l),
+            block, items = HARD_CONFIG
+            _, ks = timer.run(lambda: bitsknn.topk_bits(matrix, k, block, items, out_dist=out_d, out_label=out_l),
                               steps, 2)
-            entry = {"rows": name, "k": k, "block": 128, "items_per_thread": 8,
+            entry = {"rows": name, "k": k, "block": block, "items_per_thread": items,
                      "elements_per_s": rows * cols / ks, "kernel_ms": ks * 1e3,
                      "frac": (4.0 * rows * cols + 8.0 * rows * k) / ks / 1e9 / HBM_PEAK_GBS}
             if check:
@@ -451,7 +459,7 @@ def main():
         if "calibration" in legs:
             result["calibration"] = leg_calibration(bitsknn, torch, timer, matrix, few)
         if "sweep" in legs:
-            result["sweep"] = leg_sweep(bitsknn, torch, timer, oracle, matrix, args.items_per_thread, few, check)
+            result["sweep"] = leg_sweep(bitsknn, torch, timer, oracle, matrix, few, check)
         del matrix
         torch.cuda.empty_cache()
     if "hard" in legs:

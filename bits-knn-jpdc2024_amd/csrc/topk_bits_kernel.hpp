@@ -335,8 +335,9 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
         }
     };
     // Software pipelining for small batches: the next chunk is requested before the current one
-    // is filtered, at the price of E more registers and E moves per chunk.
-    constexpr bool PIPE = L <= 2;
+    // is filtered, at the price of E more registers and E moves per chunk.  Rows of two waves
+    // (128 threads) leave 8 waves per compute unit, which need the depth also with 4 loads each.
+    constexpr bool PIPE = L <= 2 || (BS == 128 && L <= 4);
     float ahead[E];
 #pragma unroll
     for (int j = 0; j < E; ++j)

@@ -67,10 +67,12 @@ def _tuned(name, rows, k):
 
 
 # (k, block, values per thread, prefetching variant): the benchmark's headline instantiation, its
-# sweep (k x block at 8 values per thread), block 128 at other depths
+# sweep (k x block with 16 / 8 / 4 values per thread), other depths
+SWEEP_ITEMS = {128: 16, 256: 8, 512: 4}
 CONFIG2 = [(32, 256, 8, False)] + \
-          [(k, block, 8, False) for k in (16, 128, 512, 2048) for block in (128, 256, 512) if k // block <= 16] + \
-          [(32, 128, 8, False), (32, 512, 8, False), (16, 128, 16, False), (128, 128, 16, True), (2048, 512, 4, False)]
+          [(k, block, SWEEP_ITEMS[block], False) for k in (16, 32, 128, 512, 2048) for block in (128, 256, 512)
+           if k // block <= 16 and (k, block) != (32, 256)] + \
+          [(32, 128, 8, False), (32, 512, 8, False), (16, 128, 12, False), (128, 128, 8, True), (2048, 512, 8, False)]
 
 
 @pytest.mark.parametrize("k,block,batch,prefetch", CONFIG2)
@@ -119,7 +121,7 @@ def test_hard_rows_at_full_size(bk, dev, oracle, hard_matrices, kind, k):
     m, cache = hard_matrices[kind]
     sample = _sample(m.shape[0], 32)
     tuned = _tuned("bits", m.shape[0], k)
-    for block, batch in {(128, 8), tuned}:
+    for block, batch in {(128, 16), (128, 8), tuned}:
         od, ol = bk.topk_bits(m, k, block, batch)
         torch.cuda.synchronize()
         _check_topk_sample(torch, oracle, cache, m, sample, od, ol, k)
