@@ -3,11 +3,16 @@
 Two halves, matching the reference's tuning workflow:
 
 * ``sweep()`` times `bits` and `bits-prefetch` over the grid of the reference's parameter search
-  (reference scripts/run-opt-ipt.sh:38-47: n = 512k, q in 64..8192, k in 2..2048, batch 1..16,
-  block size 128/256/512), ``sweep_partial_bitonic()`` times `partial-bitonic-regs` over the grid
-  of scripts/run-opt-bitonic-sort.sh:27-43 (q*n = 2^30, q in 64..4096, k in 32..2048, block size
-  64..512), and ``write_optima()`` keeps the fastest configuration of every (algorithm, q, k)
-  in a CSV with the columns of the reference's scripts/optima.csv
+  (reference scripts/run-opt-ipt.sh:38-47: n = 512k, q in 64..8192, k in 2..2048, block size
+  128/256/512; of its batch sizes 1..16 only 4, 8, 12 and 16, because the kernels load 16 bytes
+  per thread at a time and batches that round up to the same number of loads are the same
+  kernel), ``sweep_bits_sq()`` times `bits-sq` with every row cut into 2..16 parts for the query
+  counts that do not fill the GPU with one row per workgroup, ``sweep_partial_bitonic()`` times
+  `partial-bitonic-regs` over the grid of scripts/run-opt-bitonic-sort.sh:27-43 (q*n = 2^30, q in
+  64..4096, k in 32..2048, block size 64..512), ``sweep_fused()`` times `fused-cache` (whose
+  tuning parameters do not steer the matrix-core kernel: its rows carry the reference's fixed
+  choice 8,4,2 / 1 / 1), and ``write_optima()`` keeps the fastest configuration of every
+  (algorithm, q, k, dim) in a CSV with the columns of the reference's scripts/optima.csv
   (hostname, GPU, algorithm, point_count, query_count, k, dim, block_size, items_per_thread,
   items_per_thread2, items_per_thread3, deg, time), as scripts/plot-analyze-opt.py does.
 * ``config_algorithm()`` is the lookup the reference's run scripts perform on that file
@@ -15,7 +20,7 @@ Two halves, matching the reference's tuning workflow:
   of the algorithm (and host), prefer rows whose query_count / k / dim are not below the request,
   and among those the row with the smallest product of ratios to the request.
 
-    python -m bitsknn.tuning --out optima.csv        # on a GPU box; about two minutes
+    python -m bitsknn.tuning --out optima.csv        # on a GPU box; a few minutes
 
 The timed matrix is generated on the device (uniform [0,1), as `knn -g uniform`); one
 8192 x 524288 matrix (16 GiB) serves every query count as a row prefix.
@@ -33,8 +38,18 @@ DEFAULT_OPTIMA = os.path.join(os.path.dirname(os.path.abspath(__file__)), "optim
 QUERY_COUNTS = (64, 256, 512, 1024, 2048, 4096, 8192)
 K_VALUES = (2, 4, 8, 16, 32, 64, 128, 256, 512, 1024, 2048)
 BLOCK_SIZES = (128, 256, 512)
-BATCH_SIZES = tuple(range(1, 17))
+# values per thread and iteration: the kernels issue 16-byte loads, so 1..4, 5..8, 9..12 and 13..16
+# are one kernel each; the sweep times the distinct ones
+BATCH_SIZES = (4, 8, 12, 16)
 ALGORITHMS = (("bits", False), ("bits-prefetch", True))
+# bits-sq: parts a row is cut into, for query counts that leave compute units without a row
+SQ_QUERY_COUNTS = (64, 256)
+SQ_DEGREES = (2, 4, 8, 16)
+# fused-cache: (queries, points) shapes of the reference's fused runs (scripts/run-fused.sh) that
+# bound the lookup's range, dimensions and list lengths
+FUSED_SHAPES = ((1024, 1 << 20), (8192, 1 << 17))
+FUSED_DIMS = (8, 16, 32)
+FUSED_K_VALUES = (4, 8, 16, 32, 64, 128, 256)
 
 
 def config_algorithm(algorithm, query_count=None, k=None, dim=None, hostname=None,
@@ -128,6 +143,107 @@ def sweep(repeats=10, point_count=512 * 1024, query_counts=QUERY_COUNTS, k_value
                 progress(q, k)
 
 
+def bits_sq(rows, k, deg, block, batch, scratch=None):
+    """`bits-sq` through the C ABI (reference src/topk/singlepass/bits_knn.cu:132-186): every row
+    is cut into `deg` parts that are selected independently with their labels shifted by the part's
+    offset, then the deg*k partial results of a row are selected again with their labels."""
+    import torch
+    import bitsknn
+    q, n = rows.shape
+    assert n % deg == 0
+    if scratch is None:
+        scratch = {}
+    key = (q, k, deg)
+    if key not in scratch:
+        scratch[key] = (torch.empty((q * deg, k), dtype=torch.float32, device=rows.device),
+                        torch.empty((q * deg, k), dtype=torch.int32, device=rows.device),
+                        bitsknn.label_offsets(q, deg, n // deg, rows.device),
+                        torch.empty((q, k), dtype=torch.float32, device=rows.device),
+                        torch.empty((q, k), dtype=torch.int32, device=rows.device))
+    part_d, part_l, offsets, out_d, out_l = scratch[key]
+    bitsknn.topk_bits(rows.view(q * deg, n // deg), k, block, batch, True, label_offsets=offsets,
+                      out_dist=part_d, out_label=part_l)
+    bitsknn.topk_bits(part_d.view(q, deg * k), k, block, batch, True, in_label=part_l.view(q, deg * k),
+                      out_dist=out_d, out_label=out_l)
+    return out_d, out_l
+
+
+def sweep_bits_sq(repeats=10, point_count=512 * 1024, query_counts=SQ_QUERY_COUNTS, k_values=K_VALUES,
+                  block_sizes=BLOCK_SIZES, batch_sizes=BATCH_SIZES, degrees=SQ_DEGREES, seed=17,
+                  progress=None):
+    """Time bits-sq on cuda:0 over the parts per row; yields dict rows like sweep()."""
+    import torch
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    matrix = torch.rand((max(query_counts), point_count), device=dev, generator=gen)
+    for q in query_counts:
+        rows = matrix[:q]
+        for k in k_values:
+            scratch = {}
+            for deg in degrees:
+                if k * deg > point_count // deg:
+                    continue
+                for block in block_sizes:
+                    if k > block * 16:
+                        continue
+                    for batch in batch_sizes:
+                        bits_sq(rows, k, deg, block, batch, scratch)
+                        start = torch.cuda.Event(enable_timing=True)
+                        end = torch.cuda.Event(enable_timing=True)
+                        start.record()
+                        for _ in range(repeats):
+                            bits_sq(rows, k, deg, block, batch, scratch)
+                        end.record()
+                        end.synchronize()
+                        yield {"algorithm": "bits-sq", "point_count": point_count, "query_count": q,
+                               "k": k, "dim": 1, "block_size": block, "items_per_thread": batch,
+                               "items_per_thread2": 1, "items_per_thread3": 1, "deg": deg,
+                               "time": start.elapsed_time(end) / 1e3 / repeats}
+            if progress is not None:
+                progress(q, k)
+
+
+def sweep_fused(repeats=3, shapes=FUSED_SHAPES, dims=FUSED_DIMS, k_values=FUSED_K_VALUES, seed=17,
+                progress=None):
+    """Time fused-cache (with the workspace its entry point asks for) on cuda:0.  The reference's
+    parameters do not change the kernel, so there is one row per problem, with the reference's
+    fixed choice of them (scripts/optima-fixed-max_slowdown.csv: 8,4,2, block 1, deg 1)."""
+    import torch
+    import bitsknn
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    for q, n in shapes:
+        for dim in dims:
+            points = torch.rand((dim, n), device=dev, generator=gen)
+            queries = torch.rand((dim, q), device=dev, generator=gen)
+            for k in k_values:
+                out_d = torch.empty((q, k), dtype=torch.float32, device=dev)
+                out_l = torch.empty((q, k), dtype=torch.int32, device=dev)
+                workspace = torch.empty(max(1, bitsknn.fused_workspace_bytes(q, n, k)), dtype=torch.uint8,
+                                        device=dev)
+
+                def run():
+                    bitsknn.fused_l2_topk(queries, points, k, (8, 4, 2), 1, 1, out_dist=out_d, out_label=out_l,
+                                          workspace=workspace)
+                run()
+                start = torch.cuda.Event(enable_timing=True)
+                end = torch.cuda.Event(enable_timing=True)
+                start.record()
+                for _ in range(repeats):
+                    run()
+                end.record()
+                end.synchronize()
+                yield {"algorithm": "fused-cache", "point_count": n, "query_count": q, "k": k, "dim": dim,
+                       "block_size": 1, "items_per_thread": 8, "items_per_thread2": 4,
+                       "items_per_thread3": 2, "deg": 1, "time": start.elapsed_time(end) / 1e3 / repeats}
+            if progress is not None:
+                progress(q, dim)
+
+
 def sweep_partial_bitonic(repeats=5, problem_size=1 << 30, query_counts=(64, 256, 1024, 4096),
                           k_values=(32, 64, 128, 256, 512, 1024, 2048), block_sizes=(64, 128, 256, 512),
                           seed=17, progress=None):
@@ -187,7 +303,7 @@ def main(argv=None):
     ap.add_argument("--all", default=None, help="also write every measurement to this CSV")
     ap.add_argument("--repeats", type=int, default=10)
     ap.add_argument("--hostname", default="mi355x")
-    ap.add_argument("--only", choices=("bits", "partial-bitonic-regs"), default=None,
+    ap.add_argument("--only", choices=("bits", "bits-sq", "partial-bitonic-regs", "fused-cache"), default=None,
                     help="time one family only (bits covers bits and bits-prefetch)")
     args = ap.parse_args(argv)
 
@@ -197,6 +313,10 @@ def main(argv=None):
     rows = []
     if args.only in (None, "bits"):
         rows += list(sweep(repeats=args.repeats, progress=progress))
+    if args.only in (None, "bits-sq"):
+        rows += list(sweep_bits_sq(repeats=args.repeats, progress=progress))
+    if args.only in (None, "fused-cache"):
+        rows += list(sweep_fused(progress=progress))
     if args.only in (None, "partial-bitonic-regs"):
         rows += list(sweep_partial_bitonic(repeats=max(1, args.repeats // 2), progress=progress))
     if args.all:

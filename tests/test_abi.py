@@ -158,7 +158,8 @@ def test_config_lookup_matches_reference_script():
 
 def test_shipped_optima_file():
     """The MI355X optima file has the reference's columns (scripts/optima.csv, line 1) and a row
-    for every (algorithm, q, k) of the reference's search grid (scripts/run-opt-ipt.sh:38-47)."""
+    for every (algorithm, q, k) of the reference's search grid (scripts/run-opt-ipt.sh:38-47),
+    for bits-sq on the query counts that leave compute units idle, and for fused-cache."""
     import csv
     tuning = _load_tuning()
     with open(tuning.DEFAULT_OPTIMA, newline="") as handle:
@@ -171,7 +172,27 @@ def test_shipped_optima_file():
                 assert (name, q, k) in seen
     assert sum(r["algorithm"] == "partial-bitonic-regs" for r in rows) == 28
     for r in rows:
-        assert int(r["block_size"]) in (64, 128, 256, 512) and 1 <= int(r["items_per_thread"]) <= 16
         assert float(r["time"]) > 0
+        if r["algorithm"] in ("bits", "bits-prefetch", "bits-sq"):
+            # only values per thread that are kernels of their own (whole 16-byte loads)
+            assert int(r["block_size"]) in (128, 256, 512) and int(r["items_per_thread"]) in tuning.BATCH_SIZES
+        if r["algorithm"] == "partial-bitonic-regs":
+            assert int(r["block_size"]) in (64, 128, 256, 512)
     block, deg, batch, _, _ = tuning.config_algorithm("bits", 1024, 32)
-    assert block in (128, 256, 512) and deg == 1 and 1 <= batch <= 16
+    assert block in (128, 256, 512) and deg == 1 and batch in tuning.BATCH_SIZES
+    # bits-sq: every (q, k) of its grid, with the number of parts in the deg column; cutting the
+    # rows must pay where one row per workgroup leaves most of the GPU idle
+    plain = {(int(r["query_count"]), int(r["k"])): float(r["time"]) for r in rows if r["algorithm"] == "bits"}
+    for q in tuning.SQ_QUERY_COUNTS:
+        for k in tuning.K_VALUES:
+            mine = [r for r in rows if r["algorithm"] == "bits-sq" and int(r["query_count"]) == q and int(r["k"]) == k]
+            assert len(mine) == 1 and int(mine[0]["deg"]) in tuning.SQ_DEGREES
+            if q == 64:
+                assert float(mine[0]["time"]) < plain[(q, k)]
+    block, deg, batch, _, _ = tuning.config_algorithm("bits-sq", 64, 32)
+    assert deg in tuning.SQ_DEGREES
+    # fused-cache: the reference's fixed parameters (they do not steer the kernel) for every
+    # (shape, dim, k) of the grid; the lookup by (q, k, dim) returns them
+    fused = [r for r in rows if r["algorithm"] == "fused-cache"]
+    assert len(fused) == len(tuning.FUSED_SHAPES) * len(tuning.FUSED_DIMS) * len(tuning.FUSED_K_VALUES)
+    assert tuning.config_algorithm("fused-cache", 8192, 32, 16) == (1, 1, 8, 4, 2)
