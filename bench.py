@@ -25,7 +25,8 @@ which did not do its work cannot produce a figure.
   sweep        the 4 GiB matrix at k in {16,32,128,512,2048} x block size {128,256,512} with 2048
                values of a row in flight per iteration (16 / 8 / 4 values per thread), plus the
                configuration the shipped optima file names for each k
-  hard         16,384 x 65,536 rows sorted ascending / descending / drawn from 256 values, k = 32, 256
+  hard         16,384 x 65,536 rows sorted ascending / descending / drawn from 256 values, k = 32, 256,
+               with one fixed configuration and with the one the optima file names
   gemm         ||p||^2 - 2 q.p on fp32 MFMA for 1,048,576 points x 4,096 queries, d = 64 (a 16 GiB
                matrix), then bits top-k (k = 64) on it
   fused        bits-fused, 1,048,576 points x 65,536 queries, d in {8,16,32} x k in {4,16,32}, priced
@@ -214,6 +215,7 @@ def leg_hard(bitsknn, torch, timer, oracle, dev, steps, check, rows=16384, cols=
     inputs = {"ascending": asc, "descending": torch.flip(asc, dims=[1]).contiguous(),
               "256-values": torch.floor(base * 256) / 256}
     del base
+    from bitsknn import tuning
     sample = sample_indices(rows, 32)
     out = []
     for name, matrix in inputs.items():
@@ -221,15 +223,19 @@ def leg_hard(bitsknn, torch, timer, oracle, dev, steps, check, rows=16384, cols=
         for k in (32, 256):
             out_d = torch.full((rows, k), -1.0, dtype=torch.float32, device=dev)
             out_l = torch.empty((rows, k), dtype=torch.int32, device=dev)
-            block, items = HARD_CONFIG
-            _, ks = timer.run(lambda: bitsknn.topk_bits(matrix, k, block, items, out_dist=out_d, out_label=out_l),
-                              steps, 2)
-            entry = {"rows": name, "k": k, "block": block, "items_per_thread": items,
-                     "elements_per_s": rows * cols / ks, "kernel_ms": ks * 1e3,
-                     "frac": (4.0 * rows * cols + 8.0 * rows * k) / ks / 1e9 / HBM_PEAK_GBS}
-            if check:
-                entry["verified"] = verify_topk(oracle, cache, matrix, sample, k, out_d, out_l)
-            out.append(entry)
+            tuned_block, _, tuned_items, _, _ = tuning.config_algorithm("bits", rows, k)
+            for block, items, tuned in (HARD_CONFIG + (False,), (tuned_block, tuned_items, True)):
+                out_d.fill_(-1.0)
+                _, ks = timer.run(lambda: bitsknn.topk_bits(matrix, k, block, items, out_dist=out_d, out_label=out_l),
+                                  steps, 2)
+                entry = {"rows": name, "k": k, "block": block, "items_per_thread": items,
+                         "elements_per_s": rows * cols / ks, "kernel_ms": ks * 1e3,
+                         "frac": (4.0 * rows * cols + 8.0 * rows * k) / ks / 1e9 / HBM_PEAK_GBS}
+                if tuned:
+                    entry["tuned"] = True
+                if check:
+                    entry["verified"] = verify_topk(oracle, cache, matrix, sample, k, out_d, out_l)
+                out.append(entry)
     return out
 
 

@@ -12,7 +12,8 @@ constexpr int FQ_WAVES = 4;                   // waves per workgroup
 constexpr int FQ_THREADS = FQ_WAVES * WAVE;   // 256
 constexpr int FQ_QW = 32;                     // queries per wave (one MFMA column tile)
 constexpr int FQ_QB = FQ_QW * FQ_WAVES;       // queries per workgroup
-constexpr int FQ_CAP = 32;                    // buffer slots per query (= points per MFMA tile)
+constexpr int FQ_CAP = 32;                    // buffer slots per query (= points per MFMA tile); twice
+                                              // that for long lists in few dimensions (fused_geometry)
 
 struct fused_args
 {

@@ -16,7 +16,8 @@
 //  * The query fragment stays in registers for the whole kernel.  In the 32 x 32 result tile a
 //    lane holds 16 distances of ONE query (column), so the filter is a min-tree over 16
 //    registers and one compare against that query's radius.
-//  * Every query has a 32-slot buffer in LDS.  Slots are handed out without atomics: the two
+//  * Every query has a 32-slot buffer in LDS (64 slots for lists of 128 and more in up to 16
+//    dimensions).  Slots are handed out without atomics: the two
 //    lanes that share a query exchange their pass counts, and the fill is kept in a register.
 //    Before a tile would overflow any buffer of the wave, the wave merges all its buffers; the
 //    other waves of the workgroup, which would wait for it at the stage barrier, then merge
@@ -68,14 +69,22 @@ __device__ __forceinline__ float min3(float a, float b, float c)
 // the fp32 one and does not share the vector unit with it.  A stage holds, per piece and per 8
 // dimensions, one 16-byte cell per point (the A operand of v_mfma_f32_32x32x16_bf16), then the
 // norms of the points.
-template <int DP, bool SPLIT>
+// Per-query buffers: 32 slots, the points of one matrix tile.  Every merge pays for the whole list,
+// so for lists of 128 entries and more the buffers have 64 slots where the stages leave room for
+// them (up to 16 dimensions, with smaller stages): half as many merges (q = 8192, n = 2^17,
+// d = 8: 4.4 -> 2.7 ms at k = 256, 1.7 -> 1.3 ms at k = 128; at k = 64 the smaller stages cost more
+// than the merges save).
+template <int DP, bool SPLIT, int K>
 struct fused_geometry
 {
+    static constexpr bool WIDE = K >= 128 && DP <= 16 && !SPLIT;
+    static constexpr int CAP = WIDE ? 2 * FQ_CAP : FQ_CAP; // buffer slots per query
     static constexpr int DK = DP < 16 ? 16 : DP;       // SPLIT: dimensions padded to whole matrix steps
     static constexpr int KB = DK / 16;                 // SPLIT: matrix steps of 16 dimensions
     static constexpr int KS = DK / 8;                  // SPLIT: cells of 8 dimensions per point and piece
-    static constexpr int PT = SPLIT ? (DK <= 16 ? 128 : (DK <= 32 ? 64 : 32))
-                                    : (DP <= 16 ? 256 : (DP <= 32 ? 128 : (DP <= 64 ? 64 : 32)));
+    static constexpr int PT = SPLIT  ? (DK <= 16 ? 128 : (DK <= 32 ? 64 : 32))
+                              : WIDE ? (DP <= 8 ? 128 : 64)
+                                     : (DP <= 16 ? 256 : (DP <= 32 ? 128 : (DP <= 64 ? 64 : 32)));
     static constexpr int TPP = FQ_THREADS / PT; // threads per point when staging
     // point rows (zero beyond dim), then one row per staging thread of a point with its share of
     // ||p||^2 (at least two rows, so that the row count is even)
@@ -90,7 +99,7 @@ struct fused_geometry
     {
         // two stages (one being multiplied, one being filled), the query buffers, exchange slots
         return 2 * static_cast<size_t>(STAGE_FLOATS) * sizeof(float) +
-               static_cast<size_t>(FQ_WAVES) * FQ_QW * FQ_CAP * sizeof(u64) +
+               static_cast<size_t>(FQ_WAVES) * FQ_QW * CAP * sizeof(u64) +
                static_cast<size_t>(FQ_WAVES) * WAVE * sizeof(float) + 4 * sizeof(int);
     }
 };
@@ -100,8 +109,9 @@ struct fused_geometry
 template <int K, int DP, bool SPLIT>
 __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 {
-    using G = fused_geometry<DP, SPLIT>;
+    using G = fused_geometry<DP, SPLIT, K>;
     constexpr int PT = G::PT;
+    constexpr int CAP = G::CAP;
     // Norms in the accumulator: where one staging thread carries a whole point (DP <= 16) its
     // ||p||^2 is one row after the point rows and is read as the initial value of the
     // accumulators, which saves the matrix step that would add it (one of 5 at DP = 8, one of 9 at
@@ -115,7 +125,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     constexpr int VPT = G::VPT;
     constexpr int MT = G::MT;
     // merge layout: S keys per query spread over LPQ lanes, R keys per lane
-    constexpr int S = K > FQ_CAP ? K : FQ_CAP;
+    constexpr int S = K > CAP ? K : CAP;
     constexpr int R = 4;
     constexpr int LPQ = S / R;
     constexpr int QPP = WAVE / LPQ;           // queries per merge pass
@@ -123,13 +133,13 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     // Whether the waves of a workgroup merge together (below): pays for the long merges of long
     // lists (k = 256: 65 -> 52 ms); for k <= 32 the two looks at the flag per stage cost more (1 %
     // each) than the short merges they overlap.
-    constexpr bool JOIN_MERGES = K > FQ_CAP;
+    constexpr bool JOIN_MERGES = K > CAP;
 
     extern __shared__ float lds[];
     constexpr int STAGE_FLOATS = G::STAGE_FLOATS;
     float* const stages = lds;                                                    // [2][STAGE_FLOATS]
     u64* const buffers = reinterpret_cast<u64*>(lds + 2 * STAGE_FLOATS);          // [waves][32][CAP]
-    float* const xchg = reinterpret_cast<float*>(buffers + FQ_WAVES * FQ_QW * FQ_CAP);  // [waves][64]
+    float* const xchg = reinterpret_cast<float*>(buffers + FQ_WAVES * FQ_QW * CAP);  // [waves][64]
     int* const merge_wanted = reinterpret_cast<int*>(xchg + FQ_WAVES * WAVE);           // [3]
 
     const int dim = a.dim;
@@ -144,7 +154,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     const int ql = lane & 31;                 // query of this lane inside the wave
     const int wave_q0 = static_cast<int>(blockIdx.x) * FQ_QB + wave * FQ_QW;
     const int my_q = wave_q0 + ql;
-    u64* const wbuf = buffers + static_cast<size_t>(wave) * FQ_QW * FQ_CAP;
+    u64* const wbuf = buffers + static_cast<size_t>(wave) * FQ_QW * CAP;
     float* const wx = xchg + wave * WAVE;     // 32 radii, then 32 fills (as int bits)
 
     // query fragment: step s of this lane is row 2s + half, times -2 (the stages hold the plain
@@ -211,12 +221,12 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        if constexpr (K > FQ_CAP)
+        if constexpr (K > CAP)
         {
             // Lists longer than a buffer: the buffers are sorted in place first, 8 queries at a
             // time, so that the passes below only pay for the merge network of the list.
             constexpr int BR = 4;           // keys per lane
-            constexpr int BL = FQ_CAP / BR; // lanes per buffer
+            constexpr int BL = CAP / BR; // lanes per buffer
 #pragma unroll 1
             for (int pass = 0; pass < FQ_QW / (WAVE / BL); ++pass)
             {
@@ -228,13 +238,13 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 for (int r = 0; r < BR; ++r)
                 {
                     const int i = sub * BR + r;
-                    buf[r] = i < used ? wbuf[qm * FQ_CAP + i] : PAD_KEY;
+                    buf[r] = i < used ? wbuf[qm * CAP + i] : PAD_KEY;
                 }
                 net_sort<BL, BR, 2, true>(buf, nullptr, sub);
 #pragma unroll
                 for (int r = 0; r < BR; ++r)
                 {
-                    wbuf[qm * FQ_CAP + sub * BR + r] = buf[r];
+                    wbuf[qm * CAP + sub * BR + r] = buf[r];
                 }
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -275,15 +285,15 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             for (int r = 0; r < R; ++r)
             {
                 const int i = sub * R + r;
-                if constexpr (K > FQ_CAP)
+                if constexpr (K > CAP)
                 {
                     // the sorted buffer (descending, padding first) is the tail of a descending
                     // sequence of K keys
-                    buf[r] = i >= K - FQ_CAP ? wbuf[qm * FQ_CAP + i - (K - FQ_CAP)] : PAD_KEY;
+                    buf[r] = i >= K - CAP ? wbuf[qm * CAP + i - (K - CAP)] : PAD_KEY;
                 }
                 else
                 {
-                    buf[r] = i < used ? wbuf[qm * FQ_CAP + (i < FQ_CAP ? i : 0)] : PAD_KEY;
+                    buf[r] = i < used ? wbuf[qm * CAP + (i < CAP ? i : 0)] : PAD_KEY;
                 }
                 list[r] = make_key(next_dist[r], next_label[r]);
             }
@@ -292,7 +302,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 request_list(pass + 1);
             }
             // buffer descending, element-wise minimum with the ascending list, re-sort
-            if constexpr (K <= FQ_CAP)
+            if constexpr (K <= CAP)
             {
                 net_sort<LPQ, R, 2, true>(buf, nullptr, sub);
             }
@@ -352,7 +362,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         };
         int mine = compare();
         int other = static_cast<int>(lane_xor32<32>(static_cast<u32>(mine)));
-        if (__builtin_amdgcn_ballot_w64(fill + mine + other > FQ_CAP) != 0)
+        if (__builtin_amdgcn_ballot_w64(fill + mine + other > CAP) != 0)
         {
             // the other waves of the workgroup would wait for this wave at the stage barrier:
             // they are asked to merge their buffers in the meantime
@@ -373,7 +383,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             {
                 if (__builtin_amdgcn_inverse_ballot_w64(pass[r]))
                 {
-                    wbuf[ql * FQ_CAP + slot] = make_key(acc[r], first_point + 8 * (r / 4) + (r % 4));
+                    wbuf[ql * CAP + slot] = make_key(acc[r], first_point + 8 * (r / 4) + (r % 4));
                     ++slot;
                 }
             }
@@ -787,7 +797,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 template <int K, int DP, bool SPLIT>
 hipError_t launch_fused(const fused_args& a, hipStream_t stream)
 {
-    constexpr size_t lds_bytes = fused_geometry<DP, SPLIT>::lds_bytes();
+    constexpr size_t lds_bytes = fused_geometry<DP, SPLIT, K>::lds_bytes();
     if (lds_bytes > 48 * 1024)
     {
         const hipError_t status =
