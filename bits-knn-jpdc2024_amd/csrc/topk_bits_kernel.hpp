@@ -21,7 +21,11 @@
 //    direction tighten the radius at once, and for small batches the next chunk is requested
 //    before the current one is filtered;
 //  * long rows start from a radius taken from a sample of both row ends instead of from +inf,
-//    which saves the first merges (they only halve the radius each).
+//    which saves the first merges (they only halve the radius each);
+//  * lists of 1024 entries and more start from an estimate of the k-th smallest value of the
+//    row, taken from a sample spread over the row, and repeat the row from +inf in the rare case
+//    that fewer than k values lie below the estimate (a third of the values pass the filter then,
+//    and less than half the merges are needed: 0.70 -> 0.79 of the HBM peak at k = 2048).
 // Because waves drift apart, the filter compares full keys when a value equals the radius, so
 // that "equal values by lower label" holds no matter which wave saw which value first.
 
@@ -96,6 +100,20 @@ __device__ __forceinline__ u64 broadcast_radius(const u64 (&topk)[IPT], u32 k, u
     return *slot;
 }
 
+// Inserts `value` into the ascending array `lo` of the KEEP smallest values seen, dropping the
+// largest (a NaN is taken for +inf).
+template <int KEEP>
+__device__ __forceinline__ void keep_smallest(float (&lo)[KEEP], float value)
+{
+    value = fminf(value, __builtin_inff());
+#pragma unroll
+    for (int j = KEEP - 1; j > 0; --j)
+    {
+        lo[j] = __builtin_amdgcn_fmed3f(value, lo[j - 1], lo[j]);
+    }
+    lo[0] = fminf(value, lo[0]);
+}
+
 // BS threads, IPT list entries per thread, L 16-byte (or 4 x 4-byte when !VEC) loads in flight
 // per thread and iteration.
 template <int BS, int IPT, int L, bool VEC>
@@ -112,6 +130,12 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     // and 16-byte pieces per thread and end of the row (4 values looked at per value kept).
     constexpr int SAMPLE_KEEP = IPT <= 1 ? 2 : (IPT == 2 ? 4 : 8);
     constexpr u32 SAMPLE_PAIRS = SAMPLE_KEEP;
+    // Lists of 1024 entries and more start from an estimate of the k-th smallest value instead
+    // (see below): a sample of up to EST_PIECES 16-byte pieces per thread, 2^14 values, spread
+    // over the row, of which every thread keeps its EST_KEEP smallest.
+    constexpr bool ESTIMATE = NL >= 1024;
+    constexpr u32 EST_PIECES = 4096 / BS;
+    constexpr int EST_KEEP = 8;
 
     __shared__ u64 buffer[2 * NL];   // candidates; the second half is exchange space of the merges
     __shared__ u64 s_radius;
@@ -120,7 +144,7 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     __shared__ int s_more;  // some wave still has values to process after this merge
     __shared__ u32 s_sample[W];
 
-    const int t = static_cast<int>(threadIdx.x);
+    int t = static_cast<int>(threadIdx.x);
     const int lane = t & (WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(t / WAVE);
     const size_t row_idx = blockIdx.x;
@@ -150,11 +174,6 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     };
 
     u64 topk[IPT];
-#pragma unroll
-    for (int r = 0; r < IPT; ++r)
-    {
-        topk[r] = PAD_KEY;
-    }
 
     // ---- radius from a sample.  Every thread looks at up to SAMPLE_PAIRS pairs of 16-byte pieces
     // of the row, one at its front and one at its back (at most a sixteenth of the row in all), and
@@ -163,12 +182,102 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     // largest of these W values, so nothing above it can belong to the result: it serves as
     // radius until the list itself has a smaller one.  This replaces the first merges of a row,
     // which each only halve the radius and which all rows of a launch do at the same time.
+    //
+    // Long lists (ESTIMATE) on rows of at least 256 * BS values start lower, from an estimate.
+    // The sample is spread evenly over the row (at most a 64th of it) and the radius is its
+    // value of rank e + 5 sqrt(e) + 2, where e = k * sample size / n values of the sample are
+    // expected among the k smallest of the row: fewer than k values of the row lie below it with
+    // a probability under 10^-5 per row when the sample is representative, whatever the order of
+    // the row (sorted rows included).  At k = 2048 on rows of 2^20 uniform values 4 thousand values
+    // pass the filter then instead of 12 thousand, and 3 merges are needed instead of 7.  The
+    // estimate is not trusted: if the k-th key of the list has not got below it by the end of the
+    // row, the pass is repeated without it.
+    bool estimated = false;
     {
+        u32 wave_bound = 0xFFFFFFFFU;
+        bool have = false;
+        if constexpr (ESTIMATE)
+        {
+            const u32 fit = n / (256U * BS);
+            const u32 pieces = fit < EST_PIECES ? fit : EST_PIECES;
+            const float expect =
+                static_cast<float>(a.k) * static_cast<float>(pieces * 4 * BS) / static_cast<float>(n);
+            const u32 rank = static_cast<u32>(ceilf(expect + 5.0F * sqrtf(expect))) + 2;
+            if (pieces > 0 && a.k > 0 && rank <= WAVE)
+            {
+                const u32 segment = (n / pieces) & ~3U;
+                const u32 offset = (segment / 2 - 2 * BS) & ~3U; // the piece sits in the middle
+                float lo[EST_KEEP]; // ascending
+#pragma unroll
+                for (int j = 0; j < EST_KEEP; ++j)
+                {
+                    lo[j] = __builtin_inff();
+                }
+#pragma unroll 2
+                for (u32 p = 0; p < pieces; ++p)
+                {
+                    const u32 col = p * segment + offset + static_cast<u32>(t) * 4;
+                    vfloat4 x;
+                    if constexpr (VEC)
+                    {
+                        x = *reinterpret_cast<const vfloat4*>(row + col);
+                    }
+                    else
+                    {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                        {
+                            x[i] = row[col + i];
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                    {
+                        keep_smallest(lo, x[i]);
+                    }
+                }
+                u64 keys[EST_KEEP];
+#pragma unroll
+                for (int j = 0; j < EST_KEEP; ++j)
+                {
+                    keys[j] = static_cast<u64>(float_key(lo[j])) << 32U;
+                }
+                net_sort<WAVE, EST_KEEP, 2, false>(keys, nullptr, lane);
+                // the 64 smallest of every wave (sorted position p is entry p % EST_KEEP of lane
+                // p / EST_KEEP) meet in LDS; every wave sorts all of them and takes the same pick
+                u32* const meet = reinterpret_cast<u32*>(buffer);
+                if (lane < WAVE / EST_KEEP)
+                {
+#pragma unroll
+                    for (int j = 0; j < EST_KEEP; ++j)
+                    {
+                        meet[wave * WAVE + lane * EST_KEEP + j] = static_cast<u32>(keys[j] >> 32U);
+                    }
+                }
+                __syncthreads();
+                u64 all[W];
+#pragma unroll
+                for (int i = 0; i < W; ++i)
+                {
+                    all[i] = static_cast<u64>(meet[i * WAVE + lane]) << 32U;
+                }
+                net_sort<WAVE, W, 2, false>(all, nullptr, lane);
+                u32 pick = 0;
+#pragma unroll
+                for (int i = 0; i < W; ++i)
+                {
+                    pick = (rank - 1) % W == static_cast<u32>(i) ? static_cast<u32>(all[i] >> 32U) : pick;
+                }
+                wave_bound = static_cast<u32>(__builtin_amdgcn_readlane(
+                    static_cast<int>(pick), static_cast<int>((rank - 1) / W)));
+                estimated = wave_bound < float_key(__builtin_inff());
+                have = true;
+            }
+        }
         const u32 c = (a.k + W - 1) / W;
         const u32 fit = n / (128U * BS);
         const u32 pairs = fit < SAMPLE_PAIRS ? fit : SAMPLE_PAIRS;
-        u32 wave_bound = 0xFFFFFFFFU;
-        if (c <= WAVE * SAMPLE_KEEP && pairs > 0)
+        if (!have && c <= WAVE * SAMPLE_KEEP && pairs > 0)
         {
             const u32 back = VEC ? (n - pairs * 4 * BS) & ~3U : n - pairs * 4 * BS;
             float lo[SAMPLE_KEEP]; // ascending
@@ -198,13 +307,7 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
 #pragma unroll
                 for (int i = 0; i < 8; ++i)
                 {
-                    const float value = fminf(x[i / 4][i % 4], __builtin_inff()); // NaN -> +inf
-#pragma unroll
-                    for (int j = SAMPLE_KEEP - 1; j > 0; --j)
-                    {
-                        lo[j] = __builtin_amdgcn_fmed3f(value, lo[j - 1], lo[j]);
-                    }
-                    lo[0] = fminf(value, lo[0]);
+                    keep_smallest(lo, x[i / 4][i % 4]);
                 }
             }
             u64 keys[SAMPLE_KEEP];
@@ -227,346 +330,380 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
         s_sample[wave] = wave_bound;
     }
 
-    if (t == 0)
+    // (a second turn of this loop only after an estimate that proved too low)
+    for (bool again = false;; again = true)
     {
-        s_flag = 0;
-        s_more = 0;
-    }
-    __syncthreads();
-
-    float radius = __builtin_inff();
-    u64 radius_key = PAD_KEY;
-    bool sampled = false;
-    {
-        u32 bound = 0;
-#pragma unroll
-        for (int w = 0; w < W; ++w)
+        if constexpr (ESTIMATE)
         {
-            bound = s_sample[w] > bound ? s_sample[w] : bound;
+            // (the thread index made opaque per turn: what is derived from it is then computed in
+            // the turn rather than kept in registers around the whole loop, which costs 16 of them)
+            asm volatile("" : "+v"(t));
         }
-        // values up to the bound pass: the radius is the next key after it with the lowest label
-        bound = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(bound)));
-        if (bound < float_key(__builtin_inff()))
-        {
-            radius_key = static_cast<u64>(bound + 1) << 32U;
-            radius = key_float(bound + 1);
-            sampled = true;
-        }
-    }
-
-    // Without a radius from the sample the first NL values go straight to the buffer and the
-    // first merge sorts them; with one, they are filtered like the rest of the row (`head` = 0),
-    // which saves that merge.
-    const u32 head = sampled ? 0U : static_cast<u32>(NL);
-    const u32 first = n < head ? n : head;
-    const u32 full_end = n > head ? head + ((n - head) / CHUNK) * CHUNK : head;
-    // The chunks after the head are visited from both ends of the row inwards, the
-    // back first (last, first, last but one, second, ...): whichever end of a sorted row holds the
-    // small values, the radius is tight after the first NL values (ascending rows) or after the
-    // last chunk (descending rows), where a front-to-back pass over a descending row would let
-    // every value through the filter.  The result does not depend on the order.
-    const u32 chunk_count = n > head ? (n - head + CHUNK - 1) / CHUNK : 0;
-    u32 left = chunk_count;            // chunks not yet visited
-    // distance from the chunk being visited to the next one: alternating in sign and shrinking by
-    // one chunk per visit
-    // (Lists of 512 entries and more start at the front instead -- first, last, second, ... --:
-    // measured on uniform rows of 2^20 values they lose 0.4 % at k = 512 and 1.5 % at k = 2048 of
-    // the HBM roofline with the back first, more than a merge per sorted row is worth there.)
-    constexpr bool BACK_FIRST = NL < 512;
-    const std::int32_t span = chunk_count > 0 ? static_cast<std::int32_t>((chunk_count - 1) * CHUNK) : 0;
-    std::int32_t jump = BACK_FIRST ? -span : span;
-    u32 chunk = head + (BACK_FIRST ? static_cast<u32>(span) : 0U); // the next chunk to visit
-
-    // the head goes straight to the buffer: column c into slot c (the barrier at the top of the
-    // main loop orders these writes before the merge that reads them)
 #pragma unroll
-    for (int r = 0; r < IPT; ++r)
-    {
-        const u32 col = static_cast<u32>(r * BS + t);
-        if (col < first)
+        for (int r = 0; r < IPT; ++r)
         {
-            buffer[col] = make_key(row[col], label_of(col));
+            topk[r] = PAD_KEY;
         }
-    }
-    u32 cur_chunk = 0; // first column of the chunk held in v[]
-
-    float v[E];
-#pragma unroll
-    for (int j = 0; j < E; ++j)
-    {
-        v[j] = 0.0F;
-    }
-    // the values of the chunk that starts at column `first`, value j of thread t as column_of says
-    auto load_chunk = [&](float (&dst)[E], u32 first) {
-        if (first < full_end)
+        if (t == 0)
         {
-            if constexpr (VEC)
+            s_flag = 0;
+            s_more = 0;
+        }
+        __syncthreads();
+
+        float radius = __builtin_inff();
+        u64 radius_key = PAD_KEY;
+        u64 first_key = PAD_KEY; // the radius the pass starts from
+        bool sampled = false;
+        if (!again)
+        {
+            u32 bound = 0;
+#pragma unroll
+            for (int w = 0; w < W; ++w)
             {
-                const vfloat4* __restrict__ p = reinterpret_cast<const vfloat4*>(row + first) + t;
-#pragma unroll
-                for (int l = 0; l < L; ++l)
-                {
-                    const vfloat4 x = __builtin_nontemporal_load(p + l * BS);
-                    dst[4 * l + 0] = x.x;
-                    dst[4 * l + 1] = x.y;
-                    dst[4 * l + 2] = x.z;
-                    dst[4 * l + 3] = x.w;
-                }
+                bound = s_sample[w] > bound ? s_sample[w] : bound;
             }
-            else
+            // values up to the bound pass: the radius is the next key after it with the lowest label
+            bound = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(bound)));
+            if (bound < float_key(__builtin_inff()))
             {
-                const float* __restrict__ p = row + first + t;
-#pragma unroll
-                for (int j = 0; j < E; ++j)
-                {
-                    dst[j] = __builtin_nontemporal_load(p + j * BS);
-                }
+                radius_key = static_cast<u64>(bound + 1) << 32U;
+                first_key = radius_key;
+                radius = key_float(bound + 1);
+                sampled = true;
             }
         }
-        else
-        {
-            // ragged tail: bounds-checked 4-byte loads in the same value-to-thread mapping
+
+        // Without a radius from the sample the first NL values go straight to the buffer and the
+        // first merge sorts them; with one, they are filtered like the rest of the row (`head` = 0),
+        // which saves that merge.
+        const u32 head = sampled ? 0U : static_cast<u32>(NL);
+        const u32 first = n < head ? n : head;
+        const u32 full_end = n > head ? head + ((n - head) / CHUNK) * CHUNK : head;
+        // The chunks after the head are visited from both ends of the row inwards, the
+        // back first (last, first, last but one, second, ...): whichever end of a sorted row holds the
+        // small values, the radius is tight after the first NL values (ascending rows) or after the
+        // last chunk (descending rows), where a front-to-back pass over a descending row would let
+        // every value through the filter.  The result does not depend on the order.
+        const u32 chunk_count = n > head ? (n - head + CHUNK - 1) / CHUNK : 0;
+        u32 left = chunk_count;            // chunks not yet visited
+        // distance from the chunk being visited to the next one: alternating in sign and shrinking by
+        // one chunk per visit
+        // (Lists of 512 entries and more start at the front instead -- first, last, second, ... --:
+        // measured on uniform rows of 2^20 values they lose 0.4 % at k = 512 and 1.5 % at k = 2048 of
+        // the HBM roofline with the back first, more than a merge per sorted row is worth there.)
+        constexpr bool BACK_FIRST = NL < 512;
+        const std::int32_t span = chunk_count > 0 ? static_cast<std::int32_t>((chunk_count - 1) * CHUNK) : 0;
+        std::int32_t jump = BACK_FIRST ? -span : span;
+        u32 chunk = head + (BACK_FIRST ? static_cast<u32>(span) : 0U); // the next chunk to visit
+
+        // the head goes straight to the buffer: column c into slot c (the barrier at the top of the
+        // main loop orders these writes before the merge that reads them)
 #pragma unroll
-            for (int j = 0; j < E; ++j)
+        for (int r = 0; r < IPT; ++r)
+        {
+            const u32 col = static_cast<u32>(r * BS + t);
+            if (col < first)
             {
-                const u32 col = column_of(first, j);
-                dst[j] = col < n ? row[col] : __builtin_inff();
+                buffer[col] = make_key(row[col], label_of(col));
             }
         }
-    };
-    // Software pipelining for small batches: the next chunk is requested before the current one
-    // is filtered, at the price of E more registers and E moves per chunk.  Rows of two waves
-    // (128 threads) leave 8 waves per compute unit, which need the depth also with 4 loads each.
-    constexpr bool PIPE = L <= 2 || (BS == 128 && L <= 4);
-    float ahead[E];
-#pragma unroll
-    for (int j = 0; j < E; ++j)
-    {
-        ahead[j] = 0.0F;
-    }
-    if constexpr (PIPE)
-    {
-        if (left > 0)
-        {
-            load_chunk(ahead, chunk);
-        }
-    }
+        u32 cur_chunk = 0; // first column of the chunk held in v[]
 
-    // Fill of this wave's slice (wave-uniform).  Passing values take slots in the order
-    // (value index j, lane): value j of the lanes in its pass mask gets consecutive slots after
-    // those of the values before it.
-    //
-    // Only when a chunk does not fit into the slice is per-lane state kept for it: bit j of
-    // my_pass says value j of this lane passed the filter (decided with the radius of that
-    // moment), slot_base is the slot of the chunk's first passing value.  A merge empties every
-    // slice, so slot_base drops by CAP; a value is written in the round where its slot falls
-    // into [0, CAP).
-    int fill = static_cast<int>(first) - wave * CAP;
-    fill = fill < 0 ? 0 : (fill > CAP ? CAP : fill);
-    u32 my_pass = 0;
-    int slot_base = 0;
-    bool pending = false; // values of the chunk in v[] still wait for a slot
-
-    auto lane_rank = [&](u64 mask) -> int {
-        return static_cast<int>(__builtin_amdgcn_mbcnt_hi(
-            static_cast<u32>(mask >> 32U), __builtin_amdgcn_mbcnt_lo(static_cast<u32>(mask), 0U)));
-    };
-
-    // exact filter: below the radius key (an equal value is decided by its label; the +inf
-    // padding of a ragged tail never passes).  A NaN counts as +inf: it is neither below nor above
-    // the radius and its key decides, which can only succeed while the radius is +inf.
-    auto passes = [&](float value, int j) -> bool {
-        bool pass = value < radius;
-        if (!(value < radius) && !(value > radius))
-        {
-            const u32 col = column_of(cur_chunk, j);
-            pass = col < n && make_key(value, label_of(col)) < radius_key;
-        }
-        return pass;
-    };
-
-    // writes the pending values whose slot is inside the slice; returns the end of the
-    // chunk's reservation
-    auto write_pending = [&]() -> int {
-        int running = slot_base;
+        float v[E];
 #pragma unroll
         for (int j = 0; j < E; ++j)
         {
-            const bool mine = ((my_pass >> j) & 1U) != 0;
-            const u64 mask = __builtin_amdgcn_ballot_w64(mine);
-            if (mask != 0)
+            v[j] = 0.0F;
+        }
+        // the values of the chunk that starts at column `first`, value j of thread t as column_of says
+        auto load_chunk = [&](float (&dst)[E], u32 first) {
+            if (first < full_end)
             {
-                const int slot = running + lane_rank(mask);
-                if (mine && slot >= 0 && slot < CAP)
+                if constexpr (VEC)
                 {
-                    const u32 col = column_of(cur_chunk, j);
-                    slice[slot] = make_key(v[j], label_of(col));
+                    const vfloat4* __restrict__ p = reinterpret_cast<const vfloat4*>(row + first) + t;
+#pragma unroll
+                    for (int l = 0; l < L; ++l)
+                    {
+                        const vfloat4 x = __builtin_nontemporal_load(p + l * BS);
+                        dst[4 * l + 0] = x.x;
+                        dst[4 * l + 1] = x.y;
+                        dst[4 * l + 2] = x.z;
+                        dst[4 * l + 3] = x.w;
+                    }
                 }
-                running += __popcll(mask);
-            }
-        }
-        return running;
-    };
-
-    for (;;)
-    {
-        // ---- rendezvous: every wave arrives here when it needs a merge, saw the flag, or ran
-        // out of values
-        const bool more_work = pending || left > 0;
-        // (wave-uniform values, stored by every lane: a branch on the lane next to a loop exit
-        // makes the compiler treat the loop state as differing between lanes, which turns the
-        // streaming loop into an exec-masked one with its counters in vector registers)
-        s_fill[wave] = fill;
-        if (more_work)
-        {
-            s_more = 1;
-        }
-        __syncthreads();
-        // (the same in every lane; said explicitly so that the loops stay wave-uniform)
-        int total = 0;
-#pragma unroll
-        for (int w = 0; w < W; ++w)
-        {
-            total += s_fill[w];
-        }
-        total = __builtin_amdgcn_readfirstlane(total);
-        const bool more = __builtin_amdgcn_readfirstlane(s_more) != 0;
-        if (total > 0)
-        {
-            merge_buffer<BS, IPT>(topk, buffer, s_fill, t);
-            // the barriers of the merge lie between the reads above and this reset; the barrier
-            // of the broadcast publishes it together with the radius
-            if (t == 0)
-            {
-                s_flag = 0;
-                s_more = 0;
-            }
-            // (the radius from the sample stays until the list has a smaller one)
-            const u64 list_radius = broadcast_radius<IPT>(topk, a.k, &s_radius, t);
-            radius_key = list_radius < radius_key ? list_radius : radius_key;
-            radius = key_value(radius_key);
-        }
-        else
-        {
-            __syncthreads(); // orders the reads above before the reset below
-            if (t == 0)
-            {
-                s_flag = 0;
-                s_more = 0;
-            }
-            __syncthreads();
-        }
-        if (!more)
-        {
-            break;
-        }
-        fill = 0;
-        if (pending)
-        {
-            slot_base -= CAP;
-            const int end = write_pending();
-            if (end > CAP)
-            {
-                fill = CAP;
-                s_flag = 1;
-                continue;
-            }
-            fill = end;
-            pending = false;
-        }
-
-        // ---- streaming: no synchronisation with the other waves except polling the flag
-        while (left > 0)
-        {
-            if constexpr (PIPE)
-            {
-                // the values of this chunk were requested an iteration (or a merge) ago
-#pragma unroll
-                for (int j = 0; j < E; ++j)
+                else
                 {
-                    v[j] = ahead[j];
+                    const float* __restrict__ p = row + first + t;
+#pragma unroll
+                    for (int j = 0; j < E; ++j)
+                    {
+                        dst[j] = __builtin_nontemporal_load(p + j * BS);
+                    }
                 }
             }
             else
             {
-                load_chunk(v, chunk);
-            }
-            const int flag = __hip_atomic_load(&s_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            cur_chunk = chunk;
-            left -= 1;
-            chunk += static_cast<u32>(jump);
-            jump = (jump > 0 ? static_cast<std::int32_t>(CHUNK) : -static_cast<std::int32_t>(CHUNK)) - jump;
-            if constexpr (PIPE)
-            {
-                // request the next chunk before this one is filtered: the loads stay in flight
-                // through the filter and through a merge, if one comes
-                if (left > 0)
-                {
-                    load_chunk(ahead, chunk);
-                }
-            }
-
-            // NaN-propagating minimum (v_minimum3_f32): a lane that holds a NaN of any kind gets a NaN
-            // here and takes the look at every value below (the NaN-ignoring minimum would need
-            // every operand quietened first, and loses values after a signalling NaN otherwise)
-            float smallest = v[0];
-#pragma unroll
-            for (int j = 1; j < E; ++j)
-            {
-                smallest = __builtin_elementwise_minimum(smallest, v[j]);
-            }
-            // A value equal to the radius passes only with a label below the radius key's.  With
-            // implicit labels every label of this chunk is at least that of its first column, so
-            // when that one is not below, equal values need no look (rows with few distinct
-            // values have one in every chunk).
-            const bool no_ties =
-                lrow == nullptr && static_cast<std::int32_t>(cur_chunk + label_offset) >= key_label(radius_key);
-            // (negated compares: true for a NaN)
-            if (__builtin_amdgcn_ballot_w64(no_ties ? !(smallest >= radius) : !(smallest > radius)) != 0)
-            {
-                int running = fill;
+                // ragged tail: bounds-checked 4-byte loads in the same value-to-thread mapping
 #pragma unroll
                 for (int j = 0; j < E; ++j)
                 {
-                    if (__builtin_amdgcn_ballot_w64(!(v[j] > radius)) != 0)
-                    {
-                        const bool pass = passes(v[j], j);
-                        const u64 mask = __builtin_amdgcn_ballot_w64(pass);
-                        if (mask != 0)
-                        {
-                            const int slot = running + lane_rank(mask);
-                            if (pass && slot < CAP)
-                            {
-                                const u32 col = column_of(cur_chunk, j);
-                                slice[slot] = make_key(v[j], label_of(col));
-                            }
-                            running += __popcll(mask);
-                        }
-                    }
+                    const u32 col = column_of(first, j);
+                    dst[j] = col < n ? row[col] : __builtin_inff();
                 }
-                if (running > CAP)
-                {
-                    // the slice is full: remember which values passed (the radius changes with
-                    // the merge) and ask for a merge
-                    my_pass = 0;
-#pragma unroll
-                    for (int j = 0; j < E; ++j)
-                    {
-                        my_pass |= passes(v[j], j) ? (1U << j) : 0U;
-                    }
-                    slot_base = fill;
-                    pending = true;
-                    fill = CAP;
-                    s_flag = 1;
-                    break;
-                }
-                fill = running;
             }
-            if (__builtin_amdgcn_readfirstlane(flag) != 0)
+        };
+        // Software pipelining for small batches: the next chunk is requested before the current one
+        // is filtered, at the price of E more registers and E moves per chunk.  Rows of two waves
+        // (128 threads) leave 8 waves per compute unit, which need the depth also with 4 loads each.
+        constexpr bool PIPE = L <= 2 || (BS == 128 && L <= 4);
+        float ahead[E];
+#pragma unroll
+        for (int j = 0; j < E; ++j)
+        {
+            ahead[j] = 0.0F;
+        }
+        if constexpr (PIPE)
+        {
+            if (left > 0)
+            {
+                load_chunk(ahead, chunk);
+            }
+        }
+
+        // Fill of this wave's slice (wave-uniform).  Passing values take slots in the order
+        // (value index j, lane): value j of the lanes in its pass mask gets consecutive slots after
+        // those of the values before it.
+        //
+        // Only when a chunk does not fit into the slice is per-lane state kept for it: bit j of
+        // my_pass says value j of this lane passed the filter (decided with the radius of that
+        // moment), slot_base is the slot of the chunk's first passing value.  A merge empties every
+        // slice, so slot_base drops by CAP; a value is written in the round where its slot falls
+        // into [0, CAP).
+        int fill = static_cast<int>(first) - wave * CAP;
+        fill = fill < 0 ? 0 : (fill > CAP ? CAP : fill);
+        u32 my_pass = 0;
+        int slot_base = 0;
+        bool pending = false; // values of the chunk in v[] still wait for a slot
+
+        auto lane_rank = [&](u64 mask) -> int {
+            return static_cast<int>(__builtin_amdgcn_mbcnt_hi(
+                static_cast<u32>(mask >> 32U), __builtin_amdgcn_mbcnt_lo(static_cast<u32>(mask), 0U)));
+        };
+
+        // exact filter: below the radius key (an equal value is decided by its label; the +inf
+        // padding of a ragged tail never passes).  A NaN counts as +inf: it is neither below nor above
+        // the radius and its key decides, which can only succeed while the radius is +inf.
+        auto passes = [&](float value, int j) -> bool {
+            bool pass = value < radius;
+            if (!(value < radius) && !(value > radius))
+            {
+                const u32 col = column_of(cur_chunk, j);
+                pass = col < n && make_key(value, label_of(col)) < radius_key;
+            }
+            return pass;
+        };
+
+        // writes the pending values whose slot is inside the slice; returns the end of the
+        // chunk's reservation
+        auto write_pending = [&]() -> int {
+            int running = slot_base;
+#pragma unroll
+            for (int j = 0; j < E; ++j)
+            {
+                const bool mine = ((my_pass >> j) & 1U) != 0;
+                const u64 mask = __builtin_amdgcn_ballot_w64(mine);
+                if (mask != 0)
+                {
+                    const int slot = running + lane_rank(mask);
+                    if (mine && slot >= 0 && slot < CAP)
+                    {
+                        const u32 col = column_of(cur_chunk, j);
+                        slice[slot] = make_key(v[j], label_of(col));
+                    }
+                    running += __popcll(mask);
+                }
+            }
+            return running;
+        };
+
+        for (;;)
+        {
+            // ---- rendezvous: every wave arrives here when it needs a merge, saw the flag, or ran
+            // out of values
+            const bool more_work = pending || left > 0;
+            // (wave-uniform values, stored by every lane: a branch on the lane next to a loop exit
+            // makes the compiler treat the loop state as differing between lanes, which turns the
+            // streaming loop into an exec-masked one with its counters in vector registers)
+            s_fill[wave] = fill;
+            if (more_work)
+            {
+                s_more = 1;
+            }
+            __syncthreads();
+            // (the same in every lane; said explicitly so that the loops stay wave-uniform)
+            int total = 0;
+#pragma unroll
+            for (int w = 0; w < W; ++w)
+            {
+                total += s_fill[w];
+            }
+            total = __builtin_amdgcn_readfirstlane(total);
+            const bool more = __builtin_amdgcn_readfirstlane(s_more) != 0;
+            if (total > 0)
+            {
+                merge_buffer<BS, IPT>(topk, buffer, s_fill, t);
+                // the barriers of the merge lie between the reads above and this reset; the barrier
+                // of the broadcast publishes it together with the radius
+                if (t == 0)
+                {
+                    s_flag = 0;
+                    s_more = 0;
+                }
+                // (the radius from the sample stays until the list has a smaller one)
+                const u64 list_radius = broadcast_radius<IPT>(topk, a.k, &s_radius, t);
+                radius_key = list_radius < radius_key ? list_radius : radius_key;
+                radius = key_value(radius_key);
+            }
+            else
+            {
+                __syncthreads(); // orders the reads above before the reset below
+                if (t == 0)
+                {
+                    s_flag = 0;
+                    s_more = 0;
+                }
+                __syncthreads();
+            }
+            if (!more)
             {
                 break;
             }
+            fill = 0;
+            if (pending)
+            {
+                slot_base -= CAP;
+                const int end = write_pending();
+                if (end > CAP)
+                {
+                    fill = CAP;
+                    s_flag = 1;
+                    continue;
+                }
+                fill = end;
+                pending = false;
+            }
+
+            // ---- streaming: no synchronisation with the other waves except polling the flag
+            while (left > 0)
+            {
+                if constexpr (PIPE)
+                {
+                    // the values of this chunk were requested an iteration (or a merge) ago
+#pragma unroll
+                    for (int j = 0; j < E; ++j)
+                    {
+                        v[j] = ahead[j];
+                    }
+                }
+                else
+                {
+                    load_chunk(v, chunk);
+                }
+                const int flag = __hip_atomic_load(&s_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                cur_chunk = chunk;
+                left -= 1;
+                chunk += static_cast<u32>(jump);
+                jump = (jump > 0 ? static_cast<std::int32_t>(CHUNK) : -static_cast<std::int32_t>(CHUNK)) - jump;
+                if constexpr (PIPE)
+                {
+                    // request the next chunk before this one is filtered: the loads stay in flight
+                    // through the filter and through a merge, if one comes
+                    if (left > 0)
+                    {
+                        load_chunk(ahead, chunk);
+                    }
+                }
+
+                // NaN-propagating minimum (v_minimum3_f32): a lane that holds a NaN of any kind gets a NaN
+                // here and takes the look at every value below (the NaN-ignoring minimum would need
+                // every operand quietened first, and loses values after a signalling NaN otherwise)
+                float smallest = v[0];
+#pragma unroll
+                for (int j = 1; j < E; ++j)
+                {
+                    smallest = __builtin_elementwise_minimum(smallest, v[j]);
+                }
+                // A value equal to the radius passes only with a label below the radius key's.  With
+                // implicit labels every label of this chunk is at least that of its first column, so
+                // when that one is not below, equal values need no look (rows with few distinct
+                // values have one in every chunk).
+                const bool no_ties =
+                    lrow == nullptr && static_cast<std::int32_t>(cur_chunk + label_offset) >= key_label(radius_key);
+                // (negated compares: true for a NaN)
+                if (__builtin_amdgcn_ballot_w64(no_ties ? !(smallest >= radius) : !(smallest > radius)) != 0)
+                {
+                    int running = fill;
+#pragma unroll
+                    for (int j = 0; j < E; ++j)
+                    {
+                        if (__builtin_amdgcn_ballot_w64(!(v[j] > radius)) != 0)
+                        {
+                            const bool pass = passes(v[j], j);
+                            const u64 mask = __builtin_amdgcn_ballot_w64(pass);
+                            if (mask != 0)
+                            {
+                                const int slot = running + lane_rank(mask);
+                                if (pass && slot < CAP)
+                                {
+                                    const u32 col = column_of(cur_chunk, j);
+                                    slice[slot] = make_key(v[j], label_of(col));
+                                }
+                                running += __popcll(mask);
+                            }
+                        }
+                    }
+                    if (running > CAP)
+                    {
+                        // the slice is full: remember which values passed (the radius changes with
+                        // the merge) and ask for a merge
+                        my_pass = 0;
+#pragma unroll
+                        for (int j = 0; j < E; ++j)
+                        {
+                            my_pass |= passes(v[j], j) ? (1U << j) : 0U;
+                        }
+                        slot_base = fill;
+                        pending = true;
+                        fill = CAP;
+                        s_flag = 1;
+                        break;
+                    }
+                    fill = running;
+                }
+                if (__builtin_amdgcn_readfirstlane(flag) != 0)
+                {
+                    break;
+                }
+            }
         }
+
+        if constexpr (ESTIMATE)
+        {
+            // Everything the filter dropped was not below the radius of that moment, and no radius
+            // was above the first one.  If the k-th key of the list got below the first radius, the
+            // dropped values all lie above the list; if not, fewer than k values of the row lie
+            // below the estimate, and the row is done again from +inf.
+            const u32 high = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(radius_key >> 32U)));
+            const u32 low = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(radius_key)));
+            if (estimated && !(((static_cast<u64>(high) << 32U) | low) < first_key))
+            {
+                estimated = false;
+                continue;
+            }
+        }
+        break;
     }
 
     float* __restrict__ out_d = a.out_dist + row_idx * a.out_stride;

@@ -138,6 +138,65 @@ def test_rows_long_enough_for_the_sampled_radius(bk, dev, oracle):
         assert np.array_equal(gd, ed) and np.array_equal(gl, el), (k, block)
 
 
+def _estimate_sample_columns(cols, block):
+    """Columns of the evenly spread sample that lists of 1024 entries and more estimate their
+    first radius from (rows of at least 256 x block size values)."""
+    pieces = min(4096 // block, cols // (256 * block))
+    segment = (cols // pieces) & ~3
+    offset = (segment // 2 - 2 * block) & ~3
+    return np.concatenate([np.arange(p * segment + offset, p * segment + offset + 4 * block)
+                           for p in range(pieces)])
+
+
+@pytest.mark.parametrize("block,k,batch", [(128, 1024, 8), (128, 2048, 16), (256, 600, 8), (256, 2048, 8),
+                                           (256, 2048, 12), (512, 513, 4), (512, 1024, 8), (512, 2047, 8),
+                                           (512, 2048, 16)])
+def test_rows_long_enough_for_the_estimated_radius(bk, dev, oracle, block, k, batch):
+    """Lists of 1024 entries and more on long rows start from an estimate of the k-th smallest
+    value and repeat the row when the estimate proves too low; the result must not depend on
+    either.  Rows where the estimate holds, rows where it cannot hold (the sampled columns hold
+    the only small values, fewer than k of them), ties at the estimate, sorted rows, rows with
+    few finite values."""
+    rng = np.random.default_rng(block + k)
+    rows, cols = 12, 1 << 18
+    sample = _estimate_sample_columns(cols, block)
+    m = oracle.uniform_matrix(77 + k, rows, cols, -2.0, 2.0)
+    m[1] = np.sort(m[1])
+    m[2] = np.sort(m[2])[::-1]
+    m[3] = 5.0 + rng.random(cols, dtype=np.float32)          # small values only where the sample looks:
+    m[3, sample] = rng.random(sample.size, dtype=np.float32)  # more than k of them
+    m[4] = 5.0 + rng.random(cols, dtype=np.float32)
+    few = rng.choice(sample, size=k // 2, replace=False)      # fewer than k of them
+    m[4, few] = rng.random(few.size, dtype=np.float32)
+    m[5] = 5.0                                                # ties above the few small values
+    m[5, few] = rng.random(few.size, dtype=np.float32)
+    m[6] = np.round(m[6] * 4) / 4                             # 17 distinct values
+    m[7] = np.inf                                             # fewer finite values than k, all sampled
+    m[7, few[:100]] = rng.random(100, dtype=np.float32)
+    m[8] = np.inf                                             # nothing finite in the sample
+    rest = np.setdiff1d(np.arange(cols), sample)
+    m[8, rest[::3]] = rng.random(rest[::3].size, dtype=np.float32)
+    m[9, sample] = np.nan                                     # a sample of NaNs
+    m[10, sample] = -3.0                                      # the sample is one value, below the rest
+    m[11] = m[11, 0]                                          # constant row
+    want = np.where(np.isnan(m), np.float32(np.inf), m)       # a NaN counts as +inf
+    gd, gl = _run(bk, dev, m, k, block=block, batch=batch)
+    ed, el = oracle.topk(want, k)
+    assert np.array_equal(gd, ed) and np.array_equal(gl, el)
+    # rows that do not start on a 16-byte boundary (4-byte loads, the sample too), explicit labels
+    import torch
+    t = torch.from_numpy(m).to(dev)
+    od, ol = bk.topk_bits(t[:, 3:], k, block, batch)
+    torch.cuda.synchronize()
+    ed, el = oracle.topk(np.ascontiguousarray(want[:, 3:]), k)
+    assert np.array_equal(od.cpu().numpy(), ed) and np.array_equal(ol.cpu().numpy(), el)
+    labels = np.stack([rng.permutation(cols) for _ in range(rows)]).astype(np.int32)
+    offsets = (np.arange(rows) * 7919).astype(np.int32)
+    gd, gl = _run(bk, dev, m, k, block=block, batch=batch, labels=labels, offsets=offsets)
+    ed, el = oracle.topk(want, k, labels=labels, label_offsets=offsets)
+    assert np.array_equal(gd, ed) and np.array_equal(gl, el)
+
+
 def test_negative_values_and_infinities(bk, dev, oracle):
     m = oracle.uniform_matrix(3, 4, 20000, -5.0, 5.0)
     m[0, 17] = -np.inf
