@@ -15,6 +15,10 @@ constexpr int FQ_QB = FQ_QW * FQ_WAVES;       // queries per workgroup
 constexpr int FQ_CAP = 32;                    // buffer slots per query (= points per MFMA tile); twice
                                               // that for long lists in few dimensions (fused_geometry)
 
+constexpr int FUSED_PLAIN = -1;
+constexpr int FUSED_REPEAT_MARKED = -2;
+constexpr int FUSED_FIRST_RADIUS_FROM = 0;
+
 struct fused_args
 {
     const float* queries; // dim-major, stride q
@@ -26,6 +30,18 @@ struct fused_args
     std::int32_t* out_label;
     int splits;           // the points are cut into `splits` ranges, one per blockIdx.y
     int split_points;     // points per range (a multiple of 256)
+    int list_stride;      // floats between the lists of consecutive (query, split) pairs: K, or more
+    // A launch over a sample of the points (sample_scale > 1): every sample_scale-th stage of the
+    // point matrix is visited, `visit` points in all, which are numbered 0 .. visit-1 in the
+    // lists.  Otherwise visit = n, sample_scale = 1 and sample_offset = 0.
+    int visit;            // points visited (the launcher sets it for a sample)
+    int sample_scale;     // visited point v of a stage that starts at v0 is point
+    int sample_offset;    //   v0 * sample_scale + sample_offset + (v - v0) of the matrix
+    // FUSED_PLAIN: radii start from +inf.  FUSED_FIRST_RADIUS_FROM + r: the radius of query g starts
+    // from out_dist[g * list_stride + r], put there by a launch over a sample; a query whose k-th
+    // distance does not get below that value is marked.  FUSED_REPEAT_MARKED: only workgroups
+    // with a marked query run, from +inf.
+    int first_radius;
 };
 
 // one per compiled list length K (fused_inst.hip); split: products from three bf16 pieces per

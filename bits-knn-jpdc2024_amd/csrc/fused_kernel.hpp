@@ -145,8 +145,9 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     const int dim = a.dim;
     // this workgroup's range of points
     const int n_begin = static_cast<int>(blockIdx.y) * a.split_points;
-    const int n = a.n < n_begin + a.split_points ? a.n : n_begin + a.split_points;
+    const int n = a.visit < n_begin + a.split_points ? a.visit : n_begin + a.split_points;
     const size_t total_points = static_cast<size_t>(a.n);
+    const size_t list_stride = static_cast<size_t>(a.list_stride);
     const int t = static_cast<int>(threadIdx.x);
     const int lane = t & (WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(t / WAVE);
@@ -209,7 +210,26 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     }
     __syncthreads();
 
-    float radius = __builtin_inff(); // k-th smallest distance of my query so far
+    // A first radius from a launch over a sample of the points (FUSED_FIRST_RADIUS_FROM + rank):
+    // what the filter drops is not below it, so the list of a query is exact if its k-th distance
+    // ends up below its first radius.  A query where it does not gets a NaN as its k-th distance (no
+    // list holds one otherwise), and a further launch (FUSED_REPEAT_MARKED) repeats the pass of the
+    // workgroups that have such a query from +inf; all others leave at once.
+    float first_radius = __builtin_inff();
+    if (a.first_radius >= FUSED_FIRST_RADIUS_FROM && my_q < a.q)
+    {
+        first_radius = a.out_dist[static_cast<size_t>(my_q) * list_stride + (a.first_radius - FUSED_FIRST_RADIUS_FROM)];
+    }
+    if (a.first_radius == FUSED_REPEAT_MARKED)
+    {
+        const bool marked =
+            my_q < a.q && __builtin_isnan(a.out_dist[static_cast<size_t>(my_q) * list_stride + K - 1]);
+        if (__syncthreads_or(marked ? 1 : 0) == 0)
+        {
+            return;
+        }
+    }
+    float radius = first_radius;     // k-th smallest distance of my query so far
     int fill = 0;                    // used slots of my query's buffer (same in both lanes of a query)
     bool have_list = false;          // wave-uniform: the lists in the output arrays are valid
     bool merged = false;             // wave-uniform: this wave has merged during the current stage
@@ -259,7 +279,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         std::int32_t next_label[R];
         auto request_list = [&](int pass) __attribute__((always_inline)) {
             const int gq = wave_q0 + pass * QPP + lane / LPQ;
-            const size_t at = (static_cast<size_t>(gq) * a.splits + blockIdx.y) * K + sub * R;
+            const size_t at = (static_cast<size_t>(gq) * a.splits + blockIdx.y) * list_stride + sub * R;
 #pragma unroll
             for (int r = 0; r < R; ++r)
             {
@@ -318,7 +338,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 const int i = sub * R + r;
                 if (i < K && gq < a.q)
                 {
-                    const size_t at = (static_cast<size_t>(gq) * a.splits + blockIdx.y) * K + i;
+                    const size_t at = (static_cast<size_t>(gq) * a.splits + blockIdx.y) * list_stride + i;
                     a.out_dist[at] = key_value(list[r]);
                     a.out_label[at] = key_label(list[r]);
                 }
@@ -331,7 +351,8 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        radius = wx[ql];
+        // (a first radius from a sample stays until the list has a smaller one)
+        radius = fminf(wx[ql], first_radius);
         fill = 0;
         have_list = true;
         merged = true;
@@ -438,9 +459,11 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                           : OUTSIDE;
     }
     auto fetch = [&](int base) {
+        // first point of the stage in the matrix (a sample visits every sample_scale-th stage)
+        const int at = base * a.sample_scale + a.sample_offset;
         if (small_points)
         {
-            const int stage_off = base * static_cast<int>(sizeof(float));
+            const int stage_off = at * static_cast<int>(sizeof(float));
             if (base + PT <= n)
             {
 #pragma unroll
@@ -465,13 +488,13 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         }
         else
         {
-            const int j = base + sp;
+            const int j = at + sp;
 #pragma unroll
             for (int i = 0; i < VPT; ++i)
             {
                 const int dd = dim_of(i);
                 pre[i] = 0.0F;
-                if (dd < dim && j < n)
+                if (dd < dim && base + sp < n)
                 {
                     pre[i] = a.points[static_cast<size_t>(dd) * total_points + j];
                 }
@@ -792,6 +815,11 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 
     // whatever is left in the buffers; also writes the lists of queries that never merged
     merge_event();
+    // (the radius is the k-th distance of the finished list now if that is below the first radius)
+    if (first_radius < __builtin_inff() && !(radius < first_radius) && half == 0)
+    {
+        a.out_dist[static_cast<size_t>(my_q) * list_stride + K - 1] = __builtin_nanf("");
+    }
 }
 
 template <int K, int DP, bool SPLIT>
@@ -808,9 +836,18 @@ hipError_t launch_fused(const fused_args& a, hipStream_t stream)
             return status;
         }
     }
+    fused_args args = a;
+    if (a.sample_scale > 1)
+    {
+        // every sample_scale-th stage, the one in the middle of its group
+        constexpr int PT = fused_geometry<DP, SPLIT, K>::PT;
+        args.visit = a.n / (PT * a.sample_scale) * PT;
+        args.sample_offset = a.sample_scale / 2 * PT;
+        args.split_points = (args.visit + 255) / 256 * 256;
+    }
     const unsigned grid = static_cast<unsigned>((a.q + FQ_QB - 1) / FQ_QB);
     hipLaunchKernelGGL((fused_kernel<K, DP, SPLIT>), dim3(grid, static_cast<unsigned>(a.splits)),
-                       dim3(FQ_THREADS), lds_bytes, stream, a);
+                       dim3(FQ_THREADS), lds_bytes, stream, args);
     return hipGetLastError();
 }
 

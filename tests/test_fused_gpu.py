@@ -221,6 +221,43 @@ def test_long_lists_stay_in_the_fused_kernel(bk, dev, oracle, k):
     assert np.array_equal(gd, fd) and np.array_equal(gl, fl)
 
 
+def _sampled_points(n, d, split):
+    """Points the launch over a sample visits (lists of 128 and more on at least 2^17 points
+    start from radii taken from it): every 64th stage, the one in the middle of its group."""
+    if split:
+        stage = 128 if d <= 16 else (64 if d <= 32 else 32)
+    else:
+        stage = 256 if d <= 16 else (128 if d <= 32 else (64 if d <= 64 else 32))
+    stages = n // (stage * 64)
+    return np.concatenate([np.arange((s * 64 + 32) * stage, (s * 64 + 33) * stage) for s in range(stages)])
+
+
+@pytest.mark.parametrize("d,k,arithmetic", [(8, 128, "fp32"), (8, 256, "fp32"), (32, 256, "fp32"), (100, 128, "fp32"),
+                                            (16, 256, "bf16x3"), (48, 128, "bf16x3")])
+def test_first_radius_from_a_sample(bk, dev, oracle, d, k, arithmetic):
+    """Long lists on many points start from radii that a launch over a sample of the points
+    estimates, and workgroups with a query whose estimate proved too low repeat their pass; the
+    result must not depend on either.  Uniform points (the estimates hold), and points whose
+    sampled stages hold the only near ones, more than k of them (every estimate is too low)."""
+    n, q = (1 << 17) + 777, 200
+    rng = np.random.default_rng(d * k)
+    queries = rng.random((q, d), dtype=np.float32)
+    points = rng.random((n, d), dtype=np.float32)
+    arithmetic = bk.FUSED_BF16X3 if arithmetic == "bf16x3" else None
+    gd, gl = _fused(bk, dev, points, queries, k, arithmetic=arithmetic)
+    _check(oracle, points, queries, k, gd, gl)
+    assert not np.isnan(gd).any()
+    sample = _sampled_points(n, d, arithmetic is not None)
+    assert sample.size >= 8 * 32
+    points = rng.random((n, d), dtype=np.float32)
+    points[:, :4] += 1.0                    # all points a step away in four dimensions ...
+    points[sample] = rng.random((sample.size, d), dtype=np.float32)    # ... but the sampled ones
+    queries[::2, :4] += 1.0                 # every other query sits among the far points
+    gd, gl = _fused(bk, dev, points, queries, k, arithmetic=arithmetic)
+    _check(oracle, points, queries, k, gd, gl)
+    assert not np.isnan(gd).any()
+
+
 def test_random_shapes_against_the_oracle(bk, dev, oracle):
     """40 random problems over dimensions on both sides of every padded size, all list lengths,
     ragged point and query counts, with the plain entry point, the workspace the library asks for
