@@ -81,22 +81,32 @@ int choose_splits(int q, int n)
 }
 
 // The first radii of a launch come from a launch over a sample of the points, one stage in every
-// SAMPLE_SCALE: the value of rank r among a query's distances to the sample, r the smallest rank
-// that at least r of the query's k nearest points fall into the sample (which is when fewer than k
-// points lie below that value, and the query's workgroup has to repeat its pass) with a probability
-// of at most 10^-10 for points in random order.  Returns 0 when the lists of the sample launch,
-// which have min(k, 32) entries, do not reach that rank.
+// `scale`: the value of rank r among a query's distances to the sample, r the smallest rank that
+// at least r of the query's k nearest points fall into the sample (which is when fewer than k
+// points lie below that value, and the query's workgroup has to repeat its pass) with a
+// probability of at most 10^-10 for points in random order.  Returns 0 when the lists of the
+// sample launch, which have min(k, 32) entries, do not reach that rank.
 //
-// Measured on 65536 queries x 2^20 points: 51.6 -> 47.5 ms at k = 256 and 44.3 -> 43.7 ms at k = 128
-// in 32 dimensions (26.1 -> 23.7 and 21.2 -> 20.6 ms in 8); up to k = 64 the launch over the sample
-// costs more than the merges it saves, so shorter lists start from +inf.
+// One range of points (many queries): every 64th stage; lists of 128 and more only.  Measured on
+// 65536 queries x 2^20 points: 51.6 -> 47.5 ms at k = 256 and 44.3 -> 43.7 ms at k = 128 in 32
+// dimensions (26.1 -> 23.7 and 21.2 -> 20.6 ms in 8); up to k = 64 the launch over the sample costs
+// more than the merges it saves.
+//
+// Several ranges (few queries): the list of a range hardly converges on its own (k (1 + ln(range / k))
+// candidates per range and query), while hardly any point of a range lies below a radius taken
+// from the whole point set (q = 8192, n = 2^17, d = 8: 2.66 -> 1.56 ms at k = 256, 1.31 -> 1.05 ms at
+// k = 128, 0.88 -> 0.78 ms at k = 64; q = 1024, n = 2^20: 2.68 -> 1.04, 1.32 -> 0.88, 0.89 -> 0.76 ms).
+// The sample launch runs on the few workgroups the queries give (it is not cut into ranges), so it
+// takes every 256th stage only.
 constexpr int SAMPLE_SCALE = 64;
-constexpr int SAMPLE_MIN_POINTS = 1 << 17; // at least 8 sampled stages of any size
+constexpr int SAMPLE_SCALE_RANGES = 256;
+constexpr int SAMPLE_MIN_POINTS = 1 << 17; // at least 8 (2 with ranges) sampled stages of any size
 constexpr int SAMPLE_MIN_K = 128;
+constexpr int SAMPLE_MIN_K_RANGES = 64; // (k <= 32: the three extra launches cost what the merges save)
 
-int first_radius_rank(int k)
+int first_radius_rank(int k, int scale)
 {
-    const double p = 1.0 / SAMPLE_SCALE;
+    const double p = 1.0 / scale;
     const int longest = k < 32 ? k : 32;
     // binomial(k, p) probabilities from the top down: the tail from r on
     double pmf[257];
@@ -228,7 +238,8 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
         splits /= 2;
     }
     const size_t pairs = static_cast<size_t>(q) * static_cast<size_t>(splits) * static_cast<size_t>(k);
-    fused_args a{queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, 1, 0, k, n, 1, 0, FUSED_PLAIN};
+    fused_args a{queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, 1, 0, k, n, 1, 0, FUSED_PLAIN,
+                 out_dist, k};
     if (splits > 1)
     {
         // partial lists [q][splits][k] in the workspace: distances first, then labels
@@ -240,35 +251,53 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
 
     auto* hip_stream = static_cast<hipStream_t>(stream);
     const bool split = arithmetic == BITSKNN_FUSED_BF16X3;
+    // one bits pass over the splits*k candidates of every query, labels carried along
+    auto reduce_ranges = [&]() -> int {
+        const size_t cols = static_cast<size_t>(splits) * static_cast<size_t>(k);
+        return bitsknn_topk_bits_f32(a.out_dist, cols, a.out_label, cols, nullptr, static_cast<size_t>(q), cols,
+                                     out_dist, out_label, static_cast<size_t>(k), static_cast<std::uint32_t>(k),
+                                     128, 4, 0, stream);
+    };
     hipError_t status = hipSuccess;
-    const int rank = splits == 1 && n >= SAMPLE_MIN_POINTS && k >= SAMPLE_MIN_K ? first_radius_rank(k) : 0;
+    const int scale = splits == 1 ? SAMPLE_SCALE : SAMPLE_SCALE_RANGES;
+    const int rank = n >= SAMPLE_MIN_POINTS && k >= (splits == 1 ? SAMPLE_MIN_K : SAMPLE_MIN_K_RANGES)
+                         ? first_radius_rank(k, scale)
+                         : 0;
     if (rank > 0)
     {
-        // lists of min(k, 32) nearest sample points into the first entries of the output rows;
-        // the launch below takes its first radii from them and then overwrites them
+        // lists of min(k, 32) nearest sample points into the first entries of the caller's output
+        // rows, one range; the launch below takes its first radii from them, and they are
+        // overwritten by its lists (one range) or by the reduced lists (several)
         fused_args sample = a;
-        sample.sample_scale = SAMPLE_SCALE;
+        sample.out_dist = out_dist;
+        sample.out_label = out_label;
+        sample.splits = 1;
+        sample.sample_scale = scale;
         status = launch_for_k(k < 32 ? k : 32, sample, split, hip_stream);
         BITSKNN_HIP_CHECK(status);
         a.first_radius = FUSED_FIRST_RADIUS_FROM + rank - 1;
     }
     status = launch_for_k(k, a, split, hip_stream);
     BITSKNN_HIP_CHECK(status);
-    if (rank > 0)
-    {
-        // the workgroups with a query whose first radius proved too low (marked by the launch
-        // above) repeat their pass from +inf; the others leave at once
-        a.first_radius = FUSED_REPEAT_MARKED;
-        status = launch_for_k(k, a, split, hip_stream);
-    }
-    BITSKNN_HIP_CHECK(status);
     if (splits > 1)
     {
-        // one bits pass over the splits*k candidates of every query, labels carried along
-        const size_t cols = static_cast<size_t>(splits) * static_cast<size_t>(k);
-        return bitsknn_topk_bits_f32(a.out_dist, cols, a.out_label, cols, nullptr, static_cast<size_t>(q),
-                                     cols, out_dist, out_label, static_cast<size_t>(k),
-                                     static_cast<std::uint32_t>(k), 128, 4, 0, stream);
+        const int reduced = reduce_ranges();
+        if (reduced != BITSKNN_OK)
+        {
+            return reduced;
+        }
+    }
+    if (rank > 0)
+    {
+        // the workgroups with a query whose first radius proved too low repeat their pass from
+        // +inf (all ranges of such a query); the others leave at once
+        a.first_radius = FUSED_REPEAT_MARKED;
+        status = launch_for_k(k, a, split, hip_stream);
+        BITSKNN_HIP_CHECK(status);
+        if (splits > 1)
+        {
+            return reduce_ranges();
+        }
     }
     return BITSKNN_OK;
 }

@@ -38,10 +38,15 @@ struct fused_args
     int sample_scale;     // visited point v of a stage that starts at v0 is point
     int sample_offset;    //   v0 * sample_scale + sample_offset + (v - v0) of the matrix
     // FUSED_PLAIN: radii start from +inf.  FUSED_FIRST_RADIUS_FROM + r: the radius of query g starts
-    // from out_dist[g * list_stride + r], put there by a launch over a sample; a query whose k-th
-    // distance does not get below that value is marked.  FUSED_REPEAT_MARKED: only workgroups
-    // with a marked query run, from +inf.
+    // from final_dist[g * final_stride + r], put there by a launch over a sample; with one range of
+    // points, a query whose k-th distance does not get below that value gets a NaN as its k-th
+    // distance (with several ranges a range's list need not fill up, and a query that is short of k
+    // distances below its first radius shows as +inf at the end of its reduced list).
+    // FUSED_REPEAT_MARKED: only workgroups with a query whose k-th final distance is NaN or +inf run,
+    // from +inf.
     int first_radius;
+    const float* final_dist; // the caller's output array (out_dist itself with one range of points)
+    int final_stride;
 };
 
 // one per compiled list length K (fused_inst.hip); split: products from three bf16 pieces per

@@ -17,7 +17,7 @@
 //    lane holds 16 distances of ONE query (column), so the filter is a min-tree over 16
 //    registers and one compare against that query's radius.
 //  * Every query has a 32-slot buffer in LDS (64 slots for lists of 128 and more in up to 16
-//    dimensions).  Slots are handed out without atomics: the two
+//    dimensions when the points are cut into ranges).  Slots are handed out without atomics: the two
 //    lanes that share a query exchange their pass counts, and the fill is kept in a register.
 //    Before a tile would overflow any buffer of the wave, the wave merges all its buffers; the
 //    other waves of the workgroup, which would wait for it at the stage barrier, then merge
@@ -70,14 +70,18 @@ __device__ __forceinline__ float min3(float a, float b, float c)
 // dimensions, one 16-byte cell per point (the A operand of v_mfma_f32_32x32x16_bf16), then the
 // norms of the points.
 // Per-query buffers: 32 slots, the points of one matrix tile.  Every merge pays for the whole list,
-// so for lists of 128 entries and more the buffers have 64 slots where the stages leave room for
-// them (up to 16 dimensions, with smaller stages): half as many merges (q = 8192, n = 2^17,
-// d = 8: 4.4 -> 2.7 ms at k = 256, 1.7 -> 1.3 ms at k = 128; at k = 64 the smaller stages cost more
-// than the merges save).
-template <int DP, bool SPLIT, int K>
+// so for lists of 128 entries and more the buffers can have 64 slots where the stages leave room
+// for them (up to 16 dimensions, with smaller stages): half as many merges.  That pays where the
+// lists hardly converge, i.e. with few queries whose points are cut into ranges (q = 8192,
+// n = 2^17, d = 8: 4.4 -> 2.7 ms at k = 256 and 1.7 -> 1.3 ms at k = 128 before the first radii from
+// a sample, 2.19 -> 1.65 and 1.18 -> 1.10 ms with them; at k = 64 the smaller stages cost more than
+// the merges save).  With one range of points the smaller stages cost more than the merges (65536
+// queries x 2^20 points, d = 16, k = 128: 33.9 ms with 64 slots, 24.8 ms with 32), so WIDE_OK is set
+// for launches over ranges only.
+template <int DP, bool SPLIT, int K, bool WIDE_OK = false>
 struct fused_geometry
 {
-    static constexpr bool WIDE = K >= 128 && DP <= 16 && !SPLIT;
+    static constexpr bool WIDE = WIDE_OK && K >= 128 && DP <= 16 && !SPLIT;
     static constexpr int CAP = WIDE ? 2 * FQ_CAP : FQ_CAP; // buffer slots per query
     static constexpr int DK = DP < 16 ? 16 : DP;       // SPLIT: dimensions padded to whole matrix steps
     static constexpr int KB = DK / 16;                 // SPLIT: matrix steps of 16 dimensions
@@ -106,10 +110,10 @@ struct fused_geometry
 
 // K: list length.  DP: dimension padded to 8, 16, 32, 64, 128 or 256 (padding rows are zero on
 // both sides of the product).
-template <int K, int DP, bool SPLIT>
+template <int K, int DP, bool SPLIT, bool WIDE_OK>
 __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 {
-    using G = fused_geometry<DP, SPLIT, K>;
+    using G = fused_geometry<DP, SPLIT, K, WIDE_OK>;
     constexpr int PT = G::PT;
     constexpr int CAP = G::CAP;
     // Norms in the accumulator: where one staging thread carries a whole point (DP <= 16) its
@@ -211,19 +215,22 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     __syncthreads();
 
     // A first radius from a launch over a sample of the points (FUSED_FIRST_RADIUS_FROM + rank):
-    // what the filter drops is not below it, so the list of a query is exact if its k-th distance
-    // ends up below its first radius.  A query where it does not gets a NaN as its k-th distance (no
-    // list holds one otherwise), and a further launch (FUSED_REPEAT_MARKED) repeats the pass of the
-    // workgroups that have such a query from +inf; all others leave at once.
+    // what the filter drops is not below it, so the list of a query is exact if k of its distances
+    // lie below its first radius.  With one range of points a query where they do not gets a NaN as
+    // its k-th distance (no list holds one otherwise); with several ranges the lists of a range need
+    // not fill up, and such a query shows as +inf at the end of its reduced list.  A further launch
+    // (FUSED_REPEAT_MARKED) repeats the pass of the workgroups that have such a query from +inf;
+    // all others leave at once.
     float first_radius = __builtin_inff();
     if (a.first_radius >= FUSED_FIRST_RADIUS_FROM && my_q < a.q)
     {
-        first_radius = a.out_dist[static_cast<size_t>(my_q) * list_stride + (a.first_radius - FUSED_FIRST_RADIUS_FROM)];
+        first_radius = a.final_dist[static_cast<size_t>(my_q) * a.final_stride + (a.first_radius - FUSED_FIRST_RADIUS_FROM)];
     }
     if (a.first_radius == FUSED_REPEAT_MARKED)
     {
+        // (negated compare: true for a NaN as well)
         const bool marked =
-            my_q < a.q && __builtin_isnan(a.out_dist[static_cast<size_t>(my_q) * list_stride + K - 1]);
+            my_q < a.q && !(a.final_dist[static_cast<size_t>(my_q) * a.final_stride + K - 1] < __builtin_inff());
         if (__syncthreads_or(marked ? 1 : 0) == 0)
         {
             return;
@@ -816,20 +823,21 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     // whatever is left in the buffers; also writes the lists of queries that never merged
     merge_event();
     // (the radius is the k-th distance of the finished list now if that is below the first radius)
-    if (first_radius < __builtin_inff() && !(radius < first_radius) && half == 0)
+    if (a.splits == 1 && first_radius < __builtin_inff() && !(radius < first_radius) && half == 0)
     {
         a.out_dist[static_cast<size_t>(my_q) * list_stride + K - 1] = __builtin_nanf("");
     }
 }
 
-template <int K, int DP, bool SPLIT>
-hipError_t launch_fused(const fused_args& a, hipStream_t stream)
+template <int K, int DP, bool SPLIT, bool WIDE_OK>
+hipError_t launch_fused_as(const fused_args& a, hipStream_t stream)
 {
-    constexpr size_t lds_bytes = fused_geometry<DP, SPLIT, K>::lds_bytes();
+    using G = fused_geometry<DP, SPLIT, K, WIDE_OK>;
+    constexpr size_t lds_bytes = G::lds_bytes();
     if (lds_bytes > 48 * 1024)
     {
         const hipError_t status =
-            hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<K, DP, SPLIT>),
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<K, DP, SPLIT, WIDE_OK>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
         if (status != hipSuccess)
         {
@@ -840,15 +848,29 @@ hipError_t launch_fused(const fused_args& a, hipStream_t stream)
     if (a.sample_scale > 1)
     {
         // every sample_scale-th stage, the one in the middle of its group
-        constexpr int PT = fused_geometry<DP, SPLIT, K>::PT;
+        constexpr int PT = G::PT;
         args.visit = a.n / (PT * a.sample_scale) * PT;
         args.sample_offset = a.sample_scale / 2 * PT;
         args.split_points = (args.visit + 255) / 256 * 256;
     }
     const unsigned grid = static_cast<unsigned>((a.q + FQ_QB - 1) / FQ_QB);
-    hipLaunchKernelGGL((fused_kernel<K, DP, SPLIT>), dim3(grid, static_cast<unsigned>(a.splits)),
+    hipLaunchKernelGGL((fused_kernel<K, DP, SPLIT, WIDE_OK>), dim3(grid, static_cast<unsigned>(a.splits)),
                        dim3(FQ_THREADS), lds_bytes, stream, args);
     return hipGetLastError();
+}
+
+// launches over ranges of points take the 64-slot buffers where the geometry has them
+template <int K, int DP, bool SPLIT>
+hipError_t launch_fused(const fused_args& a, hipStream_t stream)
+{
+    if constexpr (fused_geometry<DP, SPLIT, K, true>::WIDE)
+    {
+        if (a.splits > 1)
+        {
+            return launch_fused_as<K, DP, SPLIT, true>(a, stream);
+        }
+    }
+    return launch_fused_as<K, DP, SPLIT, false>(a, stream);
 }
 
 } // namespace

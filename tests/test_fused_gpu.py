@@ -30,7 +30,7 @@ def _fused(bk, dev, points, queries, k, params=(8, 4, 2), bqd=1, dim_mult=1, wor
     return od.cpu().numpy(), ol.cpu().numpy()
 
 
-def _check(oracle, points, queries, k, gd, gl, min_recall=0.999):
+def _check(oracle, points, queries, k, gd, gl, min_recall=0.999, bar_dim=None):
     n = points.shape[0]
     part = oracle.dist(queries, points, "partial")
     ed, el = oracle.topk(part, k)
@@ -46,7 +46,8 @@ def _check(oracle, points, queries, k, gd, gl, min_recall=0.999):
     scale = np.abs(ref_at) + qn
     assert np.max(np.abs(gd[:, :kk] - ref_at) / scale) <= REL
     # k-th neighbour distance and recall
-    assert_kth_distance(queries, ed[:, kk - 1], gd[:, kk - 1], points.shape[1], (n, queries.shape[0], k))
+    # (bar_dim: data whose distances cancel harder than uniform points' do take the bar of few dimensions)
+    assert_kth_distance(queries, ed[:, kk - 1], gd[:, kk - 1], bar_dim or points.shape[1], (n, queries.shape[0], k))
     recall = np.mean([len(set(a[:kk]) & set(b[:kk])) / kk for a, b in zip(gl, el)])
     if recall < min_recall:
         # Neighbours closer together than fp32 resolves (many points on a line, say): which of
@@ -104,7 +105,10 @@ def test_ragged_counts(bk, dev, oracle, n, q):
                                      (9000, 1000, 8, 64), (131072, 1024, 5, 128), (40000, 128, 8, 256)])
 def test_point_split_variant_with_workspace(bk, dev, oracle, n, q, d, k):
     """The workspace entry point cuts the points into ranges when queries are few; its result must
-    equal the plain entry point's bit for bit (same distances, canonical ties)."""
+    equal the plain entry point's bit for bit (same distances, canonical ties).  Lists of 128 and
+    more in up to 16 dimensions are the exception: their kernel over ranges has 64-slot buffers and
+    smaller stages, in which the norm of a point is added last instead of first, so the distances
+    may differ in their last bits (both results meet the bar against the oracle)."""
     import torch
     p, s = oracle.generate(n + q + d, n, q, d)
     # the workspace holds partial lists only, whatever the list length: never the distance matrix
@@ -113,7 +117,12 @@ def test_point_split_variant_with_workspace(bk, dev, oracle, n, q, d, k):
     gd, gl = _fused(bk, dev, p, s, k, workspace="auto")
     _check(oracle, p, s, k, gd, gl)
     pd, pl = _fused(bk, dev, p, s, k)
-    assert np.array_equal(gd, pd) and np.array_equal(gl, pl)
+    if k >= 128 and d <= 16:
+        _check(oracle, p, s, k, pd, pl)
+        scale = np.abs(pd) + (s.astype(np.float64) ** 2).sum(1)[:, None]
+        assert np.max(np.abs(gd - pd) / scale) <= 1e-6
+    else:
+        assert np.array_equal(gd, pd) and np.array_equal(gl, pl)
 
 
 def test_smaller_workspace_means_fewer_ranges(bk, dev, oracle):
@@ -221,40 +230,51 @@ def test_long_lists_stay_in_the_fused_kernel(bk, dev, oracle, k):
     assert np.array_equal(gd, fd) and np.array_equal(gl, fl)
 
 
-def _sampled_points(n, d, split):
-    """Points the launch over a sample visits (lists of 128 and more on at least 2^17 points
-    start from radii taken from it): every 64th stage, the one in the middle of its group."""
+def _sampled_points(n, d, split, scale):
+    """Points the launch over a sample visits (on at least 2^17 points, lists of 128 and more,
+    or of 64 and more when the points are cut into ranges, start from radii taken from
+    it): every `scale`-th stage, the one in the middle of its group."""
     if split:
         stage = 128 if d <= 16 else (64 if d <= 32 else 32)
     else:
         stage = 256 if d <= 16 else (128 if d <= 32 else (64 if d <= 64 else 32))
-    stages = n // (stage * 64)
-    return np.concatenate([np.arange((s * 64 + 32) * stage, (s * 64 + 33) * stage) for s in range(stages)])
+    stages = n // (stage * scale)
+    half = scale // 2
+    return np.concatenate([np.arange((s * scale + half) * stage, (s * scale + half + 1) * stage)
+                           for s in range(stages)])
 
 
-@pytest.mark.parametrize("d,k,arithmetic", [(8, 128, "fp32"), (8, 256, "fp32"), (32, 256, "fp32"), (100, 128, "fp32"),
-                                            (16, 256, "bf16x3"), (48, 128, "bf16x3")])
-def test_first_radius_from_a_sample(bk, dev, oracle, d, k, arithmetic):
-    """Long lists on many points start from radii that a launch over a sample of the points
+@pytest.mark.parametrize("d,k,arithmetic,ranges", [(8, 128, "fp32", False), (8, 256, "fp32", False),
+                                                   (32, 256, "fp32", False), (100, 128, "fp32", False),
+                                                   (16, 256, "bf16x3", False), (48, 128, "bf16x3", False),
+                                                   (8, 64, "fp32", True), (8, 256, "fp32", True),
+                                                   (16, 128, "fp32", True), (32, 64, "fp32", True),
+                                                   (24, 128, "bf16x3", True)])
+def test_first_radius_from_a_sample(bk, dev, oracle, d, k, arithmetic, ranges):
+    """Lists on many points start from radii that a launch over a sample of the points
     estimates, and workgroups with a query whose estimate proved too low repeat their pass; the
     result must not depend on either.  Uniform points (the estimates hold), and points whose
-    sampled stages hold the only near ones, more than k of them (every estimate is too low)."""
+    sampled stages hold the only near ones, more than k of them (every estimate is too low).
+    `ranges`: with a workspace, so that the few queries search the points in ranges."""
     n, q = (1 << 17) + 777, 200
     rng = np.random.default_rng(d * k)
     queries = rng.random((q, d), dtype=np.float32)
     points = rng.random((n, d), dtype=np.float32)
     arithmetic = bk.FUSED_BF16X3 if arithmetic == "bf16x3" else None
-    gd, gl = _fused(bk, dev, points, queries, k, arithmetic=arithmetic)
+    workspace = "auto" if ranges else None
+    if ranges:
+        assert bk.fused_workspace_bytes(q, n, k) > 0
+    gd, gl = _fused(bk, dev, points, queries, k, arithmetic=arithmetic, workspace=workspace)
     _check(oracle, points, queries, k, gd, gl)
     assert not np.isnan(gd).any()
-    sample = _sampled_points(n, d, arithmetic is not None)
-    assert sample.size >= 8 * 32
+    sample = _sampled_points(n, d, arithmetic is not None, 256 if ranges else 64)
+    assert sample.size >= 2 * 32
     points = rng.random((n, d), dtype=np.float32)
     points[:, :4] += 1.0                    # all points a step away in four dimensions ...
     points[sample] = rng.random((sample.size, d), dtype=np.float32)    # ... but the sampled ones
     queries[::2, :4] += 1.0                 # every other query sits among the far points
-    gd, gl = _fused(bk, dev, points, queries, k, arithmetic=arithmetic)
-    _check(oracle, points, queries, k, gd, gl)
+    gd, gl = _fused(bk, dev, points, queries, k, arithmetic=arithmetic, workspace=workspace)
+    _check(oracle, points, queries, k, gd, gl, bar_dim=8)   # norms twice those of uniform points
     assert not np.isnan(gd).any()
 
 
