@@ -31,7 +31,9 @@ which did not do its work cannot produce a figure.
                matrix), then bits top-k (k = 64) on it
   fused        bits-fused, 1,048,576 points x 65,536 queries, d in {8,16,32} x k in {4,16,32}, priced
                against the fp32 MFMA peak with 2*q*n*d flops; `fused` itself is the d = 32, k = 32
-               case (queries/s), `fused.grid` the nine cases
+               case (queries/s), `fused.grid` the nine cases; `fused.long_lists` the same shape at
+               k in {64,128,256}; `fused.few_queries` the reference's own fused shape (8192 queries,
+               131,072 points, d = 8) through the entry point that cuts the points into ranges
   cpu          `cpu_baseline`: the CPU restatement of the reference's parallel top-k (reference
                src/topk/parallel_knn.cpp:30-65) on the host cores and of its serial top-k
                (src/topk/serial_knn.cpp:35-43) on one core, on a 1024 x 65,536 matrix
@@ -294,10 +296,14 @@ def leg_gemm(bitsknn, torch, timer, oracle, dev, steps, check, q=4096, n=1 << 20
     return result
 
 
-def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=65536, n=1 << 20):
-    """Config 5: bits-fused at d x k; the d = 32, k = 32 case also with bf16x3 products."""
+def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=65536, n=1 << 20, long_ks=(),
+              workspace=False):
+    """Config 5: bits-fused at d x k; the d = 32, k = 32 case also with bf16x3 products.  long_ks:
+    list lengths beyond the configuration's, reported apart (`long_lists`).  workspace: through the
+    entry point that may cut the points into ranges (few queries)."""
     import numpy as np
     grid = []
+    long_lists = []
     headline = None
     sample = sample_indices(q, 64)
     for d in dims:
@@ -306,11 +312,14 @@ def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=6553
         points = torch.rand((d, n), device=dev, generator=gen)
         queries = torch.rand((d, q), device=dev, generator=gen)
         part = None
-        for k in ks:
+        for k in tuple(ks) + tuple(long_ks):
             out_d = torch.full((q, k), -1.0, dtype=torch.float32, device=dev)
             out_l = torch.empty((q, k), dtype=torch.int32, device=dev)
-            _, seconds = timer.run(lambda: bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l),
-                                   steps, 1)
+            space = None
+            if workspace:
+                space = torch.empty(max(1, bitsknn.fused_workspace_bytes(q, n, k)), dtype=torch.uint8, device=dev)
+            _, seconds = timer.run(lambda: bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l,
+                                                                 workspace=space), steps, 1)
             tflops = 2.0 * q * n * d / seconds / 1e12
             entry = {"d": d, "k": k, "ms": seconds * 1e3, "queries_per_s": q / seconds,
                      "pairs_per_s": q * n / seconds, "frac": tflops / MFMA_F32_PEAK_TFLOPS}
@@ -324,8 +333,8 @@ def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=6553
                                                out_l[sample].cpu().numpy(), k)
                 entry["verified"] = bool(ok)
                 entry["verification"] = detail
-            grid.append(entry)
-            if d == 32 and k == 32:
+            (grid if k in ks else long_lists).append(entry)
+            if d == 32 and k == 32 and not workspace:
                 headline = {"workload": f"bits-fused, {n} points x {q} queries, d={d}, k={k}, fp32 uniform[0,1)",
                             "arithmetic": "fp32 matrix instructions",
                             "queries_per_s": q / seconds, "ms": seconds * 1e3, "pairs_per_s": q * n / seconds,
@@ -349,8 +358,10 @@ def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=6553
                                                    out_d[sample].cpu().numpy(), out_l[sample].cpu().numpy(), k)
                     headline["bf16x3"]["verified"] = bool(ok)
         del points, queries
-    result = headline if headline is not None else {"workload": "bits-fused, restricted grid"}
+    result = headline if headline is not None else {"workload": f"bits-fused, {n} points x {q} queries"}
     result["grid"] = grid
+    if long_lists:
+        result["long_lists"] = long_lists
     return result
 
 
@@ -477,7 +488,17 @@ def main():
     if "fused" in legs:
         dims = (args.fused_d,) if args.fused_d else (8, 16, 32)
         ks = (args.fused_k,) if args.fused_k else (4, 16, 32)
-        result["fused"] = leg_fused(bitsknn, torch, timer, oracle, dev, max(2, args.steps // 10), check, dims, ks)
+        whole = not args.fused_d and not args.fused_k
+        result["fused"] = leg_fused(bitsknn, torch, timer, oracle, dev, max(2, args.steps // 10), check, dims, ks,
+                                    long_ks=(64, 128, 256) if whole else ())
+        if whole:
+            # the reference's own fused shape with few queries (its plots: 8192 queries, 2^17 points):
+            # the entry point with a workspace, which cuts the points into ranges
+            few = leg_fused(bitsknn, torch, timer, oracle, dev, max(2, args.steps // 4), check, (8,), (32,),
+                            q=8192, n=1 << 17, long_ks=(64, 256), workspace=True)
+            result["fused"]["few_queries"] = {"workload": few["workload"] + ", points cut into ranges (workspace)",
+                                              "cases": few["grid"] + few["long_lists"]}
+
         torch.cuda.empty_cache()
     if "cpu" in legs:
         result["cpu_baseline"] = leg_cpu(1024, 65536, 32)
