@@ -148,6 +148,11 @@ int bitsknn_dist_f32(int op, int dim, size_t q, size_t n, const float* queries_d
  *                             compatibility only: they describe a register tiling for the fp32
  *                             vector unit and do not change the matrix-core kernel, so a sweep
  *                             over them measures the same kernel every time
+ * A call enqueues one to three kernels on `stream` (long lists over many points are preceded by a
+ * pass over a sample of the points, which gives every query a first radius, and followed by one
+ * that repeats the queries whose first radius proved too low); until the last of them has run,
+ * out_dist and out_label hold intermediate lists.  A NaN or infinite distance is never reported
+ * as a neighbour before a finite one.
  */
 int bitsknn_fused_l2_topk_f32(const float* queries_dim_major, const float* points_dim_major,
                               int dim, int32_t q, int32_t n, float* out_dist, int32_t* out_label,
@@ -159,7 +164,9 @@ int bitsknn_fused_l2_topk_f32(const float* queries_dim_major, const float* point
  * still the fused kernel: no distance is written to memory.  When there are too few queries to
  * fill the GPU with one workgroup per 128 queries, the points are cut into ranges that are
  * searched by separate workgroups; their partial lists (k pairs per query and range) go to the
- * workspace and one bits pass (explicit labels) selects the final k.
+ * workspace and a bits pass (explicit labels) selects the final k.  Same distances bit for bit,
+ * except for k >= 128 in up to 16 dimensions, where the kernel over ranges adds the norm of a
+ * point last instead of first (last-bit differences).
  *
  * No counterpart in the reference, whose fused kernel always runs one thread block per query tile
  * (src/topk/singlepass/fused_cache_knn.cu:60-69); the host wrapper that owns the device memory
