@@ -193,14 +193,16 @@ def test_parameter_validation(bk, dev):
             bk.fused_l2_topk(*args)
 
 
-def test_point_matrix_of_2_gib_takes_the_plain_loads(bk, dev):
+@pytest.mark.parametrize("k", [16, 128])
+def test_point_matrix_of_2_gib_takes_the_plain_loads(bk, dev, k):
     """dim * n * 4 bytes >= 2 GiB: the staging falls back from buffer loads (32-bit offsets) to
-    ordinary loads.  Checked against the GEMM distance kernel + bits top-k on the same inputs:
-    k-th distance within 1e-5 of the scale of the cancelling terms, recall >= 0.999."""
+    ordinary loads (k = 128: also in the launch over a sample of the points).  Checked against the
+    GEMM distance kernel + bits top-k on the same inputs: k-th distance within 1e-5 of the scale of
+    the cancelling terms, recall >= 0.999."""
     import torch
     gen = torch.Generator(device=dev)
     gen.manual_seed(9)
-    q, n, d, k = 128, 2_200_000, 256, 16
+    q, n, d = 128, 2_200_000, 256
     assert d * n * 4 >= 1 << 31
     queries = torch.rand((d, q), device=dev, generator=gen)
     points = torch.rand((d, n), device=dev, generator=gen)
