@@ -74,10 +74,8 @@ __device__ __forceinline__ float min3(float a, float b, float c)
 // for them (up to 16 dimensions, with smaller stages): half as many merges.  That pays where the
 // lists hardly converge, i.e. with few queries whose points are cut into ranges (q = 8192,
 // n = 2^17, d = 8: 4.4 -> 2.7 ms at k = 256 and 1.7 -> 1.3 ms at k = 128 before the first radii from
-// a sample, 2.19 -> 1.65 and 1.18 -> 1.10 ms with them; at k = 64 the smaller stages cost more than
-// the merges save).  With one range of points the smaller stages cost more than the merges (65536
-// queries x 2^20 points, d = 16, k = 128: 33.9 ms with 64 slots, 24.8 ms with 32), so WIDE_OK is set
-// for launches over ranges only.
+// a sample; at k = 64 the smaller stages cost more than the merges save).  WIDE_OK is set for
+// launches over ranges only (see launch_fused).
 template <int DP, bool SPLIT, int K, bool WIDE_OK = false>
 struct fused_geometry
 {
@@ -89,7 +87,12 @@ struct fused_geometry
     static constexpr int PT = SPLIT  ? (DK <= 16 ? 128 : (DK <= 32 ? 64 : 32))
                               : WIDE ? (DP <= 8 ? 128 : 64)
                                      : (DP <= 16 ? 256 : (DP <= 32 ? 128 : (DP <= 64 ? 64 : 32)));
-    static constexpr int TPP = FQ_THREADS / PT; // threads per point when staging
+    // threads per point when staging.  The small stages of the 64-slot geometry are staged by their
+    // first PT threads, a whole point each, so that the norm of a point is one row and can be the
+    // initial accumulator as in the 32-slot geometry (same terms in the same order: both
+    // geometries give the same bits).
+    static constexpr int TPP = WIDE ? 1 : FQ_THREADS / PT;
+    static constexpr int STAGERS = SPLIT ? FQ_THREADS : TPP * PT; // threads that stage
     // point rows (zero beyond dim), then one row per staging thread of a point with its share of
     // ||p||^2 (at least two rows, so that the row count is even)
     static constexpr int NORM_ROWS = TPP > 2 ? TPP : 2;
@@ -466,6 +469,13 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                           : OUTSIDE;
     }
     auto fetch = [&](int base) {
+        if constexpr (G::STAGERS < FQ_THREADS)
+        {
+            if (t >= G::STAGERS) // (whole waves)
+            {
+                return;
+            }
+        }
         // first point of the stage in the matrix (a sample visits every sample_scale-th stage)
         const int at = base * a.sample_scale + a.sample_offset;
         if (small_points)
@@ -509,6 +519,13 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         }
     };
     auto deposit = [&](float* stage, int base) {
+        if constexpr (G::STAGERS < FQ_THREADS)
+        {
+            if (t >= G::STAGERS)
+            {
+                return;
+            }
+        }
         float share = 0.0F;
         if constexpr (SPLIT)
         {
@@ -859,7 +876,11 @@ hipError_t launch_fused_as(const fused_args& a, hipStream_t stream)
     return hipGetLastError();
 }
 
-// launches over ranges of points take the 64-slot buffers where the geometry has them
+// Launches over ranges of points take the 64-slot buffers where the geometry has them.  With one
+// range of points the smaller stages cost more than the merges they save (65536 queries x 2^20
+// points, k = 128: d = 8 19.5 ms with 64 slots, 17.3 ms with 32; d = 16 32.2 / 24.9 ms); over ranges
+// the lists hardly converge and the merges weigh more (8192 queries x 2^17 points, d = 8, k = 256:
+// 2.19 ms with 32 slots, 1.60 ms with 64).
 template <int K, int DP, bool SPLIT>
 hipError_t launch_fused(const fused_args& a, hipStream_t stream)
 {

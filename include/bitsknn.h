@@ -164,9 +164,7 @@ int bitsknn_fused_l2_topk_f32(const float* queries_dim_major, const float* point
  * still the fused kernel: no distance is written to memory.  When there are too few queries to
  * fill the GPU with one workgroup per 128 queries, the points are cut into ranges that are
  * searched by separate workgroups; their partial lists (k pairs per query and range) go to the
- * workspace and a bits pass (explicit labels) selects the final k.  Same distances bit for bit,
- * except for k >= 128 in up to 16 dimensions, where the kernel over ranges adds the norm of a
- * point last instead of first (last-bit differences).
+ * workspace and a bits pass (explicit labels) selects the final k.  Same distances bit for bit.
  *
  * No counterpart in the reference, whose fused kernel always runs one thread block per query tile
  * (src/topk/singlepass/fused_cache_knn.cu:60-69); the host wrapper that owns the device memory
