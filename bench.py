@@ -23,8 +23,9 @@ which did not do its work cannot produce a figure.
                (the read rate this machine reaches) and 1 GiB device copies (known traffic for
                scaling byte counters read under a profiler)
   sweep        the 4 GiB matrix at k in {16,32,128,512,2048} x block size {128,256,512} with 2048
-               values of a row in flight per iteration (16 / 8 / 4 values per thread), plus the
-               configuration the shipped optima file names for each k
+               values of a row in flight per iteration (16 / 8 / 4 values per thread) and with the
+               larger batches 256 and 512 threads can take, plus the configuration the shipped
+               optima file names for each k
   hard         16,384 x 65,536 rows sorted ascending / descending / drawn from 256 values, k = 32, 256,
                with one fixed configuration and with the one the optima file names
   gemm         ||p||^2 - 2 q.p on fp32 MFMA for 1,048,576 points x 4,096 queries, d = 64 (a 16 GiB
@@ -56,8 +57,9 @@ MFMA_F32_PEAK_TFLOPS = 157.3  # dense fp32 matrix peak
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 matrix peak
 LEGS = ("headline", "calibration", "sweep", "hard", "gemm", "fused", "cpu")
 # values per thread in the block-size sweep: the same 2048 values of a row in flight per iteration
-# whatever the workgroup size (fewer waves per row need more loads each)
-SWEEP_ITEMS = {128: 16, 256: 8, 512: 4}
+# whatever the workgroup size (fewer waves per row need more loads each), and the larger batches
+# that long lists need where few rows fit a compute unit
+SWEEP_ITEMS = {128: (16,), 256: (8, 16), 512: (4, 8, 16)}
 REL = 1e-5
 MIN_RECALL = 0.999
 
@@ -188,7 +190,8 @@ def leg_sweep(bitsknn, torch, timer, oracle, matrix, steps, check):
         out_d = torch.empty((rows, k), dtype=torch.float32, device=matrix.device)
         out_l = torch.empty((rows, k), dtype=torch.int32, device=matrix.device)
         tuned_block, _, tuned_batch, _, _ = tuning.config_algorithm("bits", rows, k)
-        cases = [(block, SWEEP_ITEMS[block], False) for block in (128, 256, 512) if k // block <= 16]
+        cases = [(block, items, False) for block in (128, 256, 512) if k // block <= 16
+                 for items in SWEEP_ITEMS[block]]
         cases.append((tuned_block, tuned_batch, True))
         for block, items, tuned in cases:
             out_d.fill_(-1.0)
