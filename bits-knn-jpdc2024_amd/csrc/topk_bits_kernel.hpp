@@ -22,10 +22,11 @@
 //    before the current one is filtered;
 //  * long rows start from a radius taken from a sample of both row ends instead of from +inf,
 //    which saves the first merges (they only halve the radius each);
-//  * lists of 1024 entries and more start from an estimate of the k-th smallest value of the
-//    row, taken from a sample spread over the row, and repeat the row from +inf in the rare case
-//    that fewer than k values lie below the estimate (a third of the values pass the filter then,
-//    and less than half the merges are needed: 0.70 -> 0.79 of the HBM peak at k = 2048).
+//  * long lists also take an estimate of the k-th smallest value of the row from a sample spread
+//    over the row, and repeat the row without it in the rare case that fewer than k values lie
+//    below the estimate (a third of the values pass the filter then, and less than half the merges
+//    are needed: 0.70 -> 0.79 of the HBM peak at k = 2048, 0.74-0.75 -> 0.83 at k = 512 with 128 and
+//    256 threads per row).
 // Because waves drift apart, the filter compares full keys when a value equals the radius, so
 // that "equal values by lower label" holds no matter which wave saw which value first.
 
@@ -130,10 +131,13 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     // and 16-byte pieces per thread and end of the row (4 values looked at per value kept).
     constexpr int SAMPLE_KEEP = IPT <= 1 ? 2 : (IPT == 2 ? 4 : 8);
     constexpr u32 SAMPLE_PAIRS = SAMPLE_KEEP;
-    // Lists of 1024 entries and more start from an estimate of the k-th smallest value instead
-    // (see below): a sample of up to EST_PIECES 16-byte pieces per thread, 2^14 values, spread
-    // over the row, of which every thread keeps its EST_KEEP smallest.
-    constexpr bool ESTIMATE = NL >= 1024;
+    // Lists of 1024 entries and more, and lists of 256 and more with at least two entries per
+    // thread, also take an estimate of the k-th smallest value (see below): a sample of up to
+    // EST_PIECES 16-byte pieces per thread, 2^14 values, spread over the row, of which every thread
+    // keeps its EST_KEEP smallest.  (With one entry per thread -- 512 threads up to k = 512, 256
+    // up to k = 256 -- the merges are cheap and the estimate costs more than it saves: 0.83 ->
+    // 0.77-0.82 of the HBM peak at k = 512.)
+    constexpr bool ESTIMATE = NL >= 1024 || (NL >= 256 && IPT >= 2);
     constexpr u32 EST_PIECES = 4096 / BS;
     constexpr int EST_KEEP = 8;
 
@@ -183,7 +187,9 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     // radius until the list itself has a smaller one.  This replaces the first merges of a row,
     // which each only halve the radius and which all rows of a launch do at the same time.
     //
-    // Long lists (ESTIMATE) on rows of at least 256 * BS values start lower, from an estimate.
+    // Lists of two and more entries per thread (ESTIMATE) on rows of at least 256 * BS values also
+    // take an estimate, which counts where it lies below that bound (on uniform rows it does by far;
+    // on sorted rows, whose ends hold the smallest values, the guaranteed bound is the lower one).
     // The sample is spread evenly over the row (at most a 64th of it) and the radius is its
     // value of rank e + 5 sqrt(e) + 2, where e = k * sample size / n values of the sample are
     // expected among the k smallest of the row: fewer than k values of the row lie below it with
@@ -191,11 +197,11 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     // the row (sorted rows included).  At k = 2048 on rows of 2^20 uniform values 4 thousand values
     // pass the filter then instead of 12 thousand, and 3 merges are needed instead of 7.  The
     // estimate is not trusted: if the k-th key of the list has not got below it by the end of the
-    // row, the pass is repeated without it.
+    // row, the pass is repeated from the guaranteed bound.
     bool estimated = false;
+    u32 estimate = 0xFFFFFFFFU; // (the same in every wave)
     {
         u32 wave_bound = 0xFFFFFFFFU;
-        bool have = false;
         if constexpr (ESTIMATE)
         {
             const u32 fit = n / (256U * BS);
@@ -268,16 +274,19 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
                 {
                     pick = (rank - 1) % W == static_cast<u32>(i) ? static_cast<u32>(all[i] >> 32U) : pick;
                 }
-                wave_bound = static_cast<u32>(__builtin_amdgcn_readlane(
+                estimate = static_cast<u32>(__builtin_amdgcn_readlane(
                     static_cast<int>(pick), static_cast<int>((rank - 1) / W)));
-                estimated = wave_bound < float_key(__builtin_inff());
-                have = true;
             }
         }
+        // (the guaranteed bound is taken as well: on sorted rows, whose ends hold the smallest
+        // values, it lies far below any estimate from a spread sample; the lower of the two counts)
         const u32 c = (a.k + W - 1) / W;
         const u32 fit = n / (128U * BS);
-        const u32 pairs = fit < SAMPLE_PAIRS ? fit : SAMPLE_PAIRS;
-        if (!have && c <= WAVE * SAMPLE_KEEP && pairs > 0)
+        // (next to an estimate one pair of pieces is enough: it is there for the sorted rows; lists
+        // of 1024 entries and more do without it, where it costs 1-1.5 % on uniform rows)
+        const u32 wanted = estimate != 0xFFFFFFFFU ? (NL >= 1024 ? 0U : 1U) : SAMPLE_PAIRS;
+        const u32 pairs = fit < wanted ? fit : wanted;
+        if (c <= WAVE * SAMPLE_KEEP && pairs > 0)
         {
             const u32 back = VEC ? (n - pairs * 4 * BS) & ~3U : n - pairs * 4 * BS;
             float lo[SAMPLE_KEEP]; // ascending
@@ -355,7 +364,6 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
         u64 radius_key = PAD_KEY;
         u64 first_key = PAD_KEY; // the radius the pass starts from
         bool sampled = false;
-        if (!again)
         {
             u32 bound = 0;
 #pragma unroll
@@ -365,6 +373,9 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
             }
             // values up to the bound pass: the radius is the next key after it with the lowest label
             bound = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(bound)));
+            // (the estimate counts in the first turn only, and only where it is the lower one)
+            estimated = !again && estimate < bound;
+            bound = estimated ? estimate : bound;
             if (bound < float_key(__builtin_inff()))
             {
                 radius_key = static_cast<u64>(bound + 1) << 32U;
@@ -694,7 +705,7 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
             // Everything the filter dropped was not below the radius of that moment, and no radius
             // was above the first one.  If the k-th key of the list got below the first radius, the
             // dropped values all lie above the list; if not, fewer than k values of the row lie
-            // below the estimate, and the row is done again from +inf.
+            // below the estimate, and the row is done again without it.
             const u32 high = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(radius_key >> 32U)));
             const u32 low = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<int>(radius_key)));
             if (estimated && !(((static_cast<u64>(high) << 32U) | low) < first_key))
