@@ -139,8 +139,8 @@ def test_rows_long_enough_for_the_sampled_radius(bk, dev, oracle):
 
 
 def _estimate_sample_columns(cols, block):
-    """Columns of the evenly spread sample that lists of 1024 entries and more estimate their
-    first radius from (rows of at least 256 x block size values)."""
+    """Columns of the evenly spread sample that long lists estimate their first radius from (rows
+    of at least 256 x block size values)."""
     pieces = min(4096 // block, cols // (256 * block))
     segment = (cols // pieces) & ~3
     offset = (segment // 2 - 2 * block) & ~3
@@ -150,11 +150,12 @@ def _estimate_sample_columns(cols, block):
 
 @pytest.mark.parametrize("block,k,batch", [(128, 1024, 8), (128, 2048, 16), (256, 600, 8), (256, 2048, 8),
                                            (256, 2048, 12), (512, 513, 4), (512, 1024, 8), (512, 2047, 8),
-                                           (512, 2048, 16)])
+                                           (512, 2048, 16), (128, 200, 16), (128, 256, 8), (128, 500, 16),
+                                           (256, 300, 8), (256, 512, 16)])
 def test_rows_long_enough_for_the_estimated_radius(bk, dev, oracle, block, k, batch):
-    """Lists of 1024 entries and more on long rows start from an estimate of the k-th smallest
-    value and repeat the row when the estimate proves too low; the result must not depend on
-    either.  Rows where the estimate holds, rows where it cannot hold (the sampled columns hold
+    """Long lists (two and more entries per thread from 256 entries on, all from 1024 on) on long
+    rows start from an estimate of the k-th smallest value and repeat the row when the estimate
+    proves too low; the result must not depend on either.  Rows where the estimate holds, rows where it cannot hold (the sampled columns hold
     the only small values, fewer than k of them), ties at the estimate, sorted rows, rows with
     few finite values."""
     rng = np.random.default_rng(block + k)
