@@ -38,6 +38,12 @@ DEFAULT_OPTIMA = os.path.join(os.path.dirname(os.path.abspath(__file__)), "optim
 QUERY_COUNTS = (64, 256, 512, 1024, 2048, 4096, 8192)
 K_VALUES = (2, 4, 8, 16, 32, 64, 128, 256, 512, 1024, 2048)
 BLOCK_SIZES = (128, 256, 512)
+# Many short rows (the shape of the sorted / tie-heavy benchmark rows) want other launch parameters
+# than the long rows of the grid above: a row of 65,536 values is over after a few iterations of 512
+# threads.  The lookup is keyed by the query count alone, so these rows serve requests for 16,384
+# queries and more.
+SHORT_ROWS_QUERY_COUNT = 16384
+SHORT_ROWS_POINT_COUNT = 65536
 # values per thread and iteration: the kernels issue 16-byte loads, so 1..4, 5..8, 9..12 and 13..16
 # are one kernel each; the sweep times the distinct ones
 BATCH_SIZES = (4, 8, 12, 16)
@@ -313,6 +319,8 @@ def main(argv=None):
     rows = []
     if args.only in (None, "bits"):
         rows += list(sweep(repeats=args.repeats, progress=progress))
+        rows += list(sweep(repeats=args.repeats, point_count=SHORT_ROWS_POINT_COUNT,
+                           query_counts=(SHORT_ROWS_QUERY_COUNT,), progress=progress))
     if args.only in (None, "bits-sq"):
         rows += list(sweep_bits_sq(repeats=args.repeats, progress=progress))
     if args.only in (None, "fused-cache"):

@@ -170,6 +170,12 @@ def test_shipped_optima_file():
         for q in tuning.QUERY_COUNTS:
             for k in tuning.K_VALUES:
                 assert (name, q, k) in seen
+    # and the rows for many short rows, measured on their own shape
+    for name, _ in tuning.ALGORITHMS:
+        for k in tuning.K_VALUES:
+            short = [r for r in rows if r["algorithm"] == name and int(r["k"]) == k and
+                     int(r["query_count"]) == tuning.SHORT_ROWS_QUERY_COUNT]
+            assert len(short) == 1 and int(short[0]["point_count"]) == tuning.SHORT_ROWS_POINT_COUNT
     assert sum(r["algorithm"] == "partial-bitonic-regs" for r in rows) == 28
     for r in rows:
         assert float(r["time"]) > 0
