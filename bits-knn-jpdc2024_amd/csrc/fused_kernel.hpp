@@ -9,7 +9,8 @@
 //
 //  * A workgroup of 4 waves owns 128 queries (32 per wave) and walks over its range of points in
 //    stages of PT points, two stages in LDS (one being multiplied, one being filled; one barrier
-//    per stage).  A stage is the MFMA A operand: rows 0..d-1 hold the points, the following rows
+//    per stage) or, for short lists in up to 8 dimensions, a ring of four stages without barriers.
+//    A stage is the MFMA A operand: rows 0..d-1 hold the points, the following rows
 //    hold the staging threads' shares of ||p||^2, so that v_mfma_f32_32x32x2_f32 against the query
 //    fragment (-2q_0..-2q_{d-1}, 1, 1) yields ||p||^2 - 2 q.p directly, the dot product accumulated
 //    first and the norm added last.  For d <= 16 the norm is the initial accumulator instead.
@@ -101,13 +102,19 @@ struct fused_geometry
     static constexpr int VPT = SPLIT ? 8 : DP / TPP; // values a thread carries from global memory to LDS
     static constexpr int MT = PT / 32;        // MFMA row tiles per stage
     static constexpr int STAGE_FLOATS = SPLIT ? 3 * KS * PT * 4 + PT : ROWS * PT;
+    // Stages in LDS: two, with a barrier per stage (one being multiplied, one being filled), or a
+    // ring of four without barriers where they fit next to the buffers of two workgroups per compute
+    // unit (up to 8 dimensions) and the waves do not merge together (lists of up to 32 entries): a
+    // wave that appends or merges then holds up the others only once it is a whole stage behind.
+    static constexpr bool RING = !SPLIT && !WIDE && K <= FQ_CAP && DP <= 8;
+    static constexpr int NB = RING ? 4 : 2;
     static_assert(!SPLIT || (DP <= 64 && TPP == KS), "one staging thread per point and cell");
     static constexpr size_t lds_bytes()
     {
-        // two stages (one being multiplied, one being filled), the query buffers, exchange slots
-        return 2 * static_cast<size_t>(STAGE_FLOATS) * sizeof(float) +
+        // the stages, the query buffers, exchange slots, merge flags and stage counters
+        return NB * static_cast<size_t>(STAGE_FLOATS) * sizeof(float) +
                static_cast<size_t>(FQ_WAVES) * FQ_QW * CAP * sizeof(u64) +
-               static_cast<size_t>(FQ_WAVES) * WAVE * sizeof(float) + 4 * sizeof(int);
+               static_cast<size_t>(FQ_WAVES) * WAVE * sizeof(float) + 8 * sizeof(int);
     }
 };
 
@@ -144,10 +151,13 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 
     extern __shared__ float lds[];
     constexpr int STAGE_FLOATS = G::STAGE_FLOATS;
-    float* const stages = lds;                                                    // [2][STAGE_FLOATS]
-    u64* const buffers = reinterpret_cast<u64*>(lds + 2 * STAGE_FLOATS);          // [waves][32][CAP]
+    float* const stages = lds;                                                    // [NB][STAGE_FLOATS]
+    constexpr bool RING = G::RING;
+    constexpr int NB = G::NB;
+    u64* const buffers = reinterpret_cast<u64*>(lds + NB * STAGE_FLOATS);          // [waves][32][CAP]
     float* const xchg = reinterpret_cast<float*>(buffers + FQ_WAVES * FQ_QW * CAP);  // [waves][64]
     int* const merge_wanted = reinterpret_cast<int*>(xchg + FQ_WAVES * WAVE);           // [3]
+    int* const ready = merge_wanted + 4;   // [NB] waves that have written their part, per ring slot
 
     const int dim = a.dim;
     // this workgroup's range of points
@@ -206,12 +216,12 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         }
     }
 
-    // rows that never change in either stage: padding dimensions, unused norm rows
-    for (int i = t; i < 2 * STAGE_FLOATS; i += FQ_THREADS)
+    // rows that never change in any stage: padding dimensions, unused norm rows
+    for (int i = t; i < NB * STAGE_FLOATS; i += FQ_THREADS)
     {
         lds[i] = 0.0F;
     }
-    if (t < 3)
+    if (t < 8)
     {
         merge_wanted[t] = 0;
     }
@@ -407,15 +417,25 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         }
         int slot = fill + (half != 0 ? other : 0);
         const int first_point = tile_base + 4 * half;
+        // Most values of a tile that has candidates fail in every lane.  They are skipped four at a
+        // time, and the writes sit out of line: a branch that is not taken costs a wave far less
+        // than one that is (16 taken branches per tile: 2-4 % of the kernel time).
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
+        for (int g = 0; g < 4; ++g)
         {
-            if (pass[r] != 0)
+            if (__builtin_expect((pass[4 * g] | pass[4 * g + 1] | pass[4 * g + 2] | pass[4 * g + 3]) != 0, 0))
             {
-                if (__builtin_amdgcn_inverse_ballot_w64(pass[r]))
+#pragma unroll
+                for (int r = 4 * g; r < 4 * g + 4; ++r)
                 {
-                    wbuf[ql * CAP + slot] = make_key(acc[r], first_point + 8 * (r / 4) + (r % 4));
-                    ++slot;
+                    if (__builtin_expect(pass[r] != 0, 0))
+                    {
+                        if (__builtin_amdgcn_inverse_ballot_w64(pass[r]))
+                        {
+                            wbuf[ql * CAP + slot] = make_key(acc[r], first_point + 8 * (r / 4) + (r % 4));
+                            ++slot;
+                        }
+                    }
                 }
             }
         }
@@ -797,43 +817,112 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             merge_event();
         }
     };
-    fetch(n_begin);
-    // the query fragment and the first stage have arrived (nothing else is in flight yet)
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    deposit(stages, n_begin);
-    if (n_begin + PT < n)
+    if constexpr (!RING)
     {
-        fetch(n_begin + PT);
-    }
-    __syncthreads();
-    int parity = 0;
-    for (int base = n_begin; base < n; base += PT)
-    {
-        merged = false;
-        multiply(stages + parity * STAGE_FLOATS, base);
-        parity ^= 1;
-        if (base + PT < n)
+        fetch(n_begin);
+        // the query fragment and the first stage have arrived (nothing else is in flight yet)
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        deposit(stages, n_begin);
+        if (n_begin + PT < n)
         {
-            deposit(stages + parity * STAGE_FLOATS, base + PT);
+            fetch(n_begin + PT);
+        }
+        __syncthreads();
+        int parity = 0;
+        for (int base = n_begin; base < n; base += PT)
+        {
+            merged = false;
+            multiply(stages + parity * STAGE_FLOATS, base);
+            parity ^= 1;
+            if (base + PT < n)
+            {
+                deposit(stages + parity * STAGE_FLOATS, base + PT);
+                if (base + 2 * PT < n)
+                {
+                    fetch(base + 2 * PT);
+                }
+            }
+            if constexpr (JOIN_MERGES)
+            {
+                merge_if_wanted();
+                __syncthreads();
+                merge_if_wanted();
+                if (t == 0)
+                {
+                    merge_wanted[(stage_slot + 2) % 3] = 0;
+                }
+                stage_slot = stage_slot == 2 ? 0 : stage_slot + 1;
+            }
+            else
+            {
+                __syncthreads();
+            }
+        }
+    }
+    else
+    {
+        // Ring of four stages, filled two stages ahead of the one being multiplied: while stage i is
+        // multiplied, stage i + 1 is complete or about to be, stage i + 2 is written and stage i + 3
+        // is on its way from memory.  A wave counts itself in at ready[slot] once its part of a stage
+        // is written (LDS executes the instructions of a wave in order: the count follows the
+        // writes), and a stage is complete when all waves have counted in: FQ_WAVES more per use of
+        // the slot.  There is no barrier: a wave starts stage i as soon as every wave has finished
+        // stage i - 2, so one that appends or merges holds up the others only when it falls a whole
+        // stage behind.  Writing stage i + 2 over stage i - 2 is safe once stage i is complete:
+        // every wave wrote its part of stage i after it had multiplied stage i - 2.  Stage i itself is
+        // overwritten by stage i + 4, which a wave writes after it has seen stage i + 2 complete,
+        // i.e. after every wave is done with stage i.
+        static_assert(NB == 4, "the ring slot is the stage index modulo 4");
+        auto count_in = [&](int index) __attribute__((always_inline)) {
+            if (lane == 0)
+            {
+                __hip_atomic_fetch_add(ready + (index & (NB - 1)), 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        };
+        auto wait_for = [&](int index) __attribute__((always_inline)) {
+            const int complete = FQ_WAVES * (index / NB + 1);
+            // Every wave counts in for every stage whatever it finds in the tiles, so the count is
+            // reached; the bound on the polls only makes sure that a wave leaves this loop whatever
+            // happens.
+            for (int polls = 0; polls < (1 << 22); ++polls)
+            {
+                if (__hip_atomic_load(ready + (index & (NB - 1)), __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) >= complete)
+                {
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+        };
+        fetch(n_begin);
+        // the query fragment and the first stage have arrived (nothing else is in flight yet)
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        deposit(stages, n_begin);
+        count_in(0);
+        if (n_begin + PT < n)
+        {
+            fetch(n_begin + PT);
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            deposit(stages + STAGE_FLOATS, n_begin + PT);
+            count_in(1);
+            if (n_begin + 2 * PT < n)
+            {
+                fetch(n_begin + 2 * PT);
+            }
+        }
+        int index = 0;
+        for (int base = n_begin; base < n; base += PT, ++index)
+        {
+            wait_for(index);
+            multiply(stages + (index & (NB - 1)) * STAGE_FLOATS, base);
             if (base + 2 * PT < n)
             {
-                fetch(base + 2 * PT);
+                deposit(stages + ((index + 2) & (NB - 1)) * STAGE_FLOATS, base + 2 * PT);
+                count_in(index + 2);
+                if (base + 3 * PT < n)
+                {
+                    fetch(base + 3 * PT);
+                }
             }
-        }
-        if constexpr (JOIN_MERGES)
-        {
-            merge_if_wanted();
-            __syncthreads();
-            merge_if_wanted();
-            if (t == 0)
-            {
-                merge_wanted[(stage_slot + 2) % 3] = 0;
-            }
-            stage_slot = stage_slot == 2 ? 0 : stage_slot + 1;
-        }
-        else
-        {
-            __syncthreads();
         }
     }
 
