@@ -50,7 +50,7 @@ BATCH_SIZES = (4, 8, 12, 16)
 ALGORITHMS = (("bits", False), ("bits-prefetch", True))
 # bits-sq: parts a row is cut into, for query counts that leave compute units without a row
 SQ_QUERY_COUNTS = (64, 256)
-SQ_DEGREES = (2, 4, 8, 16)
+SQ_DEGREES = (2, 4, 8, 16, 32)
 # fused-cache: (queries, points) shapes of the reference's fused runs (scripts/run-fused.sh) that
 # bound the lookup's range, dimensions and list lengths
 FUSED_SHAPES = ((1024, 1 << 20), (8192, 1 << 17))
