@@ -417,18 +417,20 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         }
         int slot = fill + (half != 0 ? other : 0);
         const int first_point = tile_base + 4 * half;
-        // Most values of a tile that has candidates fail in every lane.  They are skipped four at a
-        // time, and the writes sit out of line: a branch that is not taken costs a wave far less
-        // than one that is (16 taken branches per tile: 2-4 % of the kernel time).
+        // Most values of a tile that has candidates fail in every lane: they are skipped four at a
+        // time (a taken branch costs a wave far more than one that is not; 16 of them per tile were
+        // 2-4 % of the kernel time where candidates are rare).  The writes stay in line: moved out
+        // of line they gain another 0.5 % there, but cost 3-7 % where most tiles hold candidates
+        // (lists over ranges of points, which hardly converge).
 #pragma unroll
         for (int g = 0; g < 4; ++g)
         {
-            if (__builtin_expect((pass[4 * g] | pass[4 * g + 1] | pass[4 * g + 2] | pass[4 * g + 3]) != 0, 0))
+            if ((pass[4 * g] | pass[4 * g + 1] | pass[4 * g + 2] | pass[4 * g + 3]) != 0)
             {
 #pragma unroll
                 for (int r = 4 * g; r < 4 * g + 4; ++r)
                 {
-                    if (__builtin_expect(pass[r] != 0, 0))
+                    if (pass[r] != 0)
                     {
                         if (__builtin_amdgcn_inverse_ballot_w64(pass[r]))
                         {
