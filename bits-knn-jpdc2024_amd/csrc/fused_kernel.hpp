@@ -9,7 +9,8 @@
 //
 //  * A workgroup of 4 waves owns 128 queries (32 per wave) and walks over its range of points in
 //    stages of PT points, two stages in LDS (one being multiplied, one being filled; one barrier
-//    per stage) or, for short lists in up to 8 dimensions, a ring of four stages without barriers.
+//    per stage) or, for lists of up to 128 entries in up to 8 dimensions, a ring of four stages
+//    without barriers.
 //    A stage is the MFMA A operand: rows 0..d-1 hold the points, the following rows
 //    hold the staging threads' shares of ||p||^2, so that v_mfma_f32_32x32x2_f32 against the query
 //    fragment (-2q_0..-2q_{d-1}, 1, 1) yields ||p||^2 - 2 q.p directly, the dot product accumulated
@@ -104,9 +105,12 @@ struct fused_geometry
     static constexpr int STAGE_FLOATS = SPLIT ? 3 * KS * PT * 4 + PT : ROWS * PT;
     // Stages in LDS: two, with a barrier per stage (one being multiplied, one being filled), or a
     // ring of four without barriers where they fit next to the buffers of two workgroups per compute
-    // unit (up to 8 dimensions) and the waves do not merge together (lists of up to 32 entries): a
-    // wave that appends or merges then holds up the others only once it is a whole stage behind.
-    static constexpr bool RING = !SPLIT && !WIDE && K <= FQ_CAP && DP <= 8;
+    // unit (up to 8 dimensions): a wave that appends or merges then holds up the others only once it
+    // is a whole stage behind.  Lists of 256 entries stay with the barrier: their merges are so long
+    // that the waves of a workgroup do better merging together, which leans on the barrier
+    // (65536 queries x 2^20 points, d = 8: k = 64 14.8 -> 13.9 ms, k = 128 16.4 -> 15.9 ms on the
+    // ring, k = 256 19.9 -> 21.9 ms).
+    static constexpr bool RING = !SPLIT && !WIDE && K <= 128 && DP <= 8;
     static constexpr int NB = RING ? 4 : 2;
     static_assert(!SPLIT || (DP <= 64 && TPP == KS), "one staging thread per point and cell");
     static constexpr size_t lds_bytes()
@@ -147,7 +151,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     // Whether the waves of a workgroup merge together (below): pays for the long merges of long
     // lists (k = 256: 65 -> 52 ms); for k <= 32 the two looks at the flag per stage cost more (1 %
     // each) than the short merges they overlap.
-    constexpr bool JOIN_MERGES = K > CAP;
+    constexpr bool JOIN_MERGES = K > CAP && !G::RING;
 
     extern __shared__ float lds[];
     constexpr int STAGE_FLOATS = G::STAGE_FLOATS;
