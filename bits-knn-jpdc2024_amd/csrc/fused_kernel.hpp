@@ -9,8 +9,8 @@
 //
 //  * A workgroup of 4 waves owns 128 queries (32 per wave) and walks over its range of points in
 //    stages of PT points, two stages in LDS (one being multiplied, one being filled; one barrier
-//    per stage) or, for lists of up to 128 entries in up to 8 dimensions, a ring of four stages
-//    without barriers.
+//    per stage) or, for lists of up to 128 entries in up to 8 dimensions and of up to 32 entries in
+//    16 to 128 dimensions, a ring of three stages without barriers.
 //    A stage is the MFMA A operand: rows 0..d-1 hold the points, the following rows
 //    hold the staging threads' shares of ||p||^2, so that v_mfma_f32_32x32x2_f32 against the query
 //    fragment (-2q_0..-2q_{d-1}, 1, 1) yields ||p||^2 - 2 q.p directly, the dot product accumulated
@@ -78,6 +78,8 @@ __device__ __forceinline__ float min3(float a, float b, float c)
 // n = 2^17, d = 8: 4.4 -> 2.7 ms at k = 256 and 1.7 -> 1.3 ms at k = 128 before the first radii from
 // a sample; at k = 64 the smaller stages cost more than the merges save).  WIDE_OK is set for
 // launches over ranges only (see launch_fused).
+constexpr int RING_MAX_DP = 128; // largest padded dimension that takes the ring of stages
+
 template <int DP, bool SPLIT, int K, bool WIDE_OK = false>
 struct fused_geometry
 {
@@ -97,27 +99,36 @@ struct fused_geometry
     static constexpr int STAGERS = SPLIT ? FQ_THREADS : TPP * PT; // threads that stage
     // point rows (zero beyond dim), then one row per staging thread of a point with its share of
     // ||p||^2 (at least two rows, so that the row count is even)
-    static constexpr int NORM_ROWS = TPP > 2 ? TPP : 2;
+    // (one row where it is read as the initial accumulator and never multiplied)
+    static constexpr int NORM_ROWS = (!SPLIT && TPP == 1 && PT >= 64) ? 1 : (TPP > 2 ? TPP : 2);
     static constexpr int ROWS = DP + NORM_ROWS;
     static constexpr int STEPS = ROWS / 2;    // MFMA steps of 2 rows
     static constexpr int VPT = SPLIT ? 8 : DP / TPP; // values a thread carries from global memory to LDS
     static constexpr int MT = PT / 32;        // MFMA row tiles per stage
     static constexpr int STAGE_FLOATS = SPLIT ? 3 * KS * PT * 4 + PT : ROWS * PT;
     // Stages in LDS: two, with a barrier per stage (one being multiplied, one being filled), or a
-    // ring of four without barriers where they fit next to the buffers of two workgroups per compute
-    // unit (up to 8 dimensions): a wave that appends or merges then holds up the others only once it
-    // is a whole stage behind.  Lists of 256 entries stay with the barrier: their merges are so long
-    // that the waves of a workgroup do better merging together, which leans on the barrier
-    // (65536 queries x 2^20 points, d = 8: k = 64 14.8 -> 13.9 ms, k = 128 16.4 -> 15.9 ms on the
-    // ring, k = 256 19.9 -> 21.9 ms).
-    static constexpr bool RING = !SPLIT && !WIDE && K <= 128 && DP <= 8;
-    static constexpr int NB = RING ? 4 : 2;
+    // ring of three without barriers, in which a wave that appends or merges holds up the others
+    // only once it is a whole stage behind (see the stage loop of the kernel).  Two workgroups per
+    // compute unit have 80 KB of LDS each:
+    //  * up to 8 dimensions three stages fit next to the query buffers.  Lists of 256 entries stay
+    //    with the barrier: their merges are so long that the waves of a workgroup do better
+    //    merging together, which leans on the barrier (65536 queries x 2^20 points, d = 8:
+    //    k = 64 14.8 -> 13.9 ms, k = 128 16.4 -> 15.9 ms on the ring, k = 256 19.9 -> 21.9 ms);
+    //  * in 16 to 128 dimensions a stage has 17 KB, and three fit if the query buffers give up a
+    //    quarter of their slots (24 of 32: a few more merges).  Lists of up to 32 entries only:
+    //    longer ones sort their buffers in place, all 32 slots of them.  (65536 queries x 2^20
+    //    points, k = 32: d = 16 20.4 -> 19.9 ms, d = 32 38.5 -> 37.5 ms, d = 64 75.4 -> 73.0 ms,
+    //    d = 128 138.7 -> 137.9 ms.)
+    static constexpr bool RING = !SPLIT && !WIDE &&
+                                 ((DP <= 8 && K <= 128) || (DP >= 16 && DP <= RING_MAX_DP && K <= FQ_CAP));
+    static constexpr int NB = RING ? 3 : 2;
+    static constexpr int SLOTS = RING && DP >= 16 ? 24 : CAP; // slots a query buffer has in LDS
     static_assert(!SPLIT || (DP <= 64 && TPP == KS), "one staging thread per point and cell");
     static constexpr size_t lds_bytes()
     {
         // the stages, the query buffers, exchange slots, merge flags and stage counters
         return NB * static_cast<size_t>(STAGE_FLOATS) * sizeof(float) +
-               static_cast<size_t>(FQ_WAVES) * FQ_QW * CAP * sizeof(u64) +
+               static_cast<size_t>(FQ_WAVES) * FQ_QW * SLOTS * sizeof(u64) +
                static_cast<size_t>(FQ_WAVES) * WAVE * sizeof(float) + 8 * sizeof(int);
     }
 };
@@ -130,6 +141,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     using G = fused_geometry<DP, SPLIT, K, WIDE_OK>;
     constexpr int PT = G::PT;
     constexpr int CAP = G::CAP;
+    constexpr int SLOTS = G::SLOTS;
     // Norms in the accumulator: where one staging thread carries a whole point (DP <= 16) its
     // ||p||^2 is one row after the point rows and is read as the initial value of the
     // accumulators, which saves the matrix step that would add it (one of 5 at DP = 8, one of 9 at
@@ -158,10 +170,10 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     float* const stages = lds;                                                    // [NB][STAGE_FLOATS]
     constexpr bool RING = G::RING;
     constexpr int NB = G::NB;
-    u64* const buffers = reinterpret_cast<u64*>(lds + NB * STAGE_FLOATS);          // [waves][32][CAP]
-    float* const xchg = reinterpret_cast<float*>(buffers + FQ_WAVES * FQ_QW * CAP);  // [waves][64]
+    u64* const buffers = reinterpret_cast<u64*>(lds + NB * STAGE_FLOATS);          // [waves][32][SLOTS]
+    float* const xchg = reinterpret_cast<float*>(buffers + FQ_WAVES * FQ_QW * SLOTS);  // [waves][64]
     int* const merge_wanted = reinterpret_cast<int*>(xchg + FQ_WAVES * WAVE);           // [3]
-    int* const ready = merge_wanted + 4;   // [NB] waves that have written their part, per ring slot
+    int* const ready = merge_wanted + 4;   // [3] waves that have written their part, per ring slot
 
     const int dim = a.dim;
     // this workgroup's range of points
@@ -176,7 +188,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     const int ql = lane & 31;                 // query of this lane inside the wave
     const int wave_q0 = static_cast<int>(blockIdx.x) * FQ_QB + wave * FQ_QW;
     const int my_q = wave_q0 + ql;
-    u64* const wbuf = buffers + static_cast<size_t>(wave) * FQ_QW * CAP;
+    u64* const wbuf = buffers + static_cast<size_t>(wave) * FQ_QW * SLOTS;
     float* const wx = xchg + wave * WAVE;     // 32 radii, then 32 fills (as int bits)
 
     // query fragment: step s of this lane is row 2s + half, times -2 (the stages hold the plain
@@ -282,13 +294,13 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 for (int r = 0; r < BR; ++r)
                 {
                     const int i = sub * BR + r;
-                    buf[r] = i < used ? wbuf[qm * CAP + i] : PAD_KEY;
+                    buf[r] = i < used ? wbuf[qm * SLOTS + i] : PAD_KEY;
                 }
                 net_sort<BL, BR, 2, true>(buf, nullptr, sub);
 #pragma unroll
                 for (int r = 0; r < BR; ++r)
                 {
-                    wbuf[qm * CAP + sub * BR + r] = buf[r];
+                    wbuf[qm * SLOTS + sub * BR + r] = buf[r];
                 }
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -333,11 +345,11 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 {
                     // the sorted buffer (descending, padding first) is the tail of a descending
                     // sequence of K keys
-                    buf[r] = i >= K - CAP ? wbuf[qm * CAP + i - (K - CAP)] : PAD_KEY;
+                    buf[r] = i >= K - CAP ? wbuf[qm * SLOTS + i - (K - CAP)] : PAD_KEY;
                 }
                 else
                 {
-                    buf[r] = i < used ? wbuf[qm * CAP + (i < CAP ? i : 0)] : PAD_KEY;
+                    buf[r] = i < used ? wbuf[qm * SLOTS + (i < SLOTS ? i : 0)] : PAD_KEY;
                 }
                 list[r] = make_key(next_dist[r], next_label[r]);
             }
@@ -405,9 +417,56 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             }
             return count;
         };
+        // the same for the values FROM..TO-1 of every lane only
+        auto compare_some = [&](auto from_tag, auto to_tag) __attribute__((always_inline)) -> int {
+            constexpr int FROM = decltype(from_tag)::value;
+            constexpr int TO = decltype(to_tag)::value;
+            int count = 0;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+            {
+                pass[r] = 0;
+                if (r >= FROM && r < TO)
+                {
+                    const bool below = acc[r] < radius;
+                    pass[r] = __builtin_amdgcn_ballot_w64(below);
+                    count += below ? 1 : 0;
+                }
+            }
+            return count;
+        };
+        const int first_point = tile_base + 4 * half;
+        // Most values of a tile that has candidates fail in every lane: they are skipped four at a
+        // time (a taken branch costs a wave far more than one that is not; 16 of them per tile were
+        // 2-4 % of the kernel time where candidates are rare).  The writes stay in line: moved out
+        // of line they gain another 0.5 % there, but cost 3-7 % where most tiles hold candidates
+        // (lists over ranges of points, which hardly converge).
+        auto write = [&](int mine, int other) __attribute__((always_inline)) {
+            int slot = fill + (half != 0 ? other : 0);
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+            {
+                if ((pass[4 * g] | pass[4 * g + 1] | pass[4 * g + 2] | pass[4 * g + 3]) != 0)
+                {
+#pragma unroll
+                    for (int r = 4 * g; r < 4 * g + 4; ++r)
+                    {
+                        if (pass[r] != 0)
+                        {
+                            if (__builtin_amdgcn_inverse_ballot_w64(pass[r]))
+                            {
+                                wbuf[ql * SLOTS + slot] = make_key(acc[r], first_point + 8 * (r / 4) + (r % 4));
+                                ++slot;
+                            }
+                        }
+                    }
+                }
+            }
+            fill += mine + other;
+        };
         int mine = compare();
         int other = static_cast<int>(lane_xor32<32>(static_cast<u32>(mine)));
-        if (__builtin_amdgcn_ballot_w64(fill + mine + other > CAP) != 0)
+        if (__builtin_amdgcn_ballot_w64(fill + mine + other > SLOTS) != 0)
         {
             // the other waves of the workgroup would wait for this wave at the stage barrier:
             // they are asked to merge their buffers in the meantime
@@ -418,34 +477,25 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             merge_event();
             mine = compare();
             other = static_cast<int>(lane_xor32<32>(static_cast<u32>(mine)));
-        }
-        int slot = fill + (half != 0 ? other : 0);
-        const int first_point = tile_base + 4 * half;
-        // Most values of a tile that has candidates fail in every lane: they are skipped four at a
-        // time (a taken branch costs a wave far more than one that is not; 16 of them per tile were
-        // 2-4 % of the kernel time where candidates are rare).  The writes stay in line: moved out
-        // of line they gain another 0.5 % there, but cost 3-7 % where most tiles hold candidates
-        // (lists over ranges of points, which hardly converge).
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-        {
-            if ((pass[4 * g] | pass[4 * g + 1] | pass[4 * g + 2] | pass[4 * g + 3]) != 0)
+            if constexpr (SLOTS < FQ_CAP)
             {
-#pragma unroll
-                for (int r = 4 * g; r < 4 * g + 4; ++r)
+                // A tile can bring 32 candidates to a query (16 per lane), more than such a buffer
+                // holds: a tile that does not fit the empty buffers is taken in two halves of 8
+                // values per lane, with a merge in between.
+                static_assert(SLOTS >= 16, "half a tile fits an empty buffer");
+                if (__builtin_amdgcn_ballot_w64(mine + other > SLOTS) != 0)
                 {
-                    if (pass[r] != 0)
-                    {
-                        if (__builtin_amdgcn_inverse_ballot_w64(pass[r]))
-                        {
-                            wbuf[ql * CAP + slot] = make_key(acc[r], first_point + 8 * (r / 4) + (r % 4));
-                            ++slot;
-                        }
-                    }
+                    using std::integral_constant;
+                    mine = compare_some(integral_constant<int, 0>{}, integral_constant<int, 8>{});
+                    other = static_cast<int>(lane_xor32<32>(static_cast<u32>(mine)));
+                    write(mine, other);
+                    merge_event();
+                    mine = compare_some(integral_constant<int, 8>{}, integral_constant<int, 16>{});
+                    other = static_cast<int>(lane_xor32<32>(static_cast<u32>(mine)));
                 }
             }
         }
-        fill += mine + other;
+        write(mine, other);
     };
     auto filter_tile = [&](const vfloat16& acc, int tile_base) __attribute__((always_inline)) {
         // The first read of the tile is a compare the compiler sees, so that it places the wait
@@ -867,32 +917,30 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     }
     else
     {
-        // Ring of four stages, filled two stages ahead of the one being multiplied: while stage i is
-        // multiplied, stage i + 1 is complete or about to be, stage i + 2 is written and stage i + 3
-        // is on its way from memory.  A wave counts itself in at ready[slot] once its part of a stage
-        // is written (LDS executes the instructions of a wave in order: the count follows the
-        // writes), and a stage is complete when all waves have counted in: FQ_WAVES more per use of
-        // the slot.  There is no barrier: a wave starts stage i as soon as every wave has finished
-        // stage i - 2, so one that appends or merges holds up the others only when it falls a whole
-        // stage behind.  Writing stage i + 2 over stage i - 2 is safe once stage i is complete:
-        // every wave wrote its part of stage i after it had multiplied stage i - 2.  Stage i itself is
-        // overwritten by stage i + 4, which a wave writes after it has seen stage i + 2 complete,
-        // i.e. after every wave is done with stage i.
-        static_assert(NB == 4, "the ring slot is the stage index modulo 4");
-        auto count_in = [&](int index) __attribute__((always_inline)) {
+        // Ring of three stages.  A wave starts stage i when the stage is complete, writes its part of
+        // stage i + 1 (requested from memory a stage earlier) and then multiplies stage i.  A wave
+        // counts itself in at ready[slot] once its part of a stage is written (LDS executes the
+        // instructions of a wave in order: the count follows the writes), and a stage is complete
+        // when all waves have counted in: FQ_WAVES more per use of the slot.  There is no barrier: a
+        // wave starts stage i + 1 as soon as every wave has started stage i, so one that appends or
+        // merges holds up the others only when it falls a whole stage behind.  Stage i + 1 goes over
+        // stage i - 2, which is safe once stage i is complete: every wave wrote its part of stage i
+        // at the start of stage i - 1, after it had multiplied stage i - 2.
+        // Every wave counts in for every stage whatever it finds in the tiles, and every wait is for
+        // counts of an earlier point of the other waves' programs, so the counts are reached; the
+        // bound on the polls only makes sure that a wave leaves the loop whatever happens.
+        static_assert(NB == 3);
+        auto count_in = [&](int slot) __attribute__((always_inline)) {
             if (lane == 0)
             {
-                __hip_atomic_fetch_add(ready + (index & (NB - 1)), 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(ready + slot, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
         };
-        auto wait_for = [&](int index) __attribute__((always_inline)) {
-            const int complete = FQ_WAVES * (index / NB + 1);
-            // Every wave counts in for every stage whatever it finds in the tiles, so the count is
-            // reached; the bound on the polls only makes sure that a wave leaves this loop whatever
-            // happens.
+        auto wait_for = [&](int slot, int uses) __attribute__((always_inline)) {
+            const int complete = FQ_WAVES * uses;
             for (int polls = 0; polls < (1 << 22); ++polls)
             {
-                if (__hip_atomic_load(ready + (index & (NB - 1)), __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) >= complete)
+                if (__hip_atomic_load(ready + slot, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) >= complete)
                 {
                     break;
                 }
@@ -907,28 +955,25 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         if (n_begin + PT < n)
         {
             fetch(n_begin + PT);
-            __builtin_amdgcn_s_waitcnt(0x0F70);
-            deposit(stages + STAGE_FLOATS, n_begin + PT);
-            count_in(1);
-            if (n_begin + 2 * PT < n)
-            {
-                fetch(n_begin + 2 * PT);
-            }
         }
-        int index = 0;
-        for (int base = n_begin; base < n; base += PT, ++index)
+        int slot = 0;  // of the stage being multiplied
+        int round = 0; // how often that slot has been used before
+        for (int base = n_begin; base < n; base += PT)
         {
-            wait_for(index);
-            multiply(stages + (index & (NB - 1)) * STAGE_FLOATS, base);
-            if (base + 2 * PT < n)
+            wait_for(slot, round + 1);
+            if (base + PT < n)
             {
-                deposit(stages + ((index + 2) & (NB - 1)) * STAGE_FLOATS, base + 2 * PT);
-                count_in(index + 2);
-                if (base + 3 * PT < n)
+                const int next = slot + 1 == NB ? 0 : slot + 1;
+                deposit(stages + next * STAGE_FLOATS, base + PT);
+                count_in(next);
+                if (base + 2 * PT < n)
                 {
-                    fetch(base + 3 * PT);
+                    fetch(base + 2 * PT);
                 }
             }
+            multiply(stages + slot * STAGE_FLOATS, base);
+            slot = slot + 1 == NB ? 0 : slot + 1;
+            round += slot == 0 ? 1 : 0;
         }
     }
 

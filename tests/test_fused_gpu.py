@@ -144,6 +144,26 @@ def test_duplicate_points_are_ordered_by_index(bk, dev, oracle):
     assert np.array_equal(gl, el)
 
 
+@pytest.mark.parametrize("d,k", [(8, 32), (16, 4), (16, 32), (32, 32), (64, 16), (16, 64), (100, 32)])
+def test_points_that_come_ever_closer(bk, dev, oracle, d, k):
+    # Every point is nearer to every query than all points before it, so every tile brings each
+    # query 32 candidates: more than a query buffer of 24 slots holds even when it is empty (the
+    # geometries with three stages in LDS), which has such a tile appended in two halves.  Small
+    # integer coordinates keep the arithmetic exact, so the result must equal the oracle's bit for
+    # bit.
+    n, q = 2000, 200
+    rng = np.random.default_rng(d * 100 + k)
+    s = rng.integers(-2, 3, size=(q, d)).astype(np.float32)
+    p = np.zeros((n, d), dtype=np.float32)
+    p[:, 0] = 20 + (n - 1 - np.arange(n))         # 2019, 2018, ..., 20 along the first axis
+    p[:, 1:3] = rng.integers(-1, 2, size=(n, 2))  # (a step along it outweighs what these can add)
+    part = oracle.dist(s, p, "partial")
+    assert np.all(np.diff(part, axis=1) < 0), "the points must approach every query"
+    gd, gl = _fused(bk, dev, p, s, k)
+    ed, el = oracle.topk(part, k)
+    assert np.array_equal(gd, ed) and np.array_equal(gl, el)
+
+
 def test_exact_arithmetic_is_bit_exact(bk, dev, oracle):
     # small integers: every product and sum is exact in fp32, so the fused result must equal the
     # oracle bit for bit, labels included (heavy ties)
