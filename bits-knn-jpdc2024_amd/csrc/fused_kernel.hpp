@@ -116,7 +116,9 @@ struct fused_geometry
     //    k = 64 14.8 -> 13.9 ms, k = 128 16.4 -> 15.9 ms on the ring, k = 256 19.9 -> 21.9 ms);
     //  * in 16 to 128 dimensions a stage has 17 KB, and three fit if the query buffers give up a
     //    quarter of their slots (24 of 32: a few more merges).  Lists of up to 32 entries only:
-    //    longer ones sort their buffers in place, all 32 slots of them.  (65536 queries x 2^20
+    //    longer ones sort their buffers in place, all 32 slots of them, and with that changed they
+    //    gain 2-3 % at k = 64 on many queries but lose 4-8 % (k = 64) and 26 % (k = 128) over
+    //    ranges of points, where merges of long lists are what the time goes into.  (65536 queries x 2^20
     //    points, k = 32: d = 16 20.4 -> 19.9 ms, d = 32 38.5 -> 37.5 ms, d = 64 75.4 -> 73.0 ms,
     //    d = 128 138.7 -> 137.9 ms.)
     static constexpr bool RING = !SPLIT && !WIDE &&
