@@ -13,7 +13,8 @@ constexpr int FQ_THREADS = FQ_WAVES * WAVE;   // 256
 constexpr int FQ_QW = 32;                     // queries per wave (one MFMA column tile)
 constexpr int FQ_QB = FQ_QW * FQ_WAVES;       // queries per workgroup
 constexpr int FQ_CAP = 32;                    // buffer slots per query (= points per MFMA tile); twice
-                                              // that for long lists in few dimensions (fused_geometry)
+                                              // that for long lists in few dimensions, 24 of them in
+                                              // LDS where three stages have to fit (fused_geometry)
 
 constexpr int FUSED_PLAIN = -1;
 constexpr int FUSED_REPEAT_MARKED = -2;
