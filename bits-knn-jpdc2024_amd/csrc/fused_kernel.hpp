@@ -10,7 +10,7 @@
 //  * A workgroup of 4 waves owns 128 queries (32 per wave) and walks over its range of points in
 //    stages of PT points, two stages in LDS (one being multiplied, one being filled; one barrier
 //    per stage) or, for lists of up to 128 entries in up to 8 dimensions and of up to 32 entries in
-//    16 to 128 dimensions, a ring of three stages without barriers.
+//    16 to 128 dimensions or with bf16 pieces, a ring of three stages without barriers.
 //    A stage is the MFMA A operand: rows 0..d-1 hold the points, the following rows
 //    hold the staging threads' shares of ||p||^2, so that v_mfma_f32_32x32x2_f32 against the query
 //    fragment (-2q_0..-2q_{d-1}, 1, 1) yields ||p||^2 - 2 q.p directly, the dot product accumulated
@@ -121,10 +121,16 @@ struct fused_geometry
     //    ranges of points, where merges of long lists are what the time goes into.  (65536 queries x 2^20
     //    points, k = 32: d = 16 20.4 -> 19.9 ms, d = 32 38.5 -> 37.5 ms, d = 64 75.4 -> 73.0 ms,
     //    d = 128 138.7 -> 137.9 ms.)
-    static constexpr bool RING = !SPLIT && !WIDE &&
-                                 ((DP <= 8 && K <= 128) || (DP >= 16 && DP <= RING_MAX_DP && K <= FQ_CAP));
+    //  * the stages of the bf16 pieces have 12.5 KB in every dimension: three fit as they are.
+    //    Lists of up to 32 entries (65536 queries x 2^20 points, k = 32: d = 16 14.0 -> 13.8 ms,
+    //    d = 64 51.2 -> 47.0 ms; 8192 queries x 2^17 points over ranges: d = 16 0.78 -> 0.68 ms,
+    //    d = 32 0.96 -> 0.87 ms); lists of 64 and 128 gain 4 % on many queries and lose 14 % over
+    //    ranges.
+    static constexpr bool RING =
+        !WIDE && (SPLIT ? K <= FQ_CAP
+                        : (DP <= 8 && K <= 128) || (DP >= 16 && DP <= RING_MAX_DP && K <= FQ_CAP));
     static constexpr int NB = RING ? 3 : 2;
-    static constexpr int SLOTS = RING && DP >= 16 ? 24 : CAP; // slots a query buffer has in LDS
+    static constexpr int SLOTS = RING && !SPLIT && DP >= 16 ? 24 : CAP; // slots a query buffer has in LDS
     static_assert(!SPLIT || (DP <= 64 && TPP == KS), "one staging thread per point and cell");
     static constexpr size_t lds_bytes()
     {
