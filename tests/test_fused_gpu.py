@@ -101,6 +101,23 @@ def test_ragged_counts(bk, dev, oracle, n, q):
         _check(oracle, p, s, k, gd, gl)
 
 
+# points per stage by padded dimension: 256 up to 16 dimensions, 128 / 64 / 32 for 32 / 64 / 128
+@pytest.mark.parametrize("d,stage", [(8, 256), (16, 256), (32, 128), (64, 64), (100, 32)])
+@pytest.mark.parametrize("arithmetic", ["fp32", "bf16x3"])
+def test_point_counts_around_whole_stages(bk, dev, oracle, d, stage, arithmetic):
+    # one to five stages, each count one short of, at and one past a whole stage: the ring of three
+    # stage buffers starts, wraps around and ends at every position
+    if arithmetic == "bf16x3" and not 9 <= d <= 64:
+        pytest.skip("bf16x3 products serve 9 to 64 dimensions")
+    mode = bk.FUSED_BF16X3 if arithmetic == "bf16x3" else None
+    q = 130
+    for stages in (1, 2, 3, 4, 5):
+        for n in (stages * stage - 1, stages * stage, stages * stage + 1):
+            p, s = oracle.generate(1000 * stages + n + d, n, q, d)
+            gd, gl = _fused(bk, dev, p, s, 16, arithmetic=mode)
+            _check(oracle, p, s, 16, gd, gl)
+
+
 @pytest.mark.parametrize("n,q,d,k", [(20000, 150, 8, 32), (70001, 300, 16, 16), (300000, 33, 32, 4),
                                      (9000, 1000, 8, 64), (131072, 1024, 5, 128), (40000, 128, 8, 256),
                                      (50000, 200, 16, 256), (33000, 77, 13, 128)])
