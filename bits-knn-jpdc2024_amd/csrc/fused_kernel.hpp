@@ -100,7 +100,13 @@ struct fused_geometry
     // point rows (zero beyond dim), then one row per staging thread of a point with its share of
     // ||p||^2 (at least two rows, so that the row count is even)
     // (one row where it is read as the initial accumulator and never multiplied)
-    static constexpr int NORM_ROWS = (!SPLIT && TPP == 1 && PT >= 64) ? 1 : (TPP > 2 ? TPP : 2);
+    // PAIRED: the 2 or 4 staging threads of a point are neighbouring lanes, which add up their
+    // shares of the norm among themselves: one norm row, read as the initial accumulator
+    // (not for lists of 128 entries in 32 dimensions: that instantiation then needs 260 vector
+    // registers, 4 more than two waves per SIMD leave it)
+    static constexpr bool PAIRED =
+        !SPLIT && !WIDE && (TPP == 2 || TPP == 4) && PT >= 64 && !(DP == 32 && K == 128);
+    static constexpr int NORM_ROWS = (!SPLIT && (TPP == 1 || PAIRED) && PT >= 64) ? 1 : (TPP > 2 ? TPP : 2);
     static constexpr int ROWS = DP + NORM_ROWS;
     static constexpr int STEPS = ROWS / 2;    // MFMA steps of 2 rows
     static constexpr int VPT = SPLIT ? 8 : DP / TPP; // values a thread carries from global memory to LDS
@@ -155,7 +161,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     // accumulators, which saves the matrix step that would add it (one of 5 at DP = 8, one of 9 at
     // DP = 16; at DP = 32 the 32 registers it takes cost as much as the 17th step).  The sum then
     // starts from the norm instead of ending with it: same terms, another rounding order.
-    constexpr bool NORM_IN_C = SPLIT || (G::TPP == 1 && G::MT >= 2);
+    constexpr bool NORM_IN_C = SPLIT || ((G::TPP == 1 || G::PAIRED) && G::MT >= 2);
     constexpr int STEPS = NORM_IN_C ? DP / 2 : G::STEPS;
     constexpr int KB = G::KB;
     constexpr int KS = G::KS;
@@ -530,8 +536,8 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     // stage and adds up its share of ||p||^2 (the shares of a point meet inside the MFMA)
     // SPLIT: thread t carries the 8 dimensions 8*(t % TPP) .. + 7 of point t / TPP (the threads of
     // a point are neighbouring lanes, which add up their shares of the norm among themselves)
-    const int sp = SPLIT ? t / TPP : t % PT;
-    const int sd0 = SPLIT ? 8 * (t % TPP) : t / PT;
+    const int sp = SPLIT || G::PAIRED ? t / TPP : t % PT;
+    const int sd0 = SPLIT ? 8 * (t % TPP) : (G::PAIRED ? t % TPP : t / PT);
     auto dim_of = [&](int i) -> int { return SPLIT ? sd0 + i : sd0 + TPP * i; };
     float pre[VPT];
     // Point values are read with buffer loads: a constant byte offset per value and lane (beyond
@@ -652,7 +658,19 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             }
             // points beyond the end get an infinite distance and never pass the filter
             // (with one staging thread per point the share is the norm, in row DP)
-            stage[(DP + sd0) * PT + sp] = base + sp < n ? share : __builtin_inff();
+            if constexpr (G::PAIRED)
+            {
+                share += __builtin_bit_cast(float, lane_xor32<1>(__builtin_bit_cast(u32, share)));
+                if constexpr (TPP == 4)
+                {
+                    share += __builtin_bit_cast(float, lane_xor32<2>(__builtin_bit_cast(u32, share)));
+                }
+                stage[DP * PT + sp] = base + sp < n ? share : __builtin_inff();
+            }
+            else
+            {
+                stage[(DP + sd0) * PT + sp] = base + sp < n ? share : __builtin_inff();
+            }
         }
     };
 
