@@ -14,7 +14,8 @@
 //    A stage is the MFMA A operand: rows 0..d-1 hold the points, the following rows
 //    hold the staging threads' shares of ||p||^2, so that v_mfma_f32_32x32x2_f32 against the query
 //    fragment (-2q_0..-2q_{d-1}, 1, 1) yields ||p||^2 - 2 q.p directly, the dot product accumulated
-//    first and the norm added last.  For d <= 16 the norm is the initial accumulator instead.
+//    first and the norm added last.  For d <= 64 the norm is one row and the initial accumulator
+//    instead.
 //  * The query fragment stays in registers for the whole kernel.  In the 32 x 32 result tile a
 //    lane holds 16 distances of ONE query (column), so the filter is a min-tree over 16
 //    registers and one compare against that query's radius.
@@ -156,11 +157,13 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     constexpr int PT = G::PT;
     constexpr int CAP = G::CAP;
     constexpr int SLOTS = G::SLOTS;
-    // Norms in the accumulator: where one staging thread carries a whole point (DP <= 16) its
-    // ||p||^2 is one row after the point rows and is read as the initial value of the
-    // accumulators, which saves the matrix step that would add it (one of 5 at DP = 8, one of 9 at
-    // DP = 16; at DP = 32 the 32 registers it takes cost as much as the 17th step).  The sum then
-    // starts from the norm instead of ending with it: same terms, another rounding order.
+    // Norms in the accumulator: where ||p||^2 is one row after the point rows -- one staging thread
+    // carries a whole point (DP <= 16), or the 2 or 4 staging threads of a point are neighbouring
+    // lanes that add up their shares (DP = 32, 64) -- it is read as the initial value of the
+    // accumulators, which saves the matrix step that would add it (one of 5 at DP = 8, of 9 at 16,
+    // of 17 at 32, of 33 at 64; 65536 queries x 2^20 points, k = 32: d = 32 37.7 -> 36.4 ms, d = 64
+    // 73.0 -> 71.8 ms).  The sum then starts from the norm instead of ending with it: same terms,
+    // another rounding order.
     constexpr bool NORM_IN_C = SPLIT || ((G::TPP == 1 || G::PAIRED) && G::MT >= 2);
     constexpr int STEPS = NORM_IN_C ? DP / 2 : G::STEPS;
     constexpr int KB = G::KB;
@@ -534,8 +537,10 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     // ---- staging: global -> registers -> LDS ---------------------------------------------------
     // thread t carries dimensions (t / PT) + TPP*i of point t % PT, writes them as rows of the
     // stage and adds up its share of ||p||^2 (the shares of a point meet inside the MFMA)
-    // SPLIT: thread t carries the 8 dimensions 8*(t % TPP) .. + 7 of point t / TPP (the threads of
-    // a point are neighbouring lanes, which add up their shares of the norm among themselves)
+    // PAIRED: thread t carries dimensions (t % TPP) + TPP*i of point t / TPP: the threads of a point
+    // are neighbouring lanes, which add up their shares of the norm among themselves
+    // SPLIT: thread t carries the 8 dimensions 8*(t % TPP) .. + 7 of point t / TPP (neighbouring
+    // lanes as well)
     const int sp = SPLIT || G::PAIRED ? t / TPP : t % PT;
     const int sd0 = SPLIT ? 8 * (t % TPP) : (G::PAIRED ? t % TPP : t / PT);
     auto dim_of = [&](int i) -> int { return SPLIT ? sd0 + i : sd0 + TPP * i; };
