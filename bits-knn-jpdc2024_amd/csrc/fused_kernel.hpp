@@ -133,6 +133,9 @@ struct fused_geometry
     //    d = 64 51.2 -> 47.0 ms; 8192 queries x 2^17 points over ranges: d = 16 0.78 -> 0.68 ms,
     //    d = 32 0.96 -> 0.87 ms); lists of 64 and 128 gain 4 % on many queries and lose 14 % over
     //    ranges.
+    // (The geometry with 64-slot buffers would have room for three of its small stages, but its
+    // long lists over ranges want the waves merging together: 8192 queries x 2^17 points, d = 8,
+    // k = 128 1.10 -> 1.46 ms on the ring.)
     static constexpr bool RING =
         !WIDE && (SPLIT ? K <= FQ_CAP
                         : (DP <= 8 && K <= 128) || (DP >= 16 && DP <= RING_MAX_DP && K <= FQ_CAP));
@@ -157,6 +160,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     constexpr int PT = G::PT;
     constexpr int CAP = G::CAP;
     constexpr int SLOTS = G::SLOTS;
+    static_assert(K <= CAP || SLOTS == CAP, "lists longer than a buffer sort all CAP slots of it in place");
     // Norms in the accumulator: where ||p||^2 is one row after the point rows -- one staging thread
     // carries a whole point (DP <= 16), or the 2 or 4 staging threads of a point are neighbouring
     // lanes that add up their shares (DP = 32, 64) -- it is read as the initial value of the
