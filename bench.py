@@ -136,18 +136,28 @@ def verify_topk(oracle, cache, matrix, sample, k, out_d, out_l):
     return bool(np.array_equal(got_d.view(np.uint32), exp_d.view(np.uint32)) and np.array_equal(got_l, exp_l))
 
 
+RESOLUTION = 2.0 ** -20  # of the scale of the cancelling terms: 16 units in the last place
+
+
 def verify_neighbours(np, points, queries, exp_d, exp_l, got_d, got_l, k):
-    """k-th neighbour distance within REL of the scale of its terms (|value| + ||q||^2) and recall
-    >= MIN_RECALL against the oracle's lists of partial distances; a reported point outside the
-    oracle's list counts when its exact distance is within the tolerance of the k-th distance
-    (neighbours closer together than fp32 resolves).  Also returns the error of the completed
-    k-th distance (value + ||q||^2) relative to itself, for the record."""
+    """The bar of the parity tests on the sampled queries: recall >= MIN_RECALL against the oracle's
+    lists of partial distances (a reported point outside the oracle's list counts when its exact
+    distance is within the tolerance of the k-th distance: neighbours closer together than fp32
+    resolves), ascending lists, and the k-th neighbour distance within REL -- of the scale of its
+    terms (|value| + ||q||^2) always; of the completed distance value + ||q||^2 from 16 dimensions
+    on; below that of the reported value itself, except for queries whose error is within
+    RESOLUTION of the scale (the value is a small difference of its terms there).  Every error is
+    reported uncapped, with the number of queries that took the exception."""
+    dim = queries.shape[1]
     qn = (queries.astype(np.float64) ** 2).sum(1)
     kth_e = exp_d[:, k - 1].astype(np.float64)
     kth_g = got_d[:, k - 1].astype(np.float64)
     scale = np.abs(kth_e) + qn
-    err_scale = float(np.max(np.abs(kth_g - kth_e) / scale))
-    err_completed = float(np.max(np.abs(kth_g - kth_e) / np.maximum(kth_e + qn, 1e-30)))
+    diff = np.abs(kth_g - kth_e)
+    of_scale = diff / scale
+    completed = diff / np.maximum(kth_e + qn, 1e-30)
+    of_value = np.where(diff == 0, 0.0, diff / np.maximum(np.abs(kth_e), 1e-300))
+    excused = (diff != 0) & (of_scale <= RESOLUTION) & (of_value > REL)
     hits = 0
     for row in range(queries.shape[0]):
         want = set(exp_l[row].tolist())
@@ -160,8 +170,11 @@ def verify_neighbours(np, points, queries, exp_d, exp_l, got_d, got_l, k):
             hits += exact <= kth_e[row] + REL * scale[row]
     recall = hits / (queries.shape[0] * k)
     ascending = bool(np.all(got_d[:, 1:] >= got_d[:, :-1]))
-    ok = err_scale <= REL and recall >= MIN_RECALL and ascending
-    return ok, {"kth_err_of_scale": err_scale, "kth_err_of_completed_distance": err_completed, "recall": recall}
+    value_ok = bool(np.all(completed <= REL)) if dim >= 16 else bool(np.all((of_value <= REL) | excused))
+    ok = bool(np.all(of_scale <= REL)) and value_ok and recall >= MIN_RECALL and ascending
+    return ok, {"kth_err_of_scale": float(of_scale.max()), "kth_err_of_completed_distance": float(completed.max()),
+                "kth_err_of_value": float(of_value.max()), "queries": int(queries.shape[0]),
+                "queries_excused_below_resolution": int(excused.sum()), "recall": recall}
 
 
 def leg_calibration(bitsknn, torch, timer, matrix, steps):

@@ -12,7 +12,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "libbitsknn.so")
 
-OK, ERR_UNSUPPORTED, ERR_INVALID, ERR_HIP = 0, 1, 2, 3
+OK, ERR_UNSUPPORTED, ERR_INVALID, ERR_HIP, ERR_INTERNAL = 0, 1, 2, 3, 4
 DIST_L2, DIST_PARTIAL_L2, DIST_EXPANDED, DIST_PARTIAL_L2_BF16X3 = 0, 1, 2, 3
 
 # every symbol include/bitsknn.h declares
@@ -31,6 +31,7 @@ EXPORTS = (
     "bitsknn_fused_l2_topk_f32_ex",
     "bitsknn_fused_static_scratch_bytes",
     "bitsknn_fused_l2_topk_f32_static",
+    "bitsknn_fused_status",
 )
 
 
@@ -92,6 +93,8 @@ def lib():
         L.bitsknn_fused_static_scratch_bytes.argtypes = []
         L.bitsknn_fused_l2_topk_f32_static.restype = ctypes.c_int
         L.bitsknn_fused_l2_topk_f32_static.argtypes = L.bitsknn_fused_l2_topk_f32.argtypes
+        L.bitsknn_fused_status.restype = ctypes.c_int
+        L.bitsknn_fused_status.argtypes = [vp]
         _lib = L
     return _lib
 
@@ -241,3 +244,9 @@ def fused_workspace_bytes(q, n, k):
 
 def fused_static_scratch_bytes():
     return int(lib().bitsknn_fused_static_scratch_bytes())
+
+
+def fused_status():
+    """Synchronises the current stream and raises BitsKnnError(ERR_INTERNAL) if a fused kernel has
+    reported a wait that ran out of polls since the last check."""
+    _check(lib().bitsknn_fused_status(_stream()))

@@ -1,5 +1,6 @@
 // C-ABI entry points of bits-fused: parameter validation, the choice between the fused kernel and
 // its point-split form, and dispatch to the kernels instantiated per list length in fused_inst.hip.
+#include <cstdlib>
 #include <initializer_list>
 #include <mutex>
 
@@ -18,41 +19,68 @@ namespace
 constexpr size_t STATIC_SCRATCH_BYTES = 32ULL << 20;
 static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
 
-constexpr int MAX_DEVICES = 64;
-std::mutex g_scratch_mutex;
-void* g_scratch_ptr[MAX_DEVICES] = {}; // device address of `scratch` on each device, once known
+// Sticky fault word of the fused kernels (one copy per GPU, like `scratch`): the number of waits
+// for a stage of the ring that ran out of polls since bitsknn_fused_status last looked.
+static __device__ __align__(16) int fault_word[4];
 
-// Device address of the current device's copy of `scratch`, looked up on the first call per
-// device; nullptr (with the error recorded) when a runtime call fails.
-void* static_scratch()
+constexpr int MAX_DEVICES = 64;
+// Default bound on the polls of one wait for a stage (each poll sleeps 64 cycles: about 0.1 s in
+// all, many thousand times the longest merge a wave can be held up by).
+constexpr int DEFAULT_POLL_LIMIT = 1 << 22;
+
+struct device_symbols
+{
+    void* scratch = nullptr; // device addresses of this device's copies
+    int* fault = nullptr;
+};
+std::mutex g_symbols_mutex;
+device_symbols g_symbols[MAX_DEVICES];
+
+// Device addresses of the current device's copies of `scratch` and `fault_word`, looked up on the
+// first call per device.  Returns BITSKNN_OK or the status it has recorded with its message.
+int symbols_of_current_device(device_symbols& out)
 {
     int device = -1;
-    hipError_t status = hipGetDevice(&device);
-    if (status == hipSuccess && (device < 0 || device >= MAX_DEVICES))
+    BITSKNN_HIP_CHECK(hipGetDevice(&device));
+    if (device < 0 || device >= MAX_DEVICES)
     {
-        fail(BITSKNN_ERR_INVALID, "bitsknn_fused_l2_topk_f32_static: device %d is not supported (at most %d)",
-             device, MAX_DEVICES);
-        return nullptr;
+        return fail(BITSKNN_ERR_INVALID, "bits-fused: device %d is not supported (at most %d)", device,
+                    MAX_DEVICES);
     }
-    if (status == hipSuccess)
+    const std::lock_guard<std::mutex> lock{g_symbols_mutex};
+    device_symbols& mine = g_symbols[device];
+    if (mine.fault == nullptr)
     {
-        const std::lock_guard<std::mutex> lock{g_scratch_mutex};
-        if (g_scratch_ptr[device] == nullptr)
+        void* scratch_ptr = nullptr;
+        void* fault_ptr = nullptr;
+        BITSKNN_HIP_CHECK(hipGetSymbolAddress(&scratch_ptr, HIP_SYMBOL(scratch)));
+        BITSKNN_HIP_CHECK(hipGetSymbolAddress(&fault_ptr, HIP_SYMBOL(fault_word)));
+        mine.scratch = scratch_ptr;
+        mine.fault = static_cast<int*>(fault_ptr);
+    }
+    out = mine;
+    return BITSKNN_OK;
+}
+
+// Bound on the polls of a wait in the ring of stages: BITSKNN_FUSED_POLL_LIMIT in the environment
+// (read once; 0 makes every wait that finds its stage incomplete give up at once, which is how the
+// tests reach the failure path from the host), else DEFAULT_POLL_LIMIT.
+int poll_limit()
+{
+    static const int limit = [] {
+        const char* text = std::getenv("BITSKNN_FUSED_POLL_LIMIT");
+        if (text != nullptr && *text != '\0')
         {
-            void* ptr = nullptr;
-            status = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
-            if (status == hipSuccess)
+            char* end = nullptr;
+            const long value = std::strtol(text, &end, 10);
+            if (end != text && *end == '\0' && value >= 0 && value <= DEFAULT_POLL_LIMIT)
             {
-                g_scratch_ptr[device] = ptr;
+                return static_cast<int>(value);
             }
         }
-        if (status == hipSuccess)
-        {
-            return g_scratch_ptr[device];
-        }
-    }
-    fail(BITSKNN_ERR_HIP, "%s:%d %s: %s", __FILE__, __LINE__, hipGetErrorName(status), hipGetErrorString(status));
-    return nullptr;
+        return DEFAULT_POLL_LIMIT;
+    }();
+    return limit;
 }
 
 bool in_list(int v, std::initializer_list<int> values)
@@ -238,8 +266,14 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
         splits /= 2;
     }
     const size_t pairs = static_cast<size_t>(q) * static_cast<size_t>(splits) * static_cast<size_t>(k);
+    device_symbols symbols;
+    const int looked_up = symbols_of_current_device(symbols);
+    if (looked_up != BITSKNN_OK)
+    {
+        return looked_up;
+    }
     fused_args a{queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, 1, 0, k, n, 1, 0, FUSED_PLAIN,
-                 out_dist, k};
+                 out_dist, k, symbols.fault, poll_limit()};
     if (splits > 1)
     {
         // partial lists [q][splits][k] in the workspace: distances first, then labels
@@ -378,15 +412,44 @@ extern "C" int bitsknn_fused_l2_topk_f32_static(const float* queries_dim_major,
     void* workspace = nullptr;
     if (need != 0 && q > 0)
     {
-        workspace = static_scratch();
-        if (workspace == nullptr)
+        device_symbols symbols;
+        const int looked_up = symbols_of_current_device(symbols);
+        if (looked_up != BITSKNN_OK)
         {
-            return BITSKNN_ERR_HIP;
+            return looked_up;
         }
+        workspace = symbols.scratch;
     }
     // The kernels write every entry of the partial lists they read back (ranges without points
     // included), so nothing in the scratch memory has to be cleared between calls.
     return fused_impl(queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, k, query_reg,
                       db_reg, dim_reg, block_query_dim, dim_mult, BITSKNN_FUSED_FP32, workspace,
                       workspace != nullptr ? STATIC_SCRATCH_BYTES : 0, workspace != nullptr, stream);
+}
+
+extern "C" int bitsknn_fused_status(void* stream)
+{
+    using namespace bitsknn;
+    clear_error();
+    device_symbols symbols;
+    const int looked_up = symbols_of_current_device(symbols);
+    if (looked_up != BITSKNN_OK)
+    {
+        return looked_up;
+    }
+    auto* hip_stream = static_cast<hipStream_t>(stream);
+    int gave_up = 0;
+    BITSKNN_HIP_CHECK(hipMemcpyAsync(&gave_up, symbols.fault, sizeof(int), hipMemcpyDeviceToHost, hip_stream));
+    BITSKNN_HIP_CHECK(hipStreamSynchronize(hip_stream));
+    if (gave_up == 0)
+    {
+        return BITSKNN_OK;
+    }
+    static const int zero = 0;
+    BITSKNN_HIP_CHECK(hipMemcpyAsync(symbols.fault, &zero, sizeof(int), hipMemcpyHostToDevice, hip_stream));
+    BITSKNN_HIP_CHECK(hipStreamSynchronize(hip_stream));
+    return fail(BITSKNN_ERR_INTERNAL,
+                "bits-fused: %d waits for a stage ran out of polls; the lists of the queries concerned end "
+                "in NaN and the results of the calls since the last check must be discarded",
+                gave_up);
 }

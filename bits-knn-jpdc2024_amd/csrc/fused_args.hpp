@@ -48,6 +48,11 @@ struct fused_args
     int first_radius;
     const float* final_dist; // the caller's output array (out_dist itself with one range of points)
     int final_stride;
+    // Ring of stages: a wait that is still short of its count after poll_limit polls gives up; the
+    // wave then goes on (every wave leaves the kernel whatever happens), adds one to *fault at the
+    // end and overwrites the k-th distances of its queries with NaN.
+    int* fault;
+    int poll_limit;
 };
 
 // one per compiled list length K (fused_inst.hip); split: products from three bf16 pieces per

@@ -291,6 +291,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     bool have_list = false;          // wave-uniform: the lists in the output arrays are valid
     bool merged = false;             // wave-uniform: this wave has merged during the current stage
     int stage_slot = 0;              // stage index modulo 3: the slot of merge_wanted in use
+    bool gave_up = false;            // wave-uniform: a wait for a stage of the ring ran out of polls
 
     // ---- merge of all buffers of this wave into the lists --------------------------------------
     auto merge_event = [&]() __attribute__((always_inline)) {
@@ -963,7 +964,9 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         // at the start of stage i - 1, after it had multiplied stage i - 2.
         // Every wave counts in for every stage whatever it finds in the tiles, and every wait is for
         // counts of an earlier point of the other waves' programs, so the counts are reached; the
-        // bound on the polls only makes sure that a wave leaves the loop whatever happens.
+        // bound on the polls only makes sure that a wave leaves the loop whatever happens.  A wave
+        // whose wait ran out of polls goes on with a stage that may be incomplete, so it marks what
+        // it reports at the end: NaN as the k-th distance of its queries and a count in *a.fault.
         static_assert(NB == 3);
         auto count_in = [&](int slot) __attribute__((always_inline)) {
             if (lane == 0)
@@ -973,12 +976,15 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         };
         auto wait_for = [&](int slot, int uses) __attribute__((always_inline)) {
             const int complete = FQ_WAVES * uses;
-            for (int polls = 0; polls < (1 << 22); ++polls)
+            int polls = a.poll_limit;
+            while (__hip_atomic_load(ready + slot, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < complete)
             {
-                if (__hip_atomic_load(ready + slot, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) >= complete)
+                if (polls <= 0)
                 {
+                    gave_up = true;
                     break;
                 }
+                --polls;
                 __builtin_amdgcn_s_sleep(1);
             }
         };
@@ -1018,6 +1024,21 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     if (a.splits == 1 && first_radius < __builtin_inff() && !(radius < first_radius) && half == 0)
     {
         a.out_dist[static_cast<size_t>(my_q) * list_stride + K - 1] = __builtin_nanf("");
+    }
+    if constexpr (RING)
+    {
+        if (gave_up)
+        {
+            if (half == 0 && my_q < a.q)
+            {
+                a.out_dist[(static_cast<size_t>(my_q) * a.splits + blockIdx.y) * list_stride + K - 1] =
+                    __builtin_nanf("");
+            }
+            if (lane == 0)
+            {
+                __hip_atomic_fetch_add(a.fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
     }
 }
 

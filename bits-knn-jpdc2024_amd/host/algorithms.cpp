@@ -447,7 +447,8 @@ public:
             static_cast<int>(args_.items_per_thread[1]), static_cast<int>(args_.items_per_thread[2]),
             static_cast<int>(args_.selection_block_size), static_cast<int>(args_.deg), arithmetic_,
             workspace_.size() != 0 ? workspace_.data() : nullptr, workspace_.size(), nullptr));
-        sync_default_stream();
+        // synchronises, and fails if a wave of the kernel gave up a wait for a stage
+        BITSKNN_CHECK(bitsknn_fused_status(nullptr));
     }
 
     float transfer_in_seconds() const override { return transfer_in_.seconds(); }

@@ -27,6 +27,7 @@ extern "C" {
 #define BITSKNN_ERR_UNSUPPORTED 1 /* parameter outside the compiled lists (reference: runtime_error "Unsupported ...") */
 #define BITSKNN_ERR_INVALID 2     /* null pointer / inconsistent sizes */
 #define BITSKNN_ERR_HIP 3         /* a HIP runtime call failed (reference: CUCH -> runtime_error) */
+#define BITSKNN_ERR_INTERNAL 4    /* a kernel reported that it could not keep its own protocol (bitsknn_fused_status) */
 
 /* Message of the last error reported on this thread ("" if none). Never NULL. */
 const char* bitsknn_last_error(void);
@@ -224,6 +225,24 @@ int bitsknn_fused_l2_topk_f32_static(const float* queries_dim_major, const float
                                      int dim, int32_t q, int32_t n, float* out_dist,
                                      int32_t* out_label, int k, int query_reg, int db_reg, int dim_reg,
                                      int block_query_dim, int dim_mult, void* stream);
+
+/*
+ * Health check of the bits-fused kernels on the current device.  Where the stages of points are
+ * handed from wave to wave through counters in LDS instead of barriers, a wave waits for a stage
+ * with a bounded number of polls, so that every wave leaves the kernel whatever happens.  The
+ * bound is never reached in a correct run; if it is, the wave goes on with what it has, writes NaN
+ * as the k-th distance of each of its queries and counts the event in a word of device memory
+ * inside the library.  This call synchronises `stream`, reads that word and clears it: BITSKNN_OK
+ * when no wait has run out of polls since the last check, else BITSKNN_ERR_INTERNAL (the results
+ * of the fused calls since the last check must be discarded).  The `knn` driver checks after every
+ * fused selection, where the reference synchronises and checks its launch
+ * (src/topk/singlepass/fused_cache_knn.cu:213-215, CUCH(cudaGetLastError()) in
+ * include/bits/topk/singlepass/detail/fused_cache_kernel.cuh:38-42).
+ * BITSKNN_FUSED_POLL_LIMIT in the environment (read once per process, 0 .. 4194304, default
+ * 4194304) sets the bound; tests set it to 0 to reach this path with kernels that still end
+ * normally.
+ */
+int bitsknn_fused_status(void* stream);
 
 #ifdef __cplusplus
 }

@@ -1,6 +1,6 @@
 // Test-only timing probes of how gfx950 issues fp32 matrix instructions next to vector instructions:
 // the measurements the fused and distance kernels were shaped by (loaded by
-// tests/test_issue_probe_gpu.py, built into tests/libissueprobe.so).  Nothing in the library uses
+// tests/test_y_issue_probe_gpu.py, built into tests/libissueprobe.so).  Nothing in the library uses
 // this file.
 //
 //  * chain:   nothing but v_mfma_f32_32x32x2_f32, CHAINS independent accumulator chains per wave;

@@ -16,6 +16,9 @@ itself is v + ||q||^2.  Three measures of the k-th neighbour's error, strictest 
               in the last place of the terms, which is what fp32 can resolve.
   of_scale    |v_gpu - v_ref| / (|v_ref| + ||q||^2) relative to the terms that cancel.  Always
               asserted.
+
+Effective bar for dim < 16, per query: of_value <= 1e-5 or of_scale <= 2^-20 (and of_scale <= 1e-5
+always).  The recorded margins are not capped and count the queries that took the second clause.
 """
 import numpy as np
 
@@ -23,46 +26,72 @@ REL = 1e-5
 MIN_RECALL = 0.999
 STRICT_FROM_DIM = 16
 
-# the largest errors seen by assert_kth_distance per (dim class), for the record (pytest -s prints
-# them at the end of the session)
+# The largest errors seen by assert_kth_distance per dimension class, for the record (pytest prints
+# them at the end of the session).  Nothing in them is capped: `of_value` is the largest
+# |v_gpu - v_ref| / |v_ref| over ALL queries checked, `of_value_asserted` the largest over the
+# queries the of_value bar applies to, `excused` how many of `queries` took the RESOLUTION clause
+# instead (error within 2^-20 of the scale of the cancelling terms), and `of_value_excused` the
+# largest value-relative error among those.
 margins = {}
 
 
 RESOLUTION = 2.0 ** -20  # of the scale of the cancelling terms: 16 units in the last place
 
 
-def kth_errors(queries, exp_kth, got_kth):
-    """Largest error of each kind over the queries; of_value skips the queries whose error is
-    within RESOLUTION of the scale (the value is a small difference of its terms there)."""
+def kth_error_detail(queries, exp_kth, got_kth):
+    """Errors of the k-th neighbour distances, nothing capped: a dict with the largest `completed`,
+    `of_scale` and `of_value` errors over all queries, `of_value_asserted` (the largest of_value
+    error over the queries whose error exceeds RESOLUTION of the scale: the ones the of_value bar
+    is asserted on), `excused` (queries with a non-zero error within RESOLUTION of the scale, where
+    the reported value is a small difference of its terms), `of_value_excused` (the largest
+    of_value error among those) and `queries`."""
     qn = (queries.astype(np.float64) ** 2).sum(1)
     e = exp_kth.astype(np.float64)
     g = got_kth.astype(np.float64)
     finite = np.isfinite(e) & np.isfinite(g)
+    out = {"completed": 0.0, "of_scale": 0.0, "of_value": 0.0, "of_value_asserted": 0.0,
+           "of_value_excused": 0.0, "excused": 0, "queries": int(finite.sum())}
     if not finite.any():
-        return 0.0, 0.0, 0.0
+        return out
     e, g, qn = e[finite], g[finite], qn[finite]
     scale = np.abs(e) + qn
     diff = np.abs(g - e)
     with np.errstate(divide="ignore", invalid="ignore"):
         completed = np.where(e + qn > 0, diff / (e + qn), 0.0)
         of_scale = np.where(scale > 0, diff / scale, 0.0)
-        of_value = np.where((of_scale <= RESOLUTION) | (diff == 0), 0.0, diff / np.abs(e))
-        of_value = np.maximum(of_value, np.where(np.abs(e) > 0, np.minimum(diff / np.abs(e), REL), 0.0))
-    return float(completed.max()), float(of_value.max()), float(of_scale.max())
+        of_value = np.where(diff == 0, 0.0, diff / np.abs(e))
+    excused = (diff != 0) & (of_scale <= RESOLUTION) & (of_value > REL)
+    asserted = ~excused
+    out["completed"] = float(completed.max())
+    out["of_scale"] = float(of_scale.max())
+    out["of_value"] = float(of_value.max())
+    out["of_value_asserted"] = float(of_value[asserted].max()) if asserted.any() else 0.0
+    out["of_value_excused"] = float(of_value[excused].max()) if excused.any() else 0.0
+    out["excused"] = int(excused.sum())
+    return out
+
+
+def kth_errors(queries, exp_kth, got_kth):
+    """(completed, of_value over the queries the bar is asserted on, of_scale), nothing capped."""
+    d = kth_error_detail(queries, exp_kth, got_kth)
+    return d["completed"], d["of_value_asserted"], d["of_scale"]
 
 
 def assert_kth_distance(queries, exp_kth, got_kth, dim, what=""):
     """The k-th neighbour distances `got_kth` (partial distances, one per query) against the
-    oracle's `exp_kth`, to the bar described in the module docstring."""
-    completed, of_value, of_scale = kth_errors(queries, exp_kth, got_kth)
+    oracle's `exp_kth`, to the bar described in the module docstring: for dim < 16 a query passes
+    when its of_value error is <= REL or its of_scale error is <= RESOLUTION."""
+    d = kth_error_detail(queries, exp_kth, got_kth)
     key = "dim>=16" if dim >= STRICT_FROM_DIM else "dim<16"
-    seen = margins.setdefault(key, {"completed": 0.0, "of_value": 0.0, "of_scale": 0.0})
-    seen["completed"] = max(seen["completed"], completed)
-    seen["of_value"] = max(seen["of_value"], of_value)
-    seen["of_scale"] = max(seen["of_scale"], of_scale)
-    assert of_scale <= REL, (what, "of_scale", of_scale)
+    seen = margins.setdefault(key, {"completed": 0.0, "of_value": 0.0, "of_value_asserted": 0.0,
+                                    "of_value_excused": 0.0, "of_scale": 0.0, "excused": 0, "queries": 0})
+    for name in ("completed", "of_value", "of_value_asserted", "of_value_excused", "of_scale"):
+        seen[name] = max(seen[name], d[name])
+    seen["excused"] += d["excused"]
+    seen["queries"] += d["queries"]
+    assert d["of_scale"] <= REL, (what, "of_scale", d["of_scale"])
     if dim >= STRICT_FROM_DIM:
-        assert completed <= REL, (what, "completed distance", completed)
+        assert d["completed"] <= REL, (what, "completed distance", d["completed"])
     else:
-        assert of_value <= REL, (what, "of_value", of_value)
-    return completed, of_value, of_scale
+        assert d["of_value_asserted"] <= REL, (what, "of_value", d["of_value_asserted"])
+    return d["completed"], d["of_value_asserted"], d["of_scale"]

@@ -202,3 +202,25 @@ def test_shipped_optima_file():
     fused = [r for r in rows if r["algorithm"] == "fused-cache"]
     assert len(fused) == len(tuning.FUSED_SHAPES) * len(tuning.FUSED_DIMS) * len(tuning.FUSED_K_VALUES)
     assert tuning.config_algorithm("fused-cache", 8192, 32, 16) == (1, 1, 8, 4, 2)
+
+
+def test_entry_points_never_allocate_device_memory():
+    """The C ABI's contract: every entry point works on the caller's memory and allocates and frees
+    nothing (bitsknn_fused_l2_topk_f32_static in particular, which exists for callers that cannot
+    allocate).  No source of the library may name an allocating or freeing runtime call, and the
+    sources behind the static entry point no memset either (a memset node recorded into a captured
+    graph is not replayed reliably)."""
+    import glob
+    import re
+    csrc = os.path.join(ROOT, "bits-knn-jpdc2024_amd", "csrc")
+    sources = sorted(glob.glob(os.path.join(csrc, "*.hip")) + glob.glob(os.path.join(csrc, "*.hpp")))
+    assert len(sources) >= 10
+    forbidden = re.compile(r"\bhip(Malloc|Free|HostMalloc|HostFree|ExtMalloc|MallocAsync|FreeAsync|MallocManaged)\w*")
+    memset = re.compile(r"\bhipMemset\w*")
+    for path in sources:
+        with open(path) as handle:
+            text = handle.read()
+        assert forbidden.search(text) is None, (path, forbidden.search(text).group(0))
+        name = os.path.basename(path)
+        if name.startswith("fused") or name.startswith("topk_bits") or name in ("common.hpp", "bitonic_net.hpp"):
+            assert memset.search(text) is None, (path, memset.search(text).group(0))

@@ -47,6 +47,39 @@ def _check_topk_sample(torch, oracle, cache, m, sample, od, ol, k):
     assert np.array_equal(ol[sample].cpu().numpy(), el), "labels differ"
 
 
+# ---- config 1: the CPU reference's own case, 1024 x 65,536 from seed 24, k = 32 ----------------
+
+@pytest.mark.parametrize("block,batch,prefetch", [(256, 8, False), (128, 16, False), (512, 4, True)])
+def test_the_cpu_reference_matrix_through_the_hip_path(bk, dev, oracle, block, batch, prefetch):
+    """The matrix the CPU baseline is timed on (seeded generator of the reference, 1024 x 65,536,
+    k = 32) through bitsknn_topk_bits_f32, against the canonical oracle and against the restated
+    serial (reference src/topk/serial_knn.cpp:35-54: full sort of every row) and parallel
+    (src/topk/parallel_knn.cpp:30-65: OpenMP heap) selections.  Values bit for bit with all three;
+    labels bit for bit with the canonical oracle everywhere, and with the two restated CPU
+    selections on every row whose k + 1 smallest values are distinct (they order by distance
+    alone, so equal values may come out in either order there)."""
+    import torch
+    rows, cols, k = 1024, 65536, 32
+    m = oracle.uniform_matrix(24, rows, cols)
+    od, ol = bk.topk_bits(torch.from_numpy(m).to(dev), k, block, batch, prefetch)
+    torch.cuda.synchronize()
+    gd, gl = od.cpu().numpy(), ol.cpu().numpy()
+    ed, el = oracle.topk(m, k)
+    assert np.array_equal(gd.view(np.uint32), ed.view(np.uint32)), "values differ from the canonical oracle"
+    assert np.array_equal(gl, el), "labels differ from the canonical oracle"
+    sd, sl = oracle.topk_serial(m, k)
+    pd, pl, _ = oracle.topk_parallel(m, k, 8)
+    assert np.array_equal(gd.view(np.uint32), sd.view(np.uint32)), "values differ from serial_knn"
+    assert np.array_equal(gd.view(np.uint32), pd.view(np.uint32)), "values differ from parallel_knn"
+    smallest = np.sort(np.partition(m, k + 1, axis=1)[:, :k + 1], axis=1)
+    distinct = np.all(smallest[:, 1:] != smallest[:, :-1], axis=1)
+    assert distinct.sum() >= rows - 8, "seeded uniform rows should hardly ever tie among their smallest values"
+    assert np.array_equal(gl[distinct], sl[distinct]), "labels differ from serial_knn"
+    assert np.array_equal(gl[distinct], pl[distinct]), "labels differ from parallel_knn"
+    # the driver's checksum of query 0 (reference src/main.cpp:410-417)
+    assert oracle.checksum(gl[0]) == oracle.checksum(sl[0]) == oracle.checksum(pl[0])
+
+
 # ---- config 2: 1024 x 2^20 uniform rows -------------------------------------------------------
 
 @pytest.fixture(scope="module")

@@ -26,7 +26,7 @@ def _fused(bk, dev, points, queries, k, params=(8, 4, 2), bqd=1, dim_mult=1, wor
     pd = _dm(points, dev).reshape(points.shape[1], points.shape[0])
     qd = _dm(queries, dev).reshape(queries.shape[1], queries.shape[0])
     od, ol = bk.fused_l2_topk(qd, pd, k, params, bqd, dim_mult, workspace=workspace, arithmetic=arithmetic)
-    torch.cuda.synchronize()
+    bk.fused_status()  # synchronises; raises if a wave gave up a wait for a stage
     return od.cpu().numpy(), ol.cpu().numpy()
 
 
@@ -407,3 +407,53 @@ def test_bf16x3_is_as_accurate_as_the_fp32_matrix_instructions(bk, dev, oracle):
             err[(d, mode)] = float(np.max(np.abs(gd - at) / (np.abs(at) + qn)))
         assert err[(d, bk.FUSED_BF16X3)] < 1e-6
         assert err[(d, bk.FUSED_BF16X3)] < 4 * err[(d, bk.FUSED_FP32)] + 1e-7
+
+
+GIVE_UP_SCRIPT = r"""
+import sys
+sys.path[:0] = [{root!r}, {pkg!r}]
+import numpy as np
+import torch
+import bitsknn
+dev = torch.device("cuda:0")
+rng = np.random.default_rng(5)
+n, q, d, k = 100000, 1024, 8, 32
+points = torch.from_numpy(rng.random((d, n), dtype=np.float32)).to(dev)
+queries = torch.from_numpy(rng.random((d, q), dtype=np.float32)).to(dev)
+print("status before any call", flush=True)
+bitsknn.fused_status()
+print("fused call with a poll limit of 0", flush=True)
+od, ol = bitsknn.fused_l2_topk(queries, points, k)
+try:
+    bitsknn.fused_status()
+except bitsknn.BitsKnnError as error:
+    assert error.code == bitsknn.ERR_INTERNAL, error.code
+    assert "ran out of polls" in str(error), str(error)
+else:
+    raise SystemExit("no wait gave up although the poll limit is 0")
+kth = od[:, k - 1].cpu().numpy()
+assert np.isnan(kth).any(), "no list is marked"
+labels = ol.cpu().numpy()
+assert labels.min() >= 0 and labels.max() < n
+print("marked lists:", int(np.isnan(kth).sum()), "of", q, flush=True)
+bitsknn.fused_status()  # the check has cleared the word
+print("ok", flush=True)
+"""
+
+
+def test_a_wait_that_gives_up_is_reported(bk, dev):
+    """The failure path of the ring of stages, forced from the host: with BITSKNN_FUSED_POLL_LIMIT=0
+    (read once per process, hence the child process) every wait that finds its stage incomplete
+    gives up at once.  Every kernel still ends normally; the lists of the waves concerned end in
+    NaN, bitsknn_fused_status reports BITSKNN_ERR_INTERNAL once and is clear afterwards."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    pkg = os.path.join(root, "bits-knn-jpdc2024_amd")
+    env = dict(os.environ, BITSKNN_FUSED_POLL_LIMIT="0")
+    done = subprocess.run([sys.executable, "-u", "-c", GIVE_UP_SCRIPT.format(root=root, pkg=pkg)], env=env,
+                          capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, (done.stdout, done.stderr)
+    assert done.stdout.strip().endswith("ok"), done.stdout
+    bk.fused_status()  # this process, with the default limit, has seen no wait give up

@@ -46,6 +46,40 @@ def test_static_scratch_matches_the_workspace_entry_point(bk, dev, oracle):
     assert np.max(np.abs(got_d[:, k - 1] - exp_d[:, k - 1]) / scale) <= 1e-5
 
 
+def test_static_scratch_call_replayed_from_a_graph(bk, dev, oracle):
+    """The call is meant for code under HIP graph capture: after one eager call on the device (which
+    looks up the array's address and sets the kernels' LDS sizes), the same call is captured into a
+    graph and replayed several times with eager work and synchronisations in between; every replay
+    must give the workspace entry point's result bit for bit.  An allocation inside the library
+    (hipMalloc is not allowed while a stream is being captured) would fail the capture."""
+    import torch
+    n, q, d, k = 120000, 500, 16, 32
+    assert 0 < bk.fused_workspace_bytes(q, n, k) <= bk.fused_static_scratch_bytes()
+    points, queries = oracle.generate(77, n, q, d)
+    pd = torch.from_numpy(np.ascontiguousarray(points.T)).to(dev)
+    qd = torch.from_numpy(np.ascontiguousarray(queries.T)).to(dev)
+    want_d, want_l = bk.fused_l2_topk(qd, pd, k, workspace="auto")
+    torch.cuda.synchronize()
+    out_d = torch.empty((q, k), dtype=torch.float32, device=dev)
+    out_l = torch.empty((q, k), dtype=torch.int32, device=dev)
+    bk.fused_l2_topk(qd, pd, k, workspace="static", out_dist=out_d, out_label=out_l)  # eager warm-up
+    torch.cuda.synchronize()
+    assert torch.equal(out_d, want_d) and torch.equal(out_l, want_l)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        bk.fused_l2_topk(qd, pd, k, workspace="static", out_dist=out_d, out_label=out_l)
+    for replay in range(3):
+        out_d.fill_(-1.0)
+        out_l.fill_(-1)
+        # eager work on the same scratch memory between the replays: a smaller problem
+        bk.fused_l2_topk(qd[:, :100].contiguous(), pd[:, :50000].contiguous(), 16, workspace="static")
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_d, want_d) and torch.equal(out_l, want_l), replay
+    bk.fused_status()
+
+
 def test_static_scratch_rejects_problems_beyond_its_size(bk, dev):
     import torch
     q, n, k = 8192, 1 << 17, 256
