@@ -51,4 +51,5 @@ def pytest_sessionfinish(session, exitstatus):
     except ImportError:
         return
     for key, seen in sorted(parity.margins.items()):
-        print("\nparity margin %s: %s" % (key, ", ".join("%s %.3g" % kv for kv in sorted(seen.items()))))
+        print("\nparity margin %s: %s" % (key, ", ".join(
+            ("%s %d" if isinstance(kv[1], int) else "%s %.3g") % kv for kv in sorted(seen.items()))))

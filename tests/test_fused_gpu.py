@@ -433,8 +433,6 @@ else:
     raise SystemExit("no wait gave up although the poll limit is 0")
 kth = od[:, k - 1].cpu().numpy()
 assert np.isnan(kth).any(), "no list is marked"
-labels = ol.cpu().numpy()
-assert labels.min() >= 0 and labels.max() < n
 print("marked lists:", int(np.isnan(kth).sum()), "of", q, flush=True)
 bitsknn.fused_status()  # the check has cleared the word
 print("ok", flush=True)
