@@ -272,6 +272,7 @@ def leg_gemm(bitsknn, torch, timer, oracle, dev, steps, check, q=4096, n=1 << 20
     dist.fill_(-1.0)
     _, t_dist = timer.run(lambda: bitsknn.distances(queries, points, bitsknn.DIST_PARTIAL_L2, out=dist), steps, 2)
     _, t_topk = timer.run(lambda: bitsknn.topk_bits(dist, k, 256, 8, out_dist=out_d, out_label=out_l), steps, 2)
+    dist_rows = dist[sample_indices(q, 16)].clone()  # what the checks below look at
     tflops = 2.0 * q * n * d / t_dist / 1e12
     bytes_dist = 4.0 * q * n + 4.0 * (q + n) * d
     result = {"workload": f"GEMM distance + bits, {n} points x {q} queries, d={d}, k={k}",
@@ -289,12 +290,30 @@ def leg_gemm(bitsknn, torch, timer, oracle, dev, steps, check, q=4096, n=1 << 20
                                                "frac": bytes_dist / t_split / 1e9 / HBM_PEAK_GBS}},
               "selection_ms": t_topk * 1e3, "selection_elements_per_s": q * n / t_topk,
               "selection_frac": (4.0 * q * n + 8.0 * q * k) / t_topk / 1e9 / HBM_PEAK_GBS}
+    result["end_to_end_ms"] = (t_dist + t_topk) * 1e3
+    result["end_to_end_bf16x3_ms"] = (t_split + t_topk) * 1e3
+    # the same problem without the matrix: bits-fused through the entry point that cuts the points
+    # into ranges (4096 queries are 32 workgroups of 128 queries)
+    del dist
+    torch.cuda.empty_cache()
+    space = torch.empty(max(1, bitsknn.fused_workspace_bytes(q, n, k)), dtype=torch.uint8, device=dev)
+    alt_d = torch.full((q, k), -1.0, dtype=torch.float32, device=dev)
+    alt_l = torch.empty((q, k), dtype=torch.int32, device=dev)
+    _, t_fused = timer.run(lambda: bitsknn.fused_l2_topk(queries, points, k, out_dist=alt_d, out_label=alt_l,
+                                                         workspace=space), steps, 2)
+    fused_tflops = 2.0 * q * n * d / t_fused / 1e12
+    result["fused_alternative"] = {
+        "workload": f"bits-fused over ranges of points (workspace of {space.numel()} bytes), same {n} points x "
+                    f"{q} queries, d={d}, k={k}; no distance matrix",
+        "ms": t_fused * 1e3, "queries_per_s": q / t_fused,
+        "roofline": {"bound": "mfma", "achieved": fused_tflops, "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": fused_tflops / MFMA_F32_PEAK_TFLOPS}}
     if check:
         sample = sample_indices(q, 16)
         points_h = np.ascontiguousarray(points.cpu().numpy().T)
         queries_h = np.ascontiguousarray(queries[:, sample].cpu().numpy().T)
         part = oracle.dist(queries_h, points_h, "partial")
-        got_rows = dist[sample].cpu().numpy()
+        got_rows = dist_rows.cpu().numpy()
         qn = (queries_h.astype(np.float64) ** 2).sum(1)[:, None]
         matrix_err = float(np.max(np.abs(got_rows.astype(np.float64) - part) / (np.abs(part) + qn)))
         # the selection is exact on the matrix it was given ...
@@ -309,6 +328,10 @@ def leg_gemm(bitsknn, torch, timer, oracle, dev, steps, check, q=4096, n=1 << 20
         detail["selection_bit_exact_on_the_matrix"] = exact
         result["verified"] = bool(ok and exact and matrix_err <= REL)
         result["verification"] = detail
+        ok_alt, detail_alt = verify_neighbours(np, points_h, queries_h, exp_d, exp_l, alt_d[sample].cpu().numpy(),
+                                               alt_l[sample].cpu().numpy(), k)
+        result["fused_alternative"]["verified"] = bool(ok_alt)
+        result["fused_alternative"]["verification"] = detail_alt
     return result
 
 
@@ -352,7 +375,7 @@ def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=6553
             (grid if k in ks else long_lists).append(entry)
             if d == 32 and k == 32 and not workspace:
                 headline = {"workload": f"bits-fused, {n} points x {q} queries, d={d}, k={k}, fp32 uniform[0,1)",
-                            "arithmetic": "fp32 matrix instructions",
+                            "arithmetic": "fp32 matrix instructions", "launches_timed": steps,
                             "queries_per_s": q / seconds, "ms": seconds * 1e3, "pairs_per_s": q * n / seconds,
                             "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_F32_PEAK_TFLOPS,
                                          "unit": "TFLOP/s", "frac": tflops / MFMA_F32_PEAK_TFLOPS}}
@@ -417,6 +440,74 @@ def leg_cpu(rows, cols, k, budget_s=8.0):
             "serial": {"value": rows * cols / serial_s, "unit": "elements/s", "cores": 1,
                        "sample": f"one pass of serial_knn::selection restated (std::sort of every row) over "
                                  f"the same {rows}x{cols} matrix"}}
+
+
+def collect_verified(node, found):
+    """every `verified` flag anywhere in the result"""
+    if isinstance(node, dict):
+        for key, value in node.items():
+            if key == "verified":
+                found.append(bool(value))
+            else:
+                collect_verified(value, found)
+    elif isinstance(node, list):
+        for value in node:
+            collect_verified(value, found)
+    return found
+
+
+def summarise(result):
+    """The fractions of the roofline of every leg in a few hundred bytes, placed at the end of the
+    line: per list length the worst, best and tuned configuration of the sweep, the hard-input
+    cases, both kernels of the GEMM k-NN against both roofs, the fused grid, and whether every
+    comparison with the oracle passed."""
+    r3 = lambda x: round(float(x), 3)
+    out = {}
+    if "roofline" in result:
+        out["headline_frac"] = r3(result["roofline"]["frac"])
+    if "sweep" in result:
+        by_k = {}
+        for entry in result["sweep"]:
+            slot = by_k.setdefault(str(entry["k"]), {"min": 1e9, "max": 0.0})
+            if entry.get("tuned"):
+                slot["tuned"] = r3(entry["frac"])
+            else:
+                slot["min"] = min(slot["min"], r3(entry["frac"]))
+                slot["max"] = max(slot["max"], r3(entry["frac"]))
+        out["sweep_frac_hbm_by_k"] = by_k
+    if "hard_inputs" in result:
+        out["hard_inputs_frac_hbm"] = {
+            f"{e['rows']}_k{e['k']}{'_tuned' if e.get('tuned') else ''}": r3(e["frac"]) for e in result["hard_inputs"]}
+    if "gemm_knn" in result:
+        g = result["gemm_knn"]
+        out["gemm_knn"] = {"distance_frac_mfma": r3(g["distance_roofline"]["frac"]),
+                           "distance_frac_hbm": r3(g["distance_roofline"]["hbm_frac"]),
+                           "distance_bf16x3_frac_hbm": r3(g["distance_bf16x3"]["roofline"]["frac"]),
+                           "selection_frac_hbm": r3(g["selection_frac"]),
+                           "distance_ms": r3(g["distance_ms"]), "distance_bf16x3_ms": r3(g["distance_bf16x3"]["ms"]),
+                           "selection_ms": r3(g["selection_ms"]), "end_to_end_ms": r3(g["end_to_end_ms"]),
+                           "fused_alternative_ms": r3(g["fused_alternative"]["ms"]),
+                           "fused_alternative_frac_mfma": r3(g["fused_alternative"]["roofline"]["frac"])}
+    if "fused" in result:
+        f = result["fused"]
+        out["fused_grid_frac_mfma"] = {f"d{e['d']}_k{e['k']}": r3(e["frac"]) for e in f.get("grid", [])}
+        out["fused_grid_ms"] = {f"d{e['d']}_k{e['k']}": r3(e["ms"]) for e in f.get("grid", [])}
+        if "long_lists" in f:
+            out["fused_long_lists_frac_mfma"] = {f"d{e['d']}_k{e['k']}": r3(e["frac"]) for e in f["long_lists"]}
+        if "queries_per_s" in f:
+            out["fused_d32_k32"] = {"queries_per_s": round(f["queries_per_s"]), "frac_mfma": r3(f["roofline"]["frac"]),
+                                    "launches_timed": f.get("launches_timed")}
+            if "bf16x3" in f:
+                out["fused_d32_k32"]["bf16x3_queries_per_s"] = round(f["bf16x3"]["queries_per_s"])
+                out["fused_d32_k32"]["bf16x3_frac_bf16_mfma"] = r3(f["bf16x3"]["roofline"]["frac"])
+        if "few_queries" in f:
+            out["fused_few_queries_ms"] = {f"d{e['d']}_k{e['k']}": r3(e["ms"]) for e in f["few_queries"]["cases"]}
+    if "bits_sq" in result:
+        out["bits_sq_frac_hbm"] = {f"rows{e['rows']}_k{e['k']}": r3(e["frac"]) for e in result["bits_sq"]}
+    flags = collect_verified(result, [])
+    out["verified_checks"] = len(flags)
+    out["all_verified"] = bool(flags) and all(flags)
+    return out
 
 
 def main():
@@ -505,19 +596,25 @@ def main():
         dims = (args.fused_d,) if args.fused_d else (8, 16, 32)
         ks = (args.fused_k,) if args.fused_k else (4, 16, 32)
         whole = not args.fused_d and not args.fused_k
-        result["fused"] = leg_fused(bitsknn, torch, timer, oracle, dev, max(2, args.steps // 10), check, dims, ks,
+        result["fused"] = leg_fused(bitsknn, torch, timer, oracle, dev, max(5, args.steps // 4), check, dims, ks,
                                     long_ks=(64, 128, 256) if whole else ())
         if whole:
             # the reference's own fused shape with few queries (its plots: 8192 queries, 2^17 points):
             # the entry point with a workspace, which cuts the points into ranges
-            few = leg_fused(bitsknn, torch, timer, oracle, dev, max(2, args.steps // 4), check, (8,), (32,),
+            few = leg_fused(bitsknn, torch, timer, oracle, dev, max(5, args.steps // 4), check, (8,), (32,),
                             q=8192, n=1 << 17, long_ks=(64, 256), workspace=True)
             result["fused"]["few_queries"] = {"workload": few["workload"] + ", points cut into ranges (workspace)",
                                               "cases": few["grid"] + few["long_lists"]}
-
+        # no wave of any fused launch above gave up a wait for a stage
+        try:
+            bitsknn.fused_status()
+            result["fused"]["kernel_status"] = {"verified": True}
+        except bitsknn.BitsKnnError as error:
+            result["fused"]["kernel_status"] = {"verified": False, "message": str(error)}
         torch.cuda.empty_cache()
     if "cpu" in legs:
         result["cpu_baseline"] = leg_cpu(1024, 65536, 32)
+    result["summary"] = summarise(result)
     print(json.dumps(result))
 
 
