@@ -200,7 +200,7 @@ def distances(queries_dm, points_dm, op=DIST_L2, out=None):
     return out
 
 
-FUSED_FP32, FUSED_BF16X3 = 0, 1
+FUSED_FP32, FUSED_BF16X3, FUSED_EXACT = 0, 1, 2
 
 
 def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1, dim_mult=1,

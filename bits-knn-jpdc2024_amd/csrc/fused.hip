@@ -162,24 +162,24 @@ int first_radius_rank(int k, int scale)
     return rank <= longest ? rank : 0;
 }
 
-hipError_t launch_for_k(int k, const fused_args& a, bool split, hipStream_t stream)
+hipError_t launch_for_k(int k, const fused_args& a, int arith, hipStream_t stream)
 {
     switch (k)
     {
     case 4:
-        return launch_fused_k_4(a, split, stream);
+        return launch_fused_k_4(a, arith, stream);
     case 8:
-        return launch_fused_k_8(a, split, stream);
+        return launch_fused_k_8(a, arith, stream);
     case 16:
-        return launch_fused_k_16(a, split, stream);
+        return launch_fused_k_16(a, arith, stream);
     case 32:
-        return launch_fused_k_32(a, split, stream);
+        return launch_fused_k_32(a, arith, stream);
     case 64:
-        return launch_fused_k_64(a, split, stream);
+        return launch_fused_k_64(a, arith, stream);
     case 128:
-        return launch_fused_k_128(a, split, stream);
+        return launch_fused_k_128(a, arith, stream);
     default:
-        return launch_fused_k_256(a, split, stream);
+        return launch_fused_k_256(a, arith, stream);
     }
 }
 
@@ -235,7 +235,7 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     {
         return fail(BITSKNN_ERR_UNSUPPORTED, "Unsupported dimension: %d (at most 256)", dim);
     }
-    if (arithmetic != BITSKNN_FUSED_FP32 && arithmetic != BITSKNN_FUSED_BF16X3)
+    if (arithmetic != BITSKNN_FUSED_FP32 && arithmetic != BITSKNN_FUSED_BF16X3 && arithmetic != BITSKNN_FUSED_EXACT)
     {
         return fail(BITSKNN_ERR_INVALID, "bitsknn_fused_l2_topk_f32: unknown arithmetic %d", arithmetic);
     }
@@ -284,7 +284,9 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     a.split_points = ((n + splits - 1) / splits + 255) / 256 * 256;
 
     auto* hip_stream = static_cast<hipStream_t>(stream);
-    const bool split = arithmetic == BITSKNN_FUSED_BF16X3;
+    const int split = arithmetic == BITSKNN_FUSED_BF16X3 ? FUSED_ARITH_BF16X3
+                      : arithmetic == BITSKNN_FUSED_EXACT ? FUSED_ARITH_EXACT
+                                                          : FUSED_ARITH_MFMA_F32;
     // one bits pass over the splits*k candidates of every query, labels carried along
     auto reduce_ranges = [&]() -> int {
         const size_t cols = static_cast<size_t>(splits) * static_cast<size_t>(k);
@@ -346,7 +348,7 @@ extern "C" int bitsknn_fused_l2_topk_f32(const float* queries_dim_major,
                                          int dim_mult, void* stream)
 {
     return bitsknn::fused_impl(queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, k,
-                               query_reg, db_reg, dim_reg, block_query_dim, dim_mult, BITSKNN_FUSED_FP32,
+                               query_reg, db_reg, dim_reg, block_query_dim, dim_mult, BITSKNN_FUSED_EXACT,
                                nullptr, 0, false, stream);
 }
 
@@ -368,7 +370,7 @@ extern "C" int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major,
                                             size_t workspace_bytes, void* stream)
 {
     return bitsknn::fused_impl(queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, k,
-                               query_reg, db_reg, dim_reg, block_query_dim, dim_mult, BITSKNN_FUSED_FP32,
+                               query_reg, db_reg, dim_reg, block_query_dim, dim_mult, BITSKNN_FUSED_EXACT,
                                workspace, workspace_bytes, true, stream);
 }
 
@@ -395,7 +397,7 @@ extern "C" int bitsknn_fused_l2_topk_f32_static(const float* queries_dim_major,
     using namespace bitsknn;
     // parameter errors first, with the messages of the other entry points (no queries: validation only)
     const int valid = fused_impl(queries_dim_major, points_dim_major, dim, 0, n, out_dist, out_label, k,
-                                 query_reg, db_reg, dim_reg, block_query_dim, dim_mult, BITSKNN_FUSED_FP32,
+                                 query_reg, db_reg, dim_reg, block_query_dim, dim_mult, BITSKNN_FUSED_EXACT,
                                  nullptr, 0, false, stream);
     if (valid != BITSKNN_OK)
     {
@@ -423,7 +425,7 @@ extern "C" int bitsknn_fused_l2_topk_f32_static(const float* queries_dim_major,
     // The kernels write every entry of the partial lists they read back (ranges without points
     // included), so nothing in the scratch memory has to be cleared between calls.
     return fused_impl(queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, k, query_reg,
-                      db_reg, dim_reg, block_query_dim, dim_mult, BITSKNN_FUSED_FP32, workspace,
+                      db_reg, dim_reg, block_query_dim, dim_mult, BITSKNN_FUSED_EXACT, workspace,
                       workspace != nullptr ? STATIC_SCRATCH_BYTES : 0, workspace != nullptr, stream);
 }
 

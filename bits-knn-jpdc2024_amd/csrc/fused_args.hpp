@@ -16,6 +16,17 @@ constexpr int FQ_CAP = 32;                    // buffer slots per query (= point
                                               // that for long lists in few dimensions, 24 of them in
                                               // LDS where three stages have to fit (fused_geometry)
 
+// How the kernel computes: the arithmetic of the reported distances and how candidates are found.
+//  FUSED_ARITH_MFMA_F32  distances from fp32 matrix instructions, every pair of a tile
+//  FUSED_ARITH_BF16X3    distances from six bf16 matrix products of three pieces per operand
+//  FUSED_ARITH_EXACT     a lower bound of every distance from three bf16 matrix products of two
+//                        pieces per operand filters the tile; what passes is computed with
+//                        sequential fused multiply-adds in dimension order (the reference's
+//                        arithmetic), filtered again and appended (dimensions up to 64)
+constexpr int FUSED_ARITH_MFMA_F32 = 0;
+constexpr int FUSED_ARITH_BF16X3 = 1;
+constexpr int FUSED_ARITH_EXACT = 2;
+
 constexpr int FUSED_PLAIN = -1;
 constexpr int FUSED_REPEAT_MARKED = -2;
 constexpr int FUSED_FIRST_RADIUS_FROM = 0;
@@ -55,15 +66,15 @@ struct fused_args
     int poll_limit;
 };
 
-// one per compiled list length K (fused_inst.hip); split: products from three bf16 pieces per
-// operand where the dimension allows it
-hipError_t launch_fused_k_4(const fused_args& a, bool split, hipStream_t stream);
-hipError_t launch_fused_k_8(const fused_args& a, bool split, hipStream_t stream);
-hipError_t launch_fused_k_16(const fused_args& a, bool split, hipStream_t stream);
-hipError_t launch_fused_k_32(const fused_args& a, bool split, hipStream_t stream);
-hipError_t launch_fused_k_64(const fused_args& a, bool split, hipStream_t stream);
-hipError_t launch_fused_k_128(const fused_args& a, bool split, hipStream_t stream);
-hipError_t launch_fused_k_256(const fused_args& a, bool split, hipStream_t stream);
+// one per compiled list length K (fused_inst.hip); arith: one of FUSED_ARITH_*, used where the
+// dimension allows it (fp32 matrix instructions otherwise)
+hipError_t launch_fused_k_4(const fused_args& a, int arith, hipStream_t stream);
+hipError_t launch_fused_k_8(const fused_args& a, int arith, hipStream_t stream);
+hipError_t launch_fused_k_16(const fused_args& a, int arith, hipStream_t stream);
+hipError_t launch_fused_k_32(const fused_args& a, int arith, hipStream_t stream);
+hipError_t launch_fused_k_64(const fused_args& a, int arith, hipStream_t stream);
+hipError_t launch_fused_k_128(const fused_args& a, int arith, hipStream_t stream);
+hipError_t launch_fused_k_256(const fused_args& a, int arith, hipStream_t stream);
 
 } // namespace bitsknn
 

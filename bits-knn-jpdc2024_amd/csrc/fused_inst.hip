@@ -13,39 +13,47 @@ namespace bitsknn
 #define BITSKNN_CAT(a, b) a##b
 #define BITSKNN_CAT_EXPANDED(a, b) BITSKNN_CAT2(a, b)
 
-// split: the products of dimensions 9 .. 64 from three bf16 pieces per operand (below 9 the fp32
-// matrix instructions are as fast)
-hipError_t BITSKNN_CAT_EXPANDED(launch_fused_k_, BITSKNN_FUSED_K)(const fused_args& a, bool split,
+// FUSED_ARITH_BF16X3: dimensions 9 .. 64 (below 9 the fp32 matrix instructions are as fast);
+// FUSED_ARITH_EXACT: dimensions up to 64 (a stage holds the points twice, as fp32 rows and as bf16
+// pieces); everything else takes the fp32 matrix instructions
+hipError_t BITSKNN_CAT_EXPANDED(launch_fused_k_, BITSKNN_FUSED_K)(const fused_args& a, int arith,
                                                                   hipStream_t stream)
 {
     constexpr int K = BITSKNN_FUSED_K;
-    if (split && a.dim > 8 && a.dim <= 64)
+    if (arith == FUSED_ARITH_BF16X3 && a.dim > 8 && a.dim <= 64)
     {
-        return a.dim <= 16   ? launch_fused<K, 16, true>(a, stream)
-               : a.dim <= 32 ? launch_fused<K, 32, true>(a, stream)
-                             : launch_fused<K, 64, true>(a, stream);
+        return a.dim <= 16   ? launch_fused<K, 16, FUSED_ARITH_BF16X3>(a, stream)
+               : a.dim <= 32 ? launch_fused<K, 32, FUSED_ARITH_BF16X3>(a, stream)
+                             : launch_fused<K, 64, FUSED_ARITH_BF16X3>(a, stream);
+    }
+    if (arith == FUSED_ARITH_EXACT && a.dim <= 64)
+    {
+        return a.dim <= 8    ? launch_fused<K, 8, FUSED_ARITH_EXACT>(a, stream)
+               : a.dim <= 16 ? launch_fused<K, 16, FUSED_ARITH_EXACT>(a, stream)
+               : a.dim <= 32 ? launch_fused<K, 32, FUSED_ARITH_EXACT>(a, stream)
+                             : launch_fused<K, 64, FUSED_ARITH_EXACT>(a, stream);
     }
     if (a.dim <= 8)
     {
-        return launch_fused<K, 8, false>(a, stream);
+        return launch_fused<K, 8, FUSED_ARITH_MFMA_F32>(a, stream);
     }
     if (a.dim <= 16)
     {
-        return launch_fused<K, 16, false>(a, stream);
+        return launch_fused<K, 16, FUSED_ARITH_MFMA_F32>(a, stream);
     }
     if (a.dim <= 32)
     {
-        return launch_fused<K, 32, false>(a, stream);
+        return launch_fused<K, 32, FUSED_ARITH_MFMA_F32>(a, stream);
     }
     if (a.dim <= 64)
     {
-        return launch_fused<K, 64, false>(a, stream);
+        return launch_fused<K, 64, FUSED_ARITH_MFMA_F32>(a, stream);
     }
     if (a.dim <= 128)
     {
-        return launch_fused<K, 128, false>(a, stream);
+        return launch_fused<K, 128, FUSED_ARITH_MFMA_F32>(a, stream);
     }
-    return launch_fused<K, 256, false>(a, stream);
+    return launch_fused<K, 256, FUSED_ARITH_MFMA_F32>(a, stream);
 }
 
 } // namespace bitsknn

@@ -60,6 +60,56 @@ __device__ __forceinline__ float min3(float a, float b, float c)
     return r;
 }
 
+// the same, but a NaN operand gives a NaN
+__device__ __forceinline__ float minimum3(float a, float b, float c)
+{
+    float r;
+    asm("v_minimum3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+typedef __bf16 vbf16x2 __attribute__((ext_vector_type(2)));
+typedef float vfloat2 __attribute__((ext_vector_type(2)));
+
+// x[i] ~ x1 + x2 with two bf16 pieces rounded to nearest: x1 = bf16(x), x2 = bf16(x - x1) (the
+// difference is exact), so |x - x1 - x2| <= 2^-16 |x|.  Piece c of values 2j and 2j+1 shares word j
+// of pc (the layout of a matrix operand of 8 bf16 values).
+__device__ __forceinline__ void cut_bf16x2(const float (&x)[8], vuint4& p1, vuint4& p2)
+{
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        const vfloat2 pair{x[2 * j], x[2 * j + 1]};
+        const u32 first = __builtin_bit_cast(u32, __builtin_convertvector(pair, vbf16x2));
+        const vfloat2 rest{pair.x - __builtin_bit_cast(float, first << 16U),
+                           pair.y - __builtin_bit_cast(float, first & 0xFFFF0000U)};
+        p1[j] = first;
+        p2[j] = __builtin_bit_cast(u32, __builtin_convertvector(rest, vbf16x2));
+    }
+}
+
+// Error budget of the filter of FUSED_ARITH_EXACT.  For a query q and a point p let
+// V = fl(norm - 2 dot) be the reported value (sequential fused multiply-adds over the dimensions in
+// order) and W the filter's value: the sum, on the bf16 matrix instructions with fp32 accumulation,
+// of the lowered norm's two pieces and of the products of the pieces of -2q and p with the
+// second-order terms left out.  With Q = ||q||^2, N = ||p||^2, S = N + 2 sum |q_i p_i| <= 2 N + Q:
+//   |V - exact|          <= (d + 2) 2^-24 S                      (d <= 64: 4.0e-6 S)
+//   pieces left out      <= 3 * 2^-16 (1 + 2^-7) * 2 sum |q_i p_i|            (4.7e-5 S)
+//   accumulation in W    <= 17 * 2^-23 per matrix instruction, at most 13     (2.7e-5 S, allowing
+//                           for truncating adds of every term)
+// together below FILTER_REL = 2^-13 (1.22e-4) of S with a factor of 1.5 to spare.  The norm pieces
+// hold at most N (1 - NORM_LOWER) (1 + 2^-15.3) (cutting, the order of the staging threads' sums, one
+// rounding), and NORM_LOWER = 2^-12 + 2^-14 >= 2 FILTER_REL + 2^-15.3, so that
+//   W <= V + FILTER_REL * Q        whenever V is finite,
+// and a pair can only have V < radius if W < radius + FILTER_REL * Q.  The compare is written so
+// that a NaN in W passes; FILTER_ABS covers products of pieces that underflow.
+constexpr float FILTER_REL = 0x1.0p-13F;
+constexpr float NORM_LOWER = 0x1.4p-12F;
+constexpr float FILTER_ABS = 0x1.0p-100F;
+// norm of the points beyond the end of a range: the largest finite bf16, so that they only pass the
+// filter while a radius is still infinite (what passes is checked against the range again)
+constexpr u32 BF16_HUGE = 0x7F7FU;
+
 // Stage geometry by padded dimension DP.
 //
 // SPLIT = false: fp32 matrix instructions; a stage is (DP + norm rows) x PT floats, PT points per
@@ -80,23 +130,34 @@ __device__ __forceinline__ float min3(float a, float b, float c)
 // a sample; at k = 64 the smaller stages cost more than the merges save).  WIDE_OK is set for
 // launches over ranges only (see launch_fused).
 constexpr int RING_MAX_DP = 128; // largest padded dimension that takes the ring of stages
+constexpr int FQ_XCHG = 96;      // words a wave has for the exchange at a merge: 32 radii, fills, labels
 
-template <int DP, bool SPLIT, int K, bool WIDE_OK = false>
+template <int DP, int ARITH, int K, bool WIDE_OK = false>
 struct fused_geometry
 {
-    static constexpr bool WIDE = WIDE_OK && K >= 128 && DP <= 16 && !SPLIT;
+    static constexpr bool SPLIT = ARITH == FUSED_ARITH_BF16X3;
+    static constexpr bool EXACT = ARITH == FUSED_ARITH_EXACT;
+    static constexpr bool WIDE = WIDE_OK && K >= 128 && DP <= 16 && ARITH == FUSED_ARITH_MFMA_F32;
     static constexpr int CAP = WIDE ? 2 * FQ_CAP : FQ_CAP; // buffer slots per query
-    static constexpr int DK = DP < 16 ? 16 : DP;       // SPLIT: dimensions padded to whole matrix steps
-    static constexpr int KB = DK / 16;                 // SPLIT: matrix steps of 16 dimensions
-    static constexpr int KS = DK / 8;                  // SPLIT: cells of 8 dimensions per point and piece
-    static constexpr int PT = SPLIT  ? (DK <= 16 ? 128 : (DK <= 32 ? 64 : 32))
-                              : WIDE ? (DP <= 8 ? 128 : 64)
-                                     : (DP <= 16 ? 256 : (DP <= 32 ? 128 : (DP <= 64 ? 64 : 32)));
+    static constexpr int DK = DP < 16 ? 16 : DP;       // SPLIT, EXACT: dimensions padded to whole matrix steps
+    static constexpr int KB = DK / 16;                 // SPLIT, EXACT: matrix steps of 16 dimensions
+    static constexpr int KS = DK / 8;                  // SPLIT, EXACT: cells of 8 dimensions per point and piece
+    // EXACT: a stage holds the points as fp32 rows (for the sequential arithmetic of what passes the
+    // filter) and as 16-byte cells of bf16 pieces (the A operands of the filter's matrix
+    // instructions): two pieces per value and a cell with two pieces of the lowered norm.  Up to 8
+    // dimensions a point is three cells, (piece 1 | piece 2 | norm), used as the two halves of the
+    // 16 matrix dimensions.
+    static constexpr int CELLS = EXACT ? (DP <= 8 ? 3 : 2 * KS + 1) : 0;
+    static constexpr int PT = SPLIT   ? (DK <= 16 ? 128 : (DK <= 32 ? 64 : 32))
+                              : EXACT ? (DP <= 16 ? 128 : (DP <= 32 ? 64 : 32))
+                              : WIDE  ? (DP <= 8 ? 128 : 64)
+                                      : (DP <= 16 ? 256 : (DP <= 32 ? 128 : (DP <= 64 ? 64 : 32)));
     // threads per point when staging.  The small stages of the 64-slot geometry are staged by their
     // first PT threads, a whole point each, so that the norm of a point is one row and can be the
     // initial accumulator as in the 32-slot geometry (same terms in the same order: both
-    // geometries give the same bits).
-    static constexpr int TPP = WIDE ? 1 : FQ_THREADS / PT;
+    // geometries give the same bits).  EXACT: a thread carries 8 consecutive dimensions of a point
+    // (4 in up to 8 dimensions), as with bf16x3 products.
+    static constexpr int TPP = EXACT ? FQ_THREADS / PT : (WIDE ? 1 : FQ_THREADS / PT);
     static constexpr int STAGERS = SPLIT ? FQ_THREADS : TPP * PT; // threads that stage
     // point rows (zero beyond dim), then one row per staging thread of a point with its share of
     // ||p||^2 (at least two rows, so that the row count is even)
@@ -106,13 +167,15 @@ struct fused_geometry
     // (not for lists of 128 entries in 32 dimensions: that instantiation then needs 260 vector
     // registers, 4 more than two waves per SIMD leave it)
     static constexpr bool PAIRED =
-        !SPLIT && !WIDE && (TPP == 2 || TPP == 4) && PT >= 64 && !(DP == 32 && K == 128);
+        !SPLIT && !EXACT && !WIDE && (TPP == 2 || TPP == 4) && PT >= 64 && !(DP == 32 && K == 128);
     static constexpr int NORM_ROWS = (!SPLIT && (TPP == 1 || PAIRED) && PT >= 64) ? 1 : (TPP > 2 ? TPP : 2);
     static constexpr int ROWS = DP + NORM_ROWS;
     static constexpr int STEPS = ROWS / 2;    // MFMA steps of 2 rows
     static constexpr int VPT = SPLIT ? 8 : DP / TPP; // values a thread carries from global memory to LDS
     static constexpr int MT = PT / 32;        // MFMA row tiles per stage
-    static constexpr int STAGE_FLOATS = SPLIT ? 3 * KS * PT * 4 + PT : ROWS * PT;
+    static constexpr int STAGE_FLOATS = SPLIT   ? 3 * KS * PT * 4 + PT
+                                        : EXACT ? DP * PT + CELLS * PT * 4
+                                                : ROWS * PT;
     // Stages in LDS: two, with a barrier per stage (one being multiplied, one being filled), or a
     // ring of three without barriers, in which a wave that appends or merges holds up the others
     // only once it is a whole stage behind (see the stage loop of the kernel).  Two workgroups per
@@ -142,21 +205,26 @@ struct fused_geometry
     static constexpr int NB = RING ? 3 : 2;
     static constexpr int SLOTS = RING && !SPLIT && DP >= 16 ? 24 : CAP; // slots a query buffer has in LDS
     static_assert(!SPLIT || (DP <= 64 && TPP == KS), "one staging thread per point and cell");
+    static_assert(!EXACT || (DP <= 64 && VPT == (DP <= 8 ? 4 : 8) && PT <= 128),
+                  "the stages of the exact arithmetic serve up to 64 dimensions, in at most four tiles");
     static constexpr size_t lds_bytes()
     {
         // the stages, the query buffers, exchange slots, merge flags and stage counters
         return NB * static_cast<size_t>(STAGE_FLOATS) * sizeof(float) +
                static_cast<size_t>(FQ_WAVES) * FQ_QW * SLOTS * sizeof(u64) +
-               static_cast<size_t>(FQ_WAVES) * WAVE * sizeof(float) + 8 * sizeof(int);
+               static_cast<size_t>(FQ_WAVES) * FQ_XCHG * sizeof(float) + 8 * sizeof(int);
     }
+    static_assert(!EXACT || lds_bytes() <= 80 * 1024, "two workgroups per compute unit");
 };
 
 // K: list length.  DP: dimension padded to 8, 16, 32, 64, 128 or 256 (padding rows are zero on
 // both sides of the product).
-template <int K, int DP, bool SPLIT, bool WIDE_OK>
+template <int K, int DP, int ARITH, bool WIDE_OK>
 __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 {
-    using G = fused_geometry<DP, SPLIT, K, WIDE_OK>;
+    using G = fused_geometry<DP, ARITH, K, WIDE_OK>;
+    constexpr bool SPLIT = G::SPLIT;
+    constexpr bool EXACT = G::EXACT;
     constexpr int PT = G::PT;
     constexpr int CAP = G::CAP;
     constexpr int SLOTS = G::SLOTS;
@@ -192,8 +260,8 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     constexpr bool RING = G::RING;
     constexpr int NB = G::NB;
     u64* const buffers = reinterpret_cast<u64*>(lds + NB * STAGE_FLOATS);          // [waves][32][SLOTS]
-    float* const xchg = reinterpret_cast<float*>(buffers + FQ_WAVES * FQ_QW * SLOTS);  // [waves][64]
-    int* const merge_wanted = reinterpret_cast<int*>(xchg + FQ_WAVES * WAVE);           // [3]
+    float* const xchg = reinterpret_cast<float*>(buffers + FQ_WAVES * FQ_QW * SLOTS);  // [waves][96]
+    int* const merge_wanted = reinterpret_cast<int*>(xchg + FQ_WAVES * FQ_XCHG);        // [3]
     int* const ready = merge_wanted + 4;   // [3] waves that have written their part, per ring slot
 
     const int dim = a.dim;
@@ -210,14 +278,69 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     const int wave_q0 = static_cast<int>(blockIdx.x) * FQ_QB + wave * FQ_QW;
     const int my_q = wave_q0 + ql;
     u64* const wbuf = buffers + static_cast<size_t>(wave) * FQ_QW * SLOTS;
-    float* const wx = xchg + wave * WAVE;     // 32 radii, then 32 fills (as int bits)
+    float* const wx = xchg + wave * FQ_XCHG;  // 32 radii, then 32 fills (as int bits), then the
+                                              // labels of the radii (EXACT)
 
     // query fragment: step s of this lane is row 2s + half, times -2 (the stages hold the plain
     // point values); the norm rows are multiplied by 1
-    float qf[SPLIT ? 1 : STEPS];
+    float qf[SPLIT || EXACT ? 1 : STEPS];
     // SPLIT: the three bf16 pieces of -2q for the 8 dimensions 16*kb + 8*half .. + 7 of step kb
-    vuint4 qs[SPLIT ? 3 : 1][SPLIT ? KB : 1];
-    if constexpr (SPLIT)
+    // EXACT: two pieces; up to 8 dimensions qs[0][0] is piece 1 of dimensions 0 .. 7 in both halves
+    // of the wave and qs[1][0] piece 2 in the first half, (1, 1, 0, ...) for the norm cell in the
+    // second; from 16 dimensions on qs[2][0] is the norm cell's (1, 1, 0, ...) in the first half
+    vuint4 qs[SPLIT || EXACT ? 3 : 1][SPLIT || EXACT ? KB : 1];
+    // EXACT: the query itself, every dimension, for the sequential arithmetic; the slack of its
+    // filter threshold above the radius
+    float qx[EXACT ? DP : 1];
+    float filter_slack = 0.0F;
+    float thr = __builtin_inff();    // EXACT: what a filter value must not exceed to be looked at
+    int radius_label = 0x7FFFFFFF;   // EXACT: label of the list entry the radius comes from
+    qx[0] = 0.0F;
+    if constexpr (EXACT)
+    {
+        float qq = 0.0F;
+        // (every load from a valid address, so that they are all in flight together)
+        const bool live = my_q < a.q;
+        const float* const mine = a.queries + (live ? my_q : 0);
+#pragma unroll
+        for (int dd = 0; dd < DP; ++dd)
+        {
+            const float x = mine[static_cast<size_t>(dd < dim ? dd : 0) * a.q];
+            qx[dd] = dd < dim && live ? x : 0.0F;
+        }
+#pragma unroll
+        for (int dd = 0; dd < DP; ++dd)
+        {
+            qq = __builtin_fmaf(qx[dd], qx[dd], qq);
+        }
+        filter_slack = FILTER_REL * qq * (1.0F + 0x1.0p-20F) + FILTER_ABS * (1.0F + qq);
+        const vuint4 ones{0x3F803F80U, 0, 0, 0};
+        const vuint4 zeros{0, 0, 0, 0};
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+        {
+            float val[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+            {
+                // (a select between registers: the query is not indexed by the lane)
+                const int first = DP <= 8 ? j : 16 * kb + j;
+                const int second = DP <= 8 ? j : 16 * kb + 8 + j;
+                float lower = qx[first];
+                float upper = qx[second < DP ? second : 0];
+                asm volatile("" : "+v"(lower), "+v"(upper));
+                val[j] = -2.0F * (half != 0 ? upper : lower);
+            }
+            cut_bf16x2(val, qs[0][kb], qs[1][kb]);
+            qs[2][kb] = half == 0 ? ones : zeros;
+        }
+        if constexpr (DP <= 8)
+        {
+            qs[1][0] = half == 0 ? qs[1][0] : ones;
+        }
+        qf[0] = 0.0F;
+    }
+    else if constexpr (SPLIT)
     {
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
@@ -403,6 +526,10 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 if (i == K - 1)
                 {
                     wx[qm] = key_value(list[r]);
+                    if constexpr (EXACT)
+                    {
+                        reinterpret_cast<int*>(wx)[64 + qm] = key_label(list[r]);
+                    }
                 }
             }
         }
@@ -411,6 +538,14 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         // (a first radius from a sample stays until the list has a smaller one)
         radius = fminf(wx[ql], first_radius);
+        if constexpr (EXACT)
+        {
+            // (the slack also covers the rounding of this sum)
+            thr = radius + (filter_slack + 0x1.0p-22F * __builtin_fabsf(radius));
+            // a value equal to the radius passes if its label is below the label of the list's last
+            // entry (every label where the radius is a first radius from a sample)
+            radius_label = wx[ql] < first_radius ? reinterpret_cast<const int*>(wx)[64 + ql] : 0x7FFFFFFF;
+        }
         fill = 0;
         have_list = true;
         merged = true;
@@ -546,9 +681,9 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     // are neighbouring lanes, which add up their shares of the norm among themselves
     // SPLIT: thread t carries the 8 dimensions 8*(t % TPP) .. + 7 of point t / TPP (neighbouring
     // lanes as well)
-    const int sp = SPLIT || G::PAIRED ? t / TPP : t % PT;
-    const int sd0 = SPLIT ? 8 * (t % TPP) : (G::PAIRED ? t % TPP : t / PT);
-    auto dim_of = [&](int i) -> int { return SPLIT ? sd0 + i : sd0 + TPP * i; };
+    const int sp = SPLIT || EXACT || G::PAIRED ? t / TPP : t % PT;
+    const int sd0 = SPLIT || EXACT ? VPT * (t % TPP) : (G::PAIRED ? t % TPP : t / PT);
+    auto dim_of = [&](int i) -> int { return SPLIT || EXACT ? sd0 + i : sd0 + TPP * i; };
     float pre[VPT];
     // Point values are read with buffer loads: a constant byte offset per value and lane (beyond
     // the resource for dimensions dim .. DP-1, which then read as zero; the hardware checks the
@@ -627,7 +762,70 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             }
         }
         float share = 0.0F;
-        if constexpr (SPLIT)
+        if constexpr (EXACT)
+        {
+            // fp32 rows for the sequential arithmetic, then the cells of bf16 pieces
+            float eight[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+            {
+                eight[i] = i < VPT ? pre[i < VPT ? i : 0] : 0.0F;
+            }
+            vuint4 piece[2];
+            cut_bf16x2(eight, piece[0], piece[1]);
+#pragma unroll
+            for (int i = 0; i < VPT; ++i)
+            {
+                share = __builtin_fmaf(pre[i], pre[i], share);
+                stage[(sd0 + i) * PT + sp] = pre[i];
+            }
+            constexpr int PIECE2 = DP <= 8 ? 1 : KS; // first cell of the second pieces
+            if constexpr (VPT == 8)
+            {
+                vuint4* const cells = reinterpret_cast<vuint4*>(stage + DP * PT);
+                const int ks = sd0 / 8;
+                cells[ks * PT + sp] = piece[0];
+                cells[(PIECE2 + ks) * PT + sp] = piece[1];
+            }
+            else
+            {
+                // half a cell per thread
+                typedef u32 vuint2 __attribute__((ext_vector_type(2)));
+                vuint2* const halves = reinterpret_cast<vuint2*>(stage + DP * PT);
+                const int h = sd0 / 4;
+                halves[2 * sp + h] = vuint2{piece[0][0], piece[0][1]};
+                halves[2 * (PIECE2 * PT + sp) + h] = vuint2{piece[1][0], piece[1][1]};
+            }
+            // the threads of a point are TPP neighbouring lanes
+            if constexpr (TPP >= 2)
+            {
+                share += __builtin_bit_cast(float, lane_xor32<1>(__builtin_bit_cast(u32, share)));
+            }
+            if constexpr (TPP >= 4)
+            {
+                share += __builtin_bit_cast(float, lane_xor32<2>(__builtin_bit_cast(u32, share)));
+            }
+            if constexpr (TPP == 8)
+            {
+                share += __builtin_bit_cast(float, lane_xor32<4>(__builtin_bit_cast(u32, share)));
+            }
+            if (sd0 == 0)
+            {
+                // the lowered norm in two pieces; points beyond the end only pass an infinite radius
+                const float lowered = __builtin_fmaf(-NORM_LOWER, share, share);
+                const vfloat2 whole{lowered, 0.0F};
+                const u32 first = __builtin_bit_cast(u32, __builtin_convertvector(whole, vbf16x2)) & 0xFFFFU;
+                const vfloat2 rest{lowered - __builtin_bit_cast(float, first << 16U), 0.0F};
+                const u32 second = __builtin_bit_cast(u32, __builtin_convertvector(rest, vbf16x2)) & 0xFFFFU;
+                vuint4 cell{first | (second << 16U), 0, 0, 0};
+                if (!(base + sp < n))
+                {
+                    cell[0] = BF16_HUGE;
+                }
+                reinterpret_cast<vuint4*>(stage + DP * PT)[(G::CELLS - 1) * PT + sp] = cell;
+            }
+        }
+        else if constexpr (SPLIT)
         {
 #pragma unroll
             for (int i = 0; i < 8; ++i)
@@ -684,9 +882,191 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         }
     };
 
+    // ---- EXACT: the candidates of a stage.  `cand` has bit 16 * tile + r set where filter value r
+    // of this lane in that tile of the stage is not above the lane's threshold.  Every lane works
+    // through its own bits, lowest first: it computes the distance of its query to that point with
+    // sequential fused multiply-adds over the dimensions in order -- norm and dot product, then
+    // norm - 2 dot: the reference's arithmetic (include/bits/topk/singlepass/
+    // fused_cache_kernel_structs.cuh:457-522, :622-631) -- and appends it if its key is below the
+    // key of the list's last entry.  (The full key: the lanes of a query take its points out of
+    // index order, and a merge may fall between two of them.)  `base` is the stage's first point.
+    auto exact_candidates = [&](u64 cand, const float* stage, int base) __attribute__((always_inline)) {
+        while (__builtin_amdgcn_ballot_w64(cand != 0) != 0)
+        {
+            // an iteration brings a query at most two values
+            if (__builtin_amdgcn_ballot_w64(fill + 2 > SLOTS) != 0)
+            {
+                if (JOIN_MERGES && lane == 0)
+                {
+                    __hip_atomic_store(merge_wanted + stage_slot, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+                merge_event();
+            }
+            const bool has = cand != 0;
+            const int r = has ? __builtin_ctzll(cand) : 0;
+            cand &= cand - 1;
+            const int local = 32 * (r >> 4) + 8 * ((r >> 2) & 3) + 4 * half + (r & 3);
+            const float* const column = stage + local;
+            float norm = 0.0F;
+            float dot = 0.0F;
+#pragma unroll
+            for (int dd = 0; dd < DP; ++dd)
+            {
+                const float x = column[dd * PT];
+                norm = __builtin_fmaf(x, x, norm);
+                dot = __builtin_fmaf(qx[dd], x, dot);
+            }
+            const float value = __builtin_fmaf(-2.0F, dot, norm);
+            const int label = base + local;
+            const bool below = has && label < n && (value < radius || (value == radius && label < radius_label));
+            const u64 pass = __builtin_amdgcn_ballot_w64(below);
+            if (pass != 0)
+            {
+                const int mine = below ? 1 : 0;
+                const int other = static_cast<int>((pass >> (static_cast<unsigned>(lane) ^ 32U)) & 1U);
+                if (below)
+                {
+                    wbuf[ql * SLOTS + fill + (half != 0 ? other : 0)] = make_key(value, label);
+                }
+                fill += mine + other;
+            }
+        }
+    };
+    // the filter of a tile: the smallest of the 16 values of every lane (a NaN if there is one)
+    auto smallest_of = [&](const vfloat16& w) __attribute__((always_inline)) -> float {
+        float low[5];
+#pragma unroll
+        for (int g = 0; g < 5; ++g)
+        {
+            low[g] = minimum3(w[3 * g], w[3 * g + 1], w[3 * g + 2]);
+        }
+        return minimum3(minimum3(low[0], low[1], low[2]), low[3], low[4]);
+    };
+    // bit r where value r of this lane is not above the threshold (negated compare: a NaN counts)
+    auto bits_of = [&](const vfloat16& w) __attribute__((always_inline)) -> u32 {
+        u32 bits = 0;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+        {
+            bits |= !(w[r] > thr) ? 1U << r : 0U;
+        }
+        return bits;
+    };
+
     // all row tiles of a stage: distances, filter, append
     auto multiply = [&](const float* stage, int base) {
-        if constexpr (SPLIT)
+        if constexpr (EXACT)
+        {
+            const vuint4* const cells = reinterpret_cast<const vuint4*>(stage + DP * PT);
+            vfloat16 zero;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+            {
+                zero[r] = 0.0F;
+            }
+            // the filter values of one tile: lowered norm - 2 q.p from the pieces
+            auto filter_values = [&](int local0) __attribute__((always_inline)) -> vfloat16 {
+                const vuint4* const mine = cells + local0 + ql;
+                vfloat16 acc;
+                if constexpr (DP <= 8)
+                {
+                    // first half of the wave: piece 1 of the point against pieces 1 and 2 of the
+                    // query; second half: piece 2 against piece 1, the norm cell against (1, 1)
+                    const vuint4 a0 = mine[(half != 0 ? 1 : 0) * PT];
+                    const vuint4 a1 = mine[(half != 0 ? 2 : 0) * PT];
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(vbf16x8, a0), __builtin_bit_cast(vbf16x8, qs[0][0]), zero, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(vbf16x8, a1), __builtin_bit_cast(vbf16x8, qs[1][0]), acc, 0, 0, 0);
+                }
+                else
+                {
+                    vuint4 p1[KB];
+                    vuint4 p2[KB];
+#pragma unroll
+                    for (int kb = 0; kb < KB; ++kb)
+                    {
+                        p1[kb] = mine[(2 * kb + half) * PT];
+                        p2[kb] = mine[(KS + 2 * kb + half) * PT];
+                    }
+                    const vuint4 nn = mine[2 * KS * PT];
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(vbf16x8, nn), __builtin_bit_cast(vbf16x8, qs[2][0]), zero, 0, 0, 0);
+                    static_for<0, KB>([&](auto kb_tag) {
+                        constexpr int kb = decltype(kb_tag)::value;
+                        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(vbf16x8, p2[kb]), __builtin_bit_cast(vbf16x8, qs[0][kb]), acc, 0, 0, 0);
+                        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(vbf16x8, p1[kb]), __builtin_bit_cast(vbf16x8, qs[1][kb]), acc, 0, 0, 0);
+                        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(vbf16x8, p1[kb]), __builtin_bit_cast(vbf16x8, qs[0][kb]), acc, 0, 0, 0);
+                    });
+                }
+                return acc;
+            };
+            // First every tile of the stage is filtered without a branch: which pairs of tiles hold
+            // a value to look at is noted in `flagged` (wave-uniform).  Then the filter values of the
+            // flagged pairs are computed again (a few matrix instructions) to find the lanes and
+            // rows, and the candidates of the whole stage are worked through together.
+            constexpr int TILES = MT >= 2 ? 2 : 1;
+            constexpr int PAIRS = MT / TILES;
+            u32 flagged = 0;
+            vfloat16 w0;
+            vfloat16 w1;
+            static_for<0, PAIRS>([&](auto p_tag) {
+                constexpr int p = decltype(p_tag)::value;
+                w0 = filter_values(p * 64);
+                if constexpr (TILES == 2)
+                {
+                    w1 = filter_values(p * 64 + 32);
+                }
+                // The first read of the tiles is a compare the compiler sees, so that it places the
+                // wait states a matrix result needs before it; assembly operands are not covered by
+                // that hazard handling.
+                const u64 last_passes =
+                    __builtin_amdgcn_ballot_w64(!(w0[15] > thr) || (TILES == 2 && !(w1[15] > thr)));
+                __builtin_amdgcn_sched_barrier(0);
+                float smallest = smallest_of(w0);
+                if constexpr (TILES == 2)
+                {
+                    const float second = smallest_of(w1);
+                    smallest = minimum3(smallest, second, second);
+                }
+                flagged |= (last_passes | __builtin_amdgcn_ballot_w64(!(smallest > thr))) != 0 ? 1U << p : 0U;
+            });
+            if (flagged != 0)
+            {
+                u64 cand = 0;
+                if constexpr (PAIRS == 1)
+                {
+                    cand = bits_of(w0);
+                    if constexpr (TILES == 2)
+                    {
+                        cand |= static_cast<u64>(bits_of(w1)) << 16U;
+                    }
+                }
+                else
+                {
+                    static_assert(PAIRS == 2 && TILES == 2);
+                    u32 part[2] = {0, 0};
+#pragma unroll 1
+                    for (int p = 0; p < 2; ++p)
+                    {
+                        if ((flagged >> p & 1U) != 0)
+                        {
+                            w0 = filter_values(p * 64);
+                            w1 = filter_values(p * 64 + 32);
+                            const u32 bits = bits_of(w0) | (bits_of(w1) << 16U);
+                            part[0] = p == 0 ? bits : part[0];
+                            part[1] = p == 1 ? bits : part[1];
+                        }
+                    }
+                    cand = static_cast<u64>(part[0]) | (static_cast<u64>(part[1]) << 32U);
+                }
+                exact_candidates(cand, stage, base);
+            }
+        }
+        else if constexpr (SPLIT)
         {
             constexpr int PAIRS = MT / 2;
             const vuint4* const cells = reinterpret_cast<const vuint4*>(stage);
@@ -1042,15 +1422,15 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     }
 }
 
-template <int K, int DP, bool SPLIT, bool WIDE_OK>
+template <int K, int DP, int ARITH, bool WIDE_OK>
 hipError_t launch_fused_as(const fused_args& a, hipStream_t stream)
 {
-    using G = fused_geometry<DP, SPLIT, K, WIDE_OK>;
+    using G = fused_geometry<DP, ARITH, K, WIDE_OK>;
     constexpr size_t lds_bytes = G::lds_bytes();
     if (lds_bytes > 48 * 1024)
     {
         const hipError_t status =
-            hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<K, DP, SPLIT, WIDE_OK>),
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<K, DP, ARITH, WIDE_OK>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
         if (status != hipSuccess)
         {
@@ -1067,7 +1447,7 @@ hipError_t launch_fused_as(const fused_args& a, hipStream_t stream)
         args.split_points = (args.visit + 255) / 256 * 256;
     }
     const unsigned grid = static_cast<unsigned>((a.q + FQ_QB - 1) / FQ_QB);
-    hipLaunchKernelGGL((fused_kernel<K, DP, SPLIT, WIDE_OK>), dim3(grid, static_cast<unsigned>(a.splits)),
+    hipLaunchKernelGGL((fused_kernel<K, DP, ARITH, WIDE_OK>), dim3(grid, static_cast<unsigned>(a.splits)),
                        dim3(FQ_THREADS), lds_bytes, stream, args);
     return hipGetLastError();
 }
@@ -1077,17 +1457,17 @@ hipError_t launch_fused_as(const fused_args& a, hipStream_t stream)
 // points, k = 128: d = 8 19.5 ms with 64 slots, 17.3 ms with 32; d = 16 32.2 / 24.9 ms); over ranges
 // the lists hardly converge and the merges weigh more (8192 queries x 2^17 points, d = 8, k = 256:
 // 2.19 ms with 32 slots, 1.60 ms with 64).
-template <int K, int DP, bool SPLIT>
+template <int K, int DP, int ARITH>
 hipError_t launch_fused(const fused_args& a, hipStream_t stream)
 {
-    if constexpr (fused_geometry<DP, SPLIT, K, true>::WIDE)
+    if constexpr (fused_geometry<DP, ARITH, K, true>::WIDE)
     {
         if (a.splits > 1)
         {
-            return launch_fused_as<K, DP, SPLIT, true>(a, stream);
+            return launch_fused_as<K, DP, ARITH, true>(a, stream);
         }
     }
-    return launch_fused_as<K, DP, SPLIT, false>(a, stream);
+    return launch_fused_as<K, DP, ARITH, false>(a, stream);
 }
 
 } // namespace

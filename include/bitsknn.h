@@ -199,6 +199,7 @@ int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major, const float* po
  */
 #define BITSKNN_FUSED_FP32 0
 #define BITSKNN_FUSED_BF16X3 1
+#define BITSKNN_FUSED_EXACT 2
 int bitsknn_fused_l2_topk_f32_ex(const float* queries_dim_major, const float* points_dim_major,
                                  int dim, int32_t q, int32_t n, float* out_dist, int32_t* out_label,
                                  int k, int query_reg, int db_reg, int dim_reg, int block_query_dim,
