@@ -23,6 +23,10 @@ static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
 // for a stage of the ring that ran out of polls since bitsknn_fused_status last looked.
 static __device__ __align__(16) int fault_word[4];
 
+#ifdef BITSKNN_FUSED_TIMING
+static __device__ unsigned long long timing_words[8];
+#endif
+
 constexpr int MAX_DEVICES = 64;
 // Default bound on the polls of one wait for a stage (each poll sleeps 64 cycles: about 0.1 s in
 // all, many thousand times the longest merge a wave can be held up by).
@@ -274,6 +278,13 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     }
     fused_args a{queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, 1, 0, k, n, 1, 0, FUSED_PLAIN,
                  out_dist, k, symbols.fault, poll_limit()};
+#ifdef BITSKNN_FUSED_TIMING
+    {
+        void* timing_ptr = nullptr;
+        BITSKNN_HIP_CHECK(hipGetSymbolAddress(&timing_ptr, HIP_SYMBOL(timing_words)));
+        a.timing = static_cast<unsigned long long*>(timing_ptr);
+    }
+#endif
     if (splits > 1)
     {
         // partial lists [q][splits][k] in the workspace: distances first, then labels
@@ -455,3 +466,19 @@ extern "C" int bitsknn_fused_status(void* stream)
                 "in NaN and the results of the calls since the last check must be discarded",
                 gave_up);
 }
+
+#ifdef BITSKNN_FUSED_TIMING
+// instrumented build only: synchronises, copies the eight cycle sums out and clears them
+extern "C" int bitsknn_fused_timing(unsigned long long* out8, void* stream)
+{
+    using namespace bitsknn;
+    auto* hip_stream = static_cast<hipStream_t>(stream);
+    void* timing_ptr = nullptr;
+    BITSKNN_HIP_CHECK(hipGetSymbolAddress(&timing_ptr, HIP_SYMBOL(timing_words)));
+    BITSKNN_HIP_CHECK(hipStreamSynchronize(hip_stream));
+    BITSKNN_HIP_CHECK(hipMemcpy(out8, timing_ptr, 8 * sizeof(unsigned long long), hipMemcpyDeviceToHost));
+    static const unsigned long long zeros[8] = {};
+    BITSKNN_HIP_CHECK(hipMemcpy(timing_ptr, zeros, sizeof(zeros), hipMemcpyHostToDevice));
+    return BITSKNN_OK;
+}
+#endif

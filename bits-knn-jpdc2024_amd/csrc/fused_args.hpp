@@ -64,6 +64,10 @@ struct fused_args
     // end and overwrites the k-th distances of its queries with NaN.
     int* fault;
     int poll_limit;
+#ifdef BITSKNN_FUSED_TIMING
+    // instrumented build: cycles of all waves per phase of the stage loop, added up here
+    unsigned long long* timing;
+#endif
 };
 
 // one per compiled list length K (fused_inst.hip); arith: one of FUSED_ARITH_*, used where the

@@ -52,6 +52,25 @@ namespace bitsknn
 namespace
 {
 
+// Instrumented build (-DBITSKNN_FUSED_TIMING): every wave adds up the cycles it spends in the phases
+// of the stage loop of the ring (0 waiting for a stage, 1 waiting for the loads of the next one,
+// 2 writing it and requesting the one after, 3 filtering the stage, 4 working through candidates)
+// and adds them to fused_args::timing at the end.
+#ifdef BITSKNN_FUSED_TIMING
+#define BITSKNN_FT_LAP(i)                                                                          \
+    do                                                                                            \
+    {                                                                                             \
+        const long long ft_now = static_cast<long long>(__builtin_readcyclecounter());            \
+        ft_cycles[i] += ft_now - ft_mark;                                                         \
+        ft_mark = ft_now;                                                                         \
+    } while (0)
+#else
+#define BITSKNN_FT_LAP(i)                                                                          \
+    do                                                                                            \
+    {                                                                                             \
+    } while (0)
+#endif
+
 // minimum of three values in one instruction; a NaN operand is ignored
 __device__ __forceinline__ float min3(float a, float b, float c)
 {
@@ -415,6 +434,10 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     bool merged = false;             // wave-uniform: this wave has merged during the current stage
     int stage_slot = 0;              // stage index modulo 3: the slot of merge_wanted in use
     bool gave_up = false;            // wave-uniform: a wait for a stage of the ring ran out of polls
+#ifdef BITSKNN_FUSED_TIMING
+    long long ft_cycles[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    long long ft_mark = static_cast<long long>(__builtin_readcyclecounter());
+#endif
 
     // ---- merge of all buffers of this wave into the lists --------------------------------------
     auto merge_event = [&]() __attribute__((always_inline)) {
@@ -944,11 +967,15 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     };
     // bit r where value r of this lane is not above the threshold (negated compare: a NaN counts)
     auto bits_of = [&](const vfloat16& w) __attribute__((always_inline)) -> u32 {
+        // two instructions per value: the compare, then bits = 2 bits + its result as the carry
         u32 bits = 0;
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
+        for (int r = 15; r >= 0; --r)
         {
-            bits |= !(w[r] > thr) ? 1U << r : 0U;
+            asm("v_cmp_ngt_f32 vcc, %1, %2\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc"
+                : "+v"(bits)
+                : "v"(w[r]), "v"(thr)
+                : "vcc");
         }
         return bits;
     };
@@ -964,107 +991,93 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             {
                 zero[r] = 0.0F;
             }
-            // the filter values of one tile: lowered norm - 2 q.p from the pieces
-            auto filter_values = [&](int local0) __attribute__((always_inline)) -> vfloat16 {
-                const vuint4* const mine = cells + local0 + ql;
-                vfloat16 acc;
-                if constexpr (DP <= 8)
-                {
-                    // first half of the wave: piece 1 of the point against pieces 1 and 2 of the
-                    // query; second half: piece 2 against piece 1, the norm cell against (1, 1)
-                    const vuint4 a0 = mine[(half != 0 ? 1 : 0) * PT];
-                    const vuint4 a1 = mine[(half != 0 ? 2 : 0) * PT];
-                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(vbf16x8, a0), __builtin_bit_cast(vbf16x8, qs[0][0]), zero, 0, 0, 0);
-                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(vbf16x8, a1), __builtin_bit_cast(vbf16x8, qs[1][0]), acc, 0, 0, 0);
-                }
-                else
-                {
-                    vuint4 p1[KB];
-                    vuint4 p2[KB];
-#pragma unroll
-                    for (int kb = 0; kb < KB; ++kb)
-                    {
-                        p1[kb] = mine[(2 * kb + half) * PT];
-                        p2[kb] = mine[(KS + 2 * kb + half) * PT];
-                    }
-                    const vuint4 nn = mine[2 * KS * PT];
-                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(vbf16x8, nn), __builtin_bit_cast(vbf16x8, qs[2][0]), zero, 0, 0, 0);
-                    static_for<0, KB>([&](auto kb_tag) {
-                        constexpr int kb = decltype(kb_tag)::value;
-                        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(vbf16x8, p2[kb]), __builtin_bit_cast(vbf16x8, qs[0][kb]), acc, 0, 0, 0);
-                        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(vbf16x8, p1[kb]), __builtin_bit_cast(vbf16x8, qs[1][kb]), acc, 0, 0, 0);
-                        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(vbf16x8, p1[kb]), __builtin_bit_cast(vbf16x8, qs[0][kb]), acc, 0, 0, 0);
-                    });
-                }
-                return acc;
-            };
-            // First every tile of the stage is filtered without a branch: which pairs of tiles hold
-            // a value to look at is noted in `flagged` (wave-uniform).  Then the filter values of the
-            // flagged pairs are computed again (a few matrix instructions) to find the lanes and
-            // rows, and the candidates of the whole stage are worked through together.
-            constexpr int TILES = MT >= 2 ? 2 : 1;
-            constexpr int PAIRS = MT / TILES;
+            // First every tile of the stage is filtered without a branch: which tiles hold a value
+            // to look at is noted in `flagged` (wave-uniform).  Then the lanes and rows of the
+            // flagged tiles are collected, and the candidates of the whole stage are worked through
+            // together.  The matrix instructions of the stage's tiles take turns, term by term, so
+            // that none waits for the result of the one before it.
+            constexpr int TERMS = DP <= 8 ? 2 : 3 * KB + 1;
             u32 flagged = 0;
-            vfloat16 w0;
-            vfloat16 w1;
-            static_for<0, PAIRS>([&](auto p_tag) {
-                constexpr int p = decltype(p_tag)::value;
-                w0 = filter_values(p * 64);
-                if constexpr (TILES == 2)
+            vfloat16 w[MT];
+            {
+                vuint4 cell[MT][DP <= 8 ? 2 : 2 * KB + 1];
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
                 {
-                    w1 = filter_values(p * 64 + 32);
+                    const vuint4* const mine = cells + 32 * t + ql;
+                    if constexpr (DP <= 8)
+                    {
+                        // first half of the wave: piece 1 of the point against pieces 1 and 2 of
+                        // the query; second half: piece 2 against piece 1, the norm cell against
+                        // (1, 1)
+                        cell[t][0] = mine[(half != 0 ? 1 : 0) * PT];
+                        cell[t][1] = mine[(half != 0 ? 2 : 0) * PT];
+                    }
+                    else
+                    {
+#pragma unroll
+                        for (int kb = 0; kb < KB; ++kb)
+                        {
+                            cell[t][kb] = mine[(2 * kb + half) * PT];
+                            cell[t][KB + kb] = mine[(KS + 2 * kb + half) * PT];
+                        }
+                        cell[t][2 * KB] = mine[2 * KS * PT];
+                    }
                 }
-                // The first read of the tiles is a compare the compiler sees, so that it places the
+                __builtin_amdgcn_sched_barrier(0);
+                static_for<0, TERMS>([&](auto j_tag) {
+                    constexpr int j = decltype(j_tag)::value;
+                    // term j: which cell of the point against which operand of the query
+                    // (up to 8 dimensions: the two cells in turn; else the norm cell first, then per
+                    // 16 dimensions piece 2 x piece 1, piece 1 x piece 2, piece 1 x piece 1)
+                    constexpr int kb = DP <= 8 ? 0 : (j - 1) / 3;
+                    constexpr int which = DP <= 8 ? j : (j - 1) % 3;
+                    constexpr int a_at = DP <= 8 ? j : (j == 0 ? 2 * KB : (which == 0 ? KB + kb : kb));
+                    constexpr int b_piece = DP <= 8 ? j : (j == 0 ? 2 : (which == 1 ? 1 : 0));
+                    constexpr int b_kb = DP <= 8 || j == 0 ? 0 : kb;
+#pragma unroll
+                    for (int t = 0; t < MT; ++t)
+                    {
+                        w[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(vbf16x8, cell[t][a_at]), __builtin_bit_cast(vbf16x8, qs[b_piece][b_kb]),
+                            j == 0 ? zero : w[t], 0, 0, 0);
+                    }
+                });
+            }
+            static_for<0, MT>([&](auto t_tag) {
+                constexpr int t = decltype(t_tag)::value;
+                // The first read of the tile is a compare the compiler sees, so that it places the
                 // wait states a matrix result needs before it; assembly operands are not covered by
                 // that hazard handling.
-                const u64 last_passes =
-                    __builtin_amdgcn_ballot_w64(!(w0[15] > thr) || (TILES == 2 && !(w1[15] > thr)));
+                const u64 last_passes = __builtin_amdgcn_ballot_w64(!(w[t][15] > thr));
                 __builtin_amdgcn_sched_barrier(0);
-                float smallest = smallest_of(w0);
-                if constexpr (TILES == 2)
-                {
-                    const float second = smallest_of(w1);
-                    smallest = minimum3(smallest, second, second);
-                }
-                flagged |= (last_passes | __builtin_amdgcn_ballot_w64(!(smallest > thr))) != 0 ? 1U << p : 0U;
+                const float smallest = smallest_of(w[t]);
+                flagged |= (last_passes | __builtin_amdgcn_ballot_w64(!(smallest > thr))) != 0 ? 1U << t : 0U;
             });
+            BITSKNN_FT_LAP(3);
             if (flagged != 0)
             {
-                u64 cand = 0;
-                if constexpr (PAIRS == 1)
-                {
-                    cand = bits_of(w0);
-                    if constexpr (TILES == 2)
+                u32 part[MT];
+                static_for<0, MT>([&](auto t_tag) {
+                    constexpr int t = decltype(t_tag)::value;
+                    part[t] = 0;
+                    if ((flagged >> t & 1U) != 0)
                     {
-                        cand |= static_cast<u64>(bits_of(w1)) << 16U;
+                        part[t] = bits_of(w[t]);
                     }
+                });
+                u64 cand = part[0];
+                if constexpr (MT >= 2)
+                {
+                    cand |= static_cast<u64>(part[1]) << 16U;
                 }
-                else
+                if constexpr (MT == 4)
                 {
-                    static_assert(PAIRS == 2 && TILES == 2);
-                    u32 part[2] = {0, 0};
-#pragma unroll 1
-                    for (int p = 0; p < 2; ++p)
-                    {
-                        if ((flagged >> p & 1U) != 0)
-                        {
-                            w0 = filter_values(p * 64);
-                            w1 = filter_values(p * 64 + 32);
-                            const u32 bits = bits_of(w0) | (bits_of(w1) << 16U);
-                            part[0] = p == 0 ? bits : part[0];
-                            part[1] = p == 1 ? bits : part[1];
-                        }
-                    }
-                    cand = static_cast<u64>(part[0]) | (static_cast<u64>(part[1]) << 32U);
+                    cand |= static_cast<u64>(part[2] | (part[3] << 16U)) << 32U;
                 }
                 exact_candidates(cand, stage, base);
             }
+            BITSKNN_FT_LAP(4);
         }
         else if constexpr (SPLIT)
         {
@@ -1379,9 +1392,15 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         }
         int slot = 0;  // of the stage being multiplied
         int round = 0; // how often that slot has been used before
+        BITSKNN_FT_LAP(5);
         for (int base = n_begin; base < n; base += PT)
         {
             wait_for(slot, round + 1);
+            BITSKNN_FT_LAP(0);
+#ifdef BITSKNN_FUSED_TIMING
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            BITSKNN_FT_LAP(1);
+#endif
             if (base + PT < n)
             {
                 const int next = slot + 1 == NB ? 0 : slot + 1;
@@ -1392,6 +1411,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                     fetch(base + 2 * PT);
                 }
             }
+            BITSKNN_FT_LAP(2);
             multiply(stages + slot * STAGE_FLOATS, base);
             slot = slot + 1 == NB ? 0 : slot + 1;
             round += slot == 0 ? 1 : 0;
@@ -1400,6 +1420,16 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
 
     // whatever is left in the buffers; also writes the lists of queries that never merged
     merge_event();
+#ifdef BITSKNN_FUSED_TIMING
+    BITSKNN_FT_LAP(6);
+    if (lane == 0)
+    {
+        for (int i = 0; i < 8; ++i)
+        {
+            atomicAdd(a.timing + i, static_cast<unsigned long long>(ft_cycles[i]));
+        }
+    }
+#endif
     // (the radius is the k-th distance of the finished list now if that is below the first radius)
     if (a.splits == 1 && first_radius < __builtin_inff() && !(radius < first_radius) && half == 0)
     {
