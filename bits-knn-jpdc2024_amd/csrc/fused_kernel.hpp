@@ -832,19 +832,17 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             {
                 share += __builtin_bit_cast(float, lane_xor32<4>(__builtin_bit_cast(u32, share)));
             }
-            if (sd0 == 0)
             {
-                // the lowered norm in two pieces; points beyond the end only pass an infinite radius
+                // the lowered norm in two pieces, written by every thread of the point (same
+                // value: no branch in the staging code, which is scheduled between the matrix
+                // instructions of the stage being filtered); points beyond the end only pass an
+                // infinite radius
                 const float lowered = __builtin_fmaf(-NORM_LOWER, share, share);
                 const vfloat2 whole{lowered, 0.0F};
                 const u32 first = __builtin_bit_cast(u32, __builtin_convertvector(whole, vbf16x2)) & 0xFFFFU;
                 const vfloat2 rest{lowered - __builtin_bit_cast(float, first << 16U), 0.0F};
                 const u32 second = __builtin_bit_cast(u32, __builtin_convertvector(rest, vbf16x2)) & 0xFFFFU;
-                vuint4 cell{first | (second << 16U), 0, 0, 0};
-                if (!(base + sp < n))
-                {
-                    cell[0] = BF16_HUGE;
-                }
+                const vuint4 cell{base + sp < n ? first | (second << 16U) : BF16_HUGE, 0, 0, 0};
                 reinterpret_cast<vuint4*>(stage + DP * PT)[(G::CELLS - 1) * PT + sp] = cell;
             }
         }
@@ -980,104 +978,241 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         return bits;
     };
 
+    // EXACT, first half of a stage: the filter values of all its tiles, lowered norm - 2 q.p from the
+    // pieces.  The matrix instructions of the tiles take turns, term by term, so that none waits for
+    // the result of the one before it.
+    auto filter_values = [&](const float* stage, vfloat16 (&w)[MT]) __attribute__((always_inline)) {
+        const vuint4* const cells = reinterpret_cast<const vuint4*>(stage + DP * PT);
+        vfloat16 zero;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+        {
+            zero[r] = 0.0F;
+        }
+        constexpr int TERMS = DP <= 8 ? 2 : 3 * KB + 1;
+        vuint4 cell[MT][DP <= 8 ? 2 : 2 * KB + 1];
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+        {
+            const vuint4* const mine = cells + 32 * t + ql;
+            if constexpr (DP <= 8)
+            {
+                // first half of the wave: piece 1 of the point against pieces 1 and 2 of the query;
+                // second half: piece 2 against piece 1, the norm cell against (1, 1)
+                cell[t][0] = mine[(half != 0 ? 1 : 0) * PT];
+                cell[t][1] = mine[(half != 0 ? 2 : 0) * PT];
+            }
+            else
+            {
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+                {
+                    cell[t][kb] = mine[(2 * kb + half) * PT];
+                    cell[t][KB + kb] = mine[(KS + 2 * kb + half) * PT];
+                }
+                cell[t][2 * KB] = mine[2 * KS * PT];
+            }
+        }
+        static_for<0, TERMS>([&](auto j_tag) {
+            constexpr int j = decltype(j_tag)::value;
+            // term j: which cell of the point against which operand of the query (up to 8
+            // dimensions: the two cells in turn; else the norm cell first, then per 16 dimensions
+            // piece 2 x piece 1, piece 1 x piece 2, piece 1 x piece 1)
+            constexpr int kb = DP <= 8 ? 0 : (j - 1) / 3;
+            constexpr int which = DP <= 8 ? j : (j - 1) % 3;
+            constexpr int a_at = DP <= 8 ? j : (j == 0 ? 2 * KB : (which == 0 ? KB + kb : kb));
+            constexpr int b_piece = DP <= 8 ? j : (j == 0 ? 2 : (which == 1 ? 1 : 0));
+            constexpr int b_kb = DP <= 8 || j == 0 ? 0 : kb;
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+            {
+                w[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                    __builtin_bit_cast(vbf16x8, cell[t][a_at]), __builtin_bit_cast(vbf16x8, qs[b_piece][b_kb]),
+                    j == 0 ? zero : w[t], 0, 0, 0);
+            }
+        });
+    };
+    // EXACT: the filter values of a stage as above, with the staging of the next stage (`into`,
+    // first point `next_base`; the values are in `pre`) cut into pieces of a few vector and LDS
+    // instructions that are placed one after each of the first matrix instructions, where they
+    // execute next to it.  The staging code has no branch (every thread of a point writes the norm
+    // cell); scheduling barriers keep the order written here.
+    auto filter_values_and_stage = [&](const float* stage, vfloat16 (&w)[MT], float* into, int next_base) __attribute__((always_inline)) {
+        const vuint4* const cells = reinterpret_cast<const vuint4*>(stage + DP * PT);
+        vfloat16 zero;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+        {
+            zero[r] = 0.0F;
+        }
+        constexpr int TERMS = DP <= 8 ? 2 : 3 * KB + 1;
+        constexpr int NCELL = DP <= 8 ? 2 : 2 * KB + 1;
+        vuint4 cell[MT][NCELL];
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+        {
+            const vuint4* const mine = cells + 32 * t + ql;
+            if constexpr (DP <= 8)
+            {
+                cell[t][0] = mine[(half != 0 ? 1 : 0) * PT];
+                cell[t][1] = mine[(half != 0 ? 2 : 0) * PT];
+            }
+            else
+            {
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+                {
+                    cell[t][kb] = mine[(2 * kb + half) * PT];
+                    cell[t][KB + kb] = mine[(KS + 2 * kb + half) * PT];
+                }
+                cell[t][2 * KB] = mine[2 * KS * PT];
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // staging state
+        constexpr int PAIRS_OF_VALUES = VPT / 2;
+        constexpr int CHUNKS = PAIRS_OF_VALUES + 4;
+        static_assert(!EXACT || CHUNKS <= MT * TERMS, "a piece of staging per matrix instruction");
+        float share = 0.0F;
+        u32 piece1[4] = {0, 0, 0, 0};
+        u32 piece2[4] = {0, 0, 0, 0};
+        u32 norm_word = 0;
+        vuint4* const into_cells = reinterpret_cast<vuint4*>(into + DP * PT);
+        constexpr int PIECE2 = DP <= 8 ? 1 : KS; // first cell of the second pieces
+        auto chunk = [&](auto c_tag) __attribute__((always_inline)) {
+            constexpr int c = decltype(c_tag)::value;
+            if constexpr (c < PAIRS_OF_VALUES)
+            {
+                // two values: pieces, share of the norm, fp32 rows
+                const vfloat2 pair{pre[2 * c], pre[2 * c + 1]};
+                const u32 first = __builtin_bit_cast(u32, __builtin_convertvector(pair, vbf16x2));
+                const vfloat2 rest{pair.x - __builtin_bit_cast(float, first << 16U),
+                                   pair.y - __builtin_bit_cast(float, first & 0xFFFF0000U)};
+                piece1[c] = first;
+                piece2[c] = __builtin_bit_cast(u32, __builtin_convertvector(rest, vbf16x2));
+                share = __builtin_fmaf(pair.x, pair.x, share);
+                share = __builtin_fmaf(pair.y, pair.y, share);
+                into[(sd0 + 2 * c) * PT + sp] = pair.x;
+                into[(sd0 + 2 * c + 1) * PT + sp] = pair.y;
+            }
+            else if constexpr (c == PAIRS_OF_VALUES)
+            {
+                if constexpr (VPT == 8)
+                {
+                    const int ks = sd0 / 8;
+                    into_cells[ks * PT + sp] = vuint4{piece1[0], piece1[1], piece1[2], piece1[3]};
+                    into_cells[(PIECE2 + ks) * PT + sp] = vuint4{piece2[0], piece2[1], piece2[2], piece2[3]};
+                }
+                else
+                {
+                    // half a cell per thread
+                    typedef u32 vuint2 __attribute__((ext_vector_type(2)));
+                    vuint2* const halves = reinterpret_cast<vuint2*>(into + DP * PT);
+                    const int h = sd0 / 4;
+                    halves[2 * sp + h] = vuint2{piece1[0], piece1[1]};
+                    halves[2 * (PIECE2 * PT + sp) + h] = vuint2{piece2[0], piece2[1]};
+                }
+            }
+            else if constexpr (c == PAIRS_OF_VALUES + 1)
+            {
+                // the threads of a point are TPP neighbouring lanes
+                if constexpr (TPP >= 2)
+                {
+                    share += __builtin_bit_cast(float, lane_xor32<1>(__builtin_bit_cast(u32, share)));
+                }
+                if constexpr (TPP >= 4)
+                {
+                    share += __builtin_bit_cast(float, lane_xor32<2>(__builtin_bit_cast(u32, share)));
+                }
+                if constexpr (TPP == 8)
+                {
+                    share += __builtin_bit_cast(float, lane_xor32<4>(__builtin_bit_cast(u32, share)));
+                }
+            }
+            else if constexpr (c == PAIRS_OF_VALUES + 2)
+            {
+                const float lowered = __builtin_fmaf(-NORM_LOWER, share, share);
+                const vfloat2 whole{lowered, 0.0F};
+                const u32 first = __builtin_bit_cast(u32, __builtin_convertvector(whole, vbf16x2)) & 0xFFFFU;
+                const vfloat2 rest{lowered - __builtin_bit_cast(float, first << 16U), 0.0F};
+                const u32 second = __builtin_bit_cast(u32, __builtin_convertvector(rest, vbf16x2)) & 0xFFFFU;
+                norm_word = next_base + sp < n ? first | (second << 16U) : BF16_HUGE;
+            }
+            else
+            {
+                into_cells[(G::CELLS - 1) * PT + sp] = vuint4{norm_word, 0, 0, 0};
+            }
+        };
+        static_for<0, TERMS>([&](auto j_tag) {
+            constexpr int j = decltype(j_tag)::value;
+            constexpr int kb = DP <= 8 ? 0 : (j - 1) / 3;
+            constexpr int which = DP <= 8 ? j : (j - 1) % 3;
+            constexpr int a_at = DP <= 8 ? j : (j == 0 ? 2 * KB : (which == 0 ? KB + kb : kb));
+            constexpr int b_piece = DP <= 8 ? j : (j == 0 ? 2 : (which == 1 ? 1 : 0));
+            constexpr int b_kb = DP <= 8 || j == 0 ? 0 : kb;
+            static_for<0, MT>([&](auto t_tag) {
+                constexpr int t = decltype(t_tag)::value;
+                constexpr int m = j * MT + t; // number of this matrix instruction
+                w[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                    __builtin_bit_cast(vbf16x8, cell[t][a_at]), __builtin_bit_cast(vbf16x8, qs[b_piece][b_kb]),
+                    j == 0 ? zero : w[t], 0, 0, 0);
+                if constexpr (m < CHUNKS)
+                {
+                    chunk(std::integral_constant<int, m>{});
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        });
+    };
+    // EXACT, second half of a stage.  First every tile is filtered without a branch: which tiles hold
+    // a value to look at is noted in `flagged` (wave-uniform).  Then the lanes and rows of the
+    // flagged tiles are collected, and the candidates of the whole stage are worked through together.
+    auto filter_and_append = [&](const vfloat16 (&w)[MT], const float* stage, int base) __attribute__((always_inline)) {
+        u32 flagged = 0;
+        static_for<0, MT>([&](auto t_tag) {
+            constexpr int t = decltype(t_tag)::value;
+            // The first read of the tile is a compare the compiler sees, so that it places the
+            // wait states a matrix result needs before it; assembly operands are not covered by
+            // that hazard handling.
+            const u64 last_passes = __builtin_amdgcn_ballot_w64(!(w[t][15] > thr));
+            __builtin_amdgcn_sched_barrier(0);
+            const float smallest = smallest_of(w[t]);
+            flagged |= (last_passes | __builtin_amdgcn_ballot_w64(!(smallest > thr))) != 0 ? 1U << t : 0U;
+        });
+        BITSKNN_FT_LAP(3);
+        if (flagged != 0)
+        {
+            u32 part[MT];
+            static_for<0, MT>([&](auto t_tag) {
+                constexpr int t = decltype(t_tag)::value;
+                part[t] = 0;
+                if ((flagged >> t & 1U) != 0)
+                {
+                    part[t] = bits_of(w[t]);
+                }
+            });
+            u64 cand = part[0];
+            if constexpr (MT >= 2)
+            {
+                cand |= static_cast<u64>(part[1]) << 16U;
+            }
+            if constexpr (MT == 4)
+            {
+                cand |= static_cast<u64>(part[2] | (part[3] << 16U)) << 32U;
+            }
+            exact_candidates(cand, stage, base);
+        }
+        BITSKNN_FT_LAP(4);
+    };
+
     // all row tiles of a stage: distances, filter, append
     auto multiply = [&](const float* stage, int base) {
         if constexpr (EXACT)
         {
-            const vuint4* const cells = reinterpret_cast<const vuint4*>(stage + DP * PT);
-            vfloat16 zero;
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-            {
-                zero[r] = 0.0F;
-            }
-            // First every tile of the stage is filtered without a branch: which tiles hold a value
-            // to look at is noted in `flagged` (wave-uniform).  Then the lanes and rows of the
-            // flagged tiles are collected, and the candidates of the whole stage are worked through
-            // together.  The matrix instructions of the stage's tiles take turns, term by term, so
-            // that none waits for the result of the one before it.
-            constexpr int TERMS = DP <= 8 ? 2 : 3 * KB + 1;
-            u32 flagged = 0;
             vfloat16 w[MT];
-            {
-                vuint4 cell[MT][DP <= 8 ? 2 : 2 * KB + 1];
-#pragma unroll
-                for (int t = 0; t < MT; ++t)
-                {
-                    const vuint4* const mine = cells + 32 * t + ql;
-                    if constexpr (DP <= 8)
-                    {
-                        // first half of the wave: piece 1 of the point against pieces 1 and 2 of
-                        // the query; second half: piece 2 against piece 1, the norm cell against
-                        // (1, 1)
-                        cell[t][0] = mine[(half != 0 ? 1 : 0) * PT];
-                        cell[t][1] = mine[(half != 0 ? 2 : 0) * PT];
-                    }
-                    else
-                    {
-#pragma unroll
-                        for (int kb = 0; kb < KB; ++kb)
-                        {
-                            cell[t][kb] = mine[(2 * kb + half) * PT];
-                            cell[t][KB + kb] = mine[(KS + 2 * kb + half) * PT];
-                        }
-                        cell[t][2 * KB] = mine[2 * KS * PT];
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                static_for<0, TERMS>([&](auto j_tag) {
-                    constexpr int j = decltype(j_tag)::value;
-                    // term j: which cell of the point against which operand of the query
-                    // (up to 8 dimensions: the two cells in turn; else the norm cell first, then per
-                    // 16 dimensions piece 2 x piece 1, piece 1 x piece 2, piece 1 x piece 1)
-                    constexpr int kb = DP <= 8 ? 0 : (j - 1) / 3;
-                    constexpr int which = DP <= 8 ? j : (j - 1) % 3;
-                    constexpr int a_at = DP <= 8 ? j : (j == 0 ? 2 * KB : (which == 0 ? KB + kb : kb));
-                    constexpr int b_piece = DP <= 8 ? j : (j == 0 ? 2 : (which == 1 ? 1 : 0));
-                    constexpr int b_kb = DP <= 8 || j == 0 ? 0 : kb;
-#pragma unroll
-                    for (int t = 0; t < MT; ++t)
-                    {
-                        w[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(vbf16x8, cell[t][a_at]), __builtin_bit_cast(vbf16x8, qs[b_piece][b_kb]),
-                            j == 0 ? zero : w[t], 0, 0, 0);
-                    }
-                });
-            }
-            static_for<0, MT>([&](auto t_tag) {
-                constexpr int t = decltype(t_tag)::value;
-                // The first read of the tile is a compare the compiler sees, so that it places the
-                // wait states a matrix result needs before it; assembly operands are not covered by
-                // that hazard handling.
-                const u64 last_passes = __builtin_amdgcn_ballot_w64(!(w[t][15] > thr));
-                __builtin_amdgcn_sched_barrier(0);
-                const float smallest = smallest_of(w[t]);
-                flagged |= (last_passes | __builtin_amdgcn_ballot_w64(!(smallest > thr))) != 0 ? 1U << t : 0U;
-            });
-            BITSKNN_FT_LAP(3);
-            if (flagged != 0)
-            {
-                u32 part[MT];
-                static_for<0, MT>([&](auto t_tag) {
-                    constexpr int t = decltype(t_tag)::value;
-                    part[t] = 0;
-                    if ((flagged >> t & 1U) != 0)
-                    {
-                        part[t] = bits_of(w[t]);
-                    }
-                });
-                u64 cand = part[0];
-                if constexpr (MT >= 2)
-                {
-                    cand |= static_cast<u64>(part[1]) << 16U;
-                }
-                if constexpr (MT == 4)
-                {
-                    cand |= static_cast<u64>(part[2] | (part[3] << 16U)) << 32U;
-                }
-                exact_candidates(cand, stage, base);
-            }
-            BITSKNN_FT_LAP(4);
+            filter_values(stage, w);
+            __builtin_amdgcn_sched_barrier(0);
+            filter_and_append(w, stage, base);
         }
         else if constexpr (SPLIT)
         {
@@ -1393,6 +1528,32 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         int slot = 0;  // of the stage being multiplied
         int round = 0; // how often that slot has been used before
         BITSKNN_FT_LAP(5);
+        if constexpr (EXACT)
+        {
+            // The next stage is written while the matrix instructions of this one run (see
+            // filter_values_and_stage).  (The stage after the last one is "written" from whatever
+            // the registers hold, into a slot that nobody reads any more.)
+            for (int base = n_begin; base < n; base += PT)
+            {
+                wait_for(slot, round + 1);
+                BITSKNN_FT_LAP(0);
+                const int next = slot + 1 == NB ? 0 : slot + 1;
+                const float* const stage = stages + slot * STAGE_FLOATS;
+                vfloat16 w[MT];
+                __builtin_amdgcn_sched_barrier(0);
+                filter_values_and_stage(stage, w, stages + next * STAGE_FLOATS, base + PT);
+                count_in(next);
+                if (base + 2 * PT < n)
+                {
+                    fetch(base + 2 * PT);
+                }
+                BITSKNN_FT_LAP(2);
+                filter_and_append(w, stage, base);
+                slot = next;
+                round += slot == 0 ? 1 : 0;
+            }
+        }
+        else
         for (int base = n_begin; base < n; base += PT)
         {
             wait_for(slot, round + 1);
