@@ -265,6 +265,7 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
                          reinterpret_cast<std::uintptr_t>(workspace) % 4 == 0
                      ? choose_splits(q, n)
                      : 1;
+
     while (splits > 1 && partial_list_bytes(q, splits, k) > workspace_bytes)
     {
         splits /= 2;

@@ -222,7 +222,7 @@ struct fused_geometry
         !WIDE && (SPLIT ? K <= FQ_CAP
                         : (DP <= 8 && K <= 128) || (DP >= 16 && DP <= RING_MAX_DP && K <= FQ_CAP));
     static constexpr int NB = RING ? 3 : 2;
-    static constexpr int SLOTS = RING && !SPLIT && DP >= 16 ? 24 : CAP; // slots a query buffer has in LDS
+    static constexpr int SLOTS = EXACT && K <= 16 ? 16 : RING && !SPLIT && DP >= 16 ? 24 : CAP; // slots a query buffer has in LDS
     static_assert(!SPLIT || (DP <= 64 && TPP == KS), "one staging thread per point and cell");
     static_assert(!EXACT || (DP <= 64 && VPT == (DP <= 8 ? 4 : 8) && PT <= 128),
                   "the stages of the exact arithmetic serve up to 64 dimensions, in at most four tiles");
@@ -953,15 +953,20 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             }
         }
     };
-    // the filter of a tile: the smallest of the 16 values of every lane (a NaN if there is one)
+    // the filter of a tile: the smallest of the 16 values of every lane (a NaN if there is one),
+    // eight v_minimum3_f32
     auto smallest_of = [&](const vfloat16& w) __attribute__((always_inline)) -> float {
+        auto least = [](float a, float b, float c) __attribute__((always_inline)) -> float {
+            return __builtin_elementwise_minimum(__builtin_elementwise_minimum(a, b), c);
+        };
         float low[5];
 #pragma unroll
         for (int g = 0; g < 5; ++g)
         {
-            low[g] = minimum3(w[3 * g], w[3 * g + 1], w[3 * g + 2]);
+            low[g] = least(w[3 * g], w[3 * g + 1], w[3 * g + 2]);
         }
-        return minimum3(minimum3(low[0], low[1], low[2]), low[3], low[4]);
+        const float upper = least(low[3], low[4], w[15]);
+        return __builtin_elementwise_minimum(least(low[0], low[1], low[2]), upper);
     };
     // bit r where value r of this lane is not above the threshold (negated compare: a NaN counts)
     auto bits_of = [&](const vfloat16& w) __attribute__((always_inline)) -> u32 {
@@ -1164,29 +1169,33 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             });
         });
     };
-    // EXACT, second half of a stage.  First every tile is filtered without a branch: which tiles hold
-    // a value to look at is noted in `flagged` (wave-uniform).  Then the lanes and rows of the
-    // flagged tiles are collected, and the candidates of the whole stage are worked through together.
+    // EXACT, second half of a stage.  First every tile is filtered without a branch: the smallest
+    // filter value of every lane per tile and over the stage.  Only if some lane's is not above its
+    // threshold are the lanes and rows of the tiles concerned collected, and the candidates of the
+    // whole stage are worked through together.
     auto filter_and_append = [&](const vfloat16 (&w)[MT], const float* stage, int base) __attribute__((always_inline)) {
-        u32 flagged = 0;
-        static_for<0, MT>([&](auto t_tag) {
-            constexpr int t = decltype(t_tag)::value;
-            // The first read of the tile is a compare the compiler sees, so that it places the
-            // wait states a matrix result needs before it; assembly operands are not covered by
-            // that hazard handling.
-            const u64 last_passes = __builtin_amdgcn_ballot_w64(!(w[t][15] > thr));
-            __builtin_amdgcn_sched_barrier(0);
-            const float smallest = smallest_of(w[t]);
-            flagged |= (last_passes | __builtin_amdgcn_ballot_w64(!(smallest > thr))) != 0 ? 1U << t : 0U;
-        });
+        float smallest[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+        {
+            smallest[t] = smallest_of(w[t]);
+        }
+        float of_stage = smallest[0];
+#pragma unroll
+        for (int t = 1; t < MT; ++t)
+        {
+            of_stage = __builtin_elementwise_minimum(of_stage, smallest[t]);
+        }
+        // (negated compares: a NaN passes)
+        const bool any = __builtin_amdgcn_ballot_w64(!(of_stage > thr)) != 0;
         BITSKNN_FT_LAP(3);
-        if (flagged != 0)
+        if (any)
         {
             u32 part[MT];
             static_for<0, MT>([&](auto t_tag) {
                 constexpr int t = decltype(t_tag)::value;
                 part[t] = 0;
-                if ((flagged >> t & 1U) != 0)
+                if (__builtin_amdgcn_ballot_w64(!(smallest[t] > thr)) != 0)
                 {
                     part[t] = bits_of(w[t]);
                 }
