@@ -1,12 +1,17 @@
 """Parity of bits-fused (distance + top-k in one kernel, through the C ABI) with the CPU oracle.
 
-The distances come from fp32 MFMA, so they are not bit-identical to the reference's sequential
-fused multiply-adds.  Bar (the stated tolerance of this path): the k-th neighbour distance within
-1e-5 relative of the oracle's -- of the completed distance (value + ||q||^2) for dim >= 16, of the
-reported partial distance below that, see tests/parity.py -- and recall@k >= 0.999 against the
-oracle's neighbour sets.  Structure is checked exactly: ascending order, distinct in-range labels,
-and every reported distance equal to the oracle's distance of the reported label (to 1e-5 of the
-magnitude of the terms that cancel in it).
+Up to 64 dimensions the plain entry points report distances computed with the reference's own
+arithmetic (sequential fused multiply-adds over the dimensions in order, norm - 2 dot), found
+through a filter on the bf16 matrix instructions that is guaranteed never to drop a candidate:
+there the result must equal the oracle's BIT FOR BIT, values and labels, equal distances by lower
+index ("default" below).  With the distances taken from the fp32 matrix instructions ("mfma": every
+dimension above 64, and BITSKNN_FUSED_FP32 on request) or from bf16x3 products they are not
+bit-identical to the reference's; the bar there (the stated tolerance of this path) is the k-th
+neighbour distance within 1e-5 relative of the oracle's -- of the completed distance
+(value + ||q||^2) for dim >= 16, of the reported partial distance below that, see tests/parity.py --
+and recall@k >= 0.999 against the oracle's neighbour sets.  Structure is checked exactly in every
+mode: ascending order, distinct in-range labels, and every reported distance equal to the oracle's
+distance of the reported label (to 1e-5 of the magnitude of the terms that cancel in it).
 """
 import numpy as np
 import pytest
@@ -30,10 +35,30 @@ def _fused(bk, dev, points, queries, k, params=(8, 4, 2), bqd=1, dim_mult=1, wor
     return od.cpu().numpy(), ol.cpu().numpy()
 
 
-def _check(oracle, points, queries, k, gd, gl, min_recall=0.999, bar_dim=None):
+MODES = ["default", "mfma"]
+
+
+def _arith(bk, mode):
+    """C-ABI arithmetic of a test mode: None = the plain entry points"""
+    return {"default": None, "mfma": bk.FUSED_FP32, "bf16x3": bk.FUSED_BF16X3}[mode]
+
+
+def _bits(mode, dim):
+    """whether the result of this mode must equal the oracle's bit for bit"""
+    return mode == "default" and dim <= 64
+
+
+def _check(oracle, points, queries, k, gd, gl, min_recall=0.999, bar_dim=None, bits=False):
     n = points.shape[0]
     part = oracle.dist(queries, points, "partial")
     ed, el = oracle.topk(part, k)
+    if bits:
+        kk = min(k, n)
+        assert np.array_equal(gd[:, :kk].view(np.uint32), ed[:, :kk].view(np.uint32)), "values differ from the oracle's"
+        assert np.array_equal(gl[:, :kk], el[:, :kk]), "labels differ from the oracle's"
+        if k > n:
+            assert np.all(np.isinf(gd[:, n:]))
+        return 1.0
     qn = (queries.astype(np.float64) ** 2).sum(1)[:, None]
     kk = min(k, n)
     # structure
@@ -71,51 +96,60 @@ def _check(oracle, points, queries, k, gd, gl, min_recall=0.999, bar_dim=None):
 
 # the reference's own fused-cache test cases (tests/topk/fused_cache_kernel_test.cu:12-82):
 # (dim, k, points, queries) with items {8,4,2}, block 4, deg 2
+@pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("d,k,n,q", [(8, 32, 1024, 32), (16, 32, 1024, 1), (37, 32, 997, 43), (9, 16, 25, 7)])
-def test_reference_unit_test_shapes(bk, dev, oracle, d, k, n, q):
+def test_reference_unit_test_shapes(bk, dev, oracle, d, k, n, q, mode):
     p, s = oracle.generate(42, n, q, d)
-    gd, gl = _fused(bk, dev, p, s, k, (8, 4, 2), 4, 2)
-    _check(oracle, p, s, k, gd, gl)
+    gd, gl = _fused(bk, dev, p, s, k, (8, 4, 2), 4, 2, arithmetic=_arith(bk, mode))
+    _check(oracle, p, s, k, gd, gl, bits=_bits(mode, d))
 
 
+@pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("k", [4, 8, 16, 32, 64, 128, 256])
-@pytest.mark.parametrize("d", [4, 8, 16, 32])
-def test_all_k_values(bk, dev, oracle, k, d):
+@pytest.mark.parametrize("d", [4, 8, 16, 32, 64])
+def test_all_k_values(bk, dev, oracle, k, d, mode):
     p, s = oracle.generate(100 + k + d, 20000, 150, d)
-    gd, gl = _fused(bk, dev, p, s, k)
-    _check(oracle, p, s, k, gd, gl)
+    gd, gl = _fused(bk, dev, p, s, k, arithmetic=_arith(bk, mode))
+    _check(oracle, p, s, k, gd, gl, bits=_bits(mode, d))
 
 
-@pytest.mark.parametrize("d", [1, 2, 3, 5, 17, 33, 48, 49, 64, 100, 113, 200, 256])
-def test_dimensions(bk, dev, oracle, d):
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("d", [1, 2, 3, 5, 7, 9, 15, 17, 31, 33, 48, 49, 63, 64, 65, 100, 113, 200, 256])
+def test_dimensions(bk, dev, oracle, d, mode):
     p, s = oracle.generate(d, 3000, 70, d)
-    gd, gl = _fused(bk, dev, p, s, 16, (2, 4, 1), 1, 1)
-    _check(oracle, p, s, 16, gd, gl)
+    gd, gl = _fused(bk, dev, p, s, 16, (2, 4, 1), 1, 1, arithmetic=_arith(bk, mode))
+    _check(oracle, p, s, 16, gd, gl, bits=_bits(mode, d))
 
 
+@pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("n,q", [(1, 1), (31, 5), (32, 33), (33, 127), (255, 128), (257, 129), (1000, 300), (5001, 1)])
-def test_ragged_counts(bk, dev, oracle, n, q):
-    p, s = oracle.generate(n + q, n, q, 8)
-    for k in (4, 32):
-        gd, gl = _fused(bk, dev, p, s, k)
-        _check(oracle, p, s, k, gd, gl)
+def test_ragged_counts(bk, dev, oracle, n, q, mode):
+    for d in (8, 24):
+        p, s = oracle.generate(n + q + d, n, q, d)
+        for k in (4, 32):
+            gd, gl = _fused(bk, dev, p, s, k, arithmetic=_arith(bk, mode))
+            _check(oracle, p, s, k, gd, gl, bits=_bits(mode, d))
 
 
-# points per stage by padded dimension: 256 up to 16 dimensions, 128 / 64 / 32 for 32 / 64 / 128
-@pytest.mark.parametrize("d,stage", [(8, 256), (16, 256), (32, 128), (64, 64), (100, 32)])
-@pytest.mark.parametrize("arithmetic", ["fp32", "bf16x3"])
-def test_point_counts_around_whole_stages(bk, dev, oracle, d, stage, arithmetic):
+# points per stage by padded dimension.  fp32 matrix instructions: 256 up to 16 dimensions, 128 / 64
+# / 32 for 32 / 64 / 128; the exact arithmetic and bf16x3: 128 up to 16 dimensions, 64 / 32 for 32 / 64
+@pytest.mark.parametrize("d", [8, 16, 32, 64, 100])
+@pytest.mark.parametrize("mode", ["default", "mfma", "bf16x3"])
+def test_point_counts_around_whole_stages(bk, dev, oracle, d, mode):
     # one to five stages, each count one short of, at and one past a whole stage: the ring of three
     # stage buffers starts, wraps around and ends at every position
-    if arithmetic == "bf16x3" and not 9 <= d <= 64:
+    if mode == "bf16x3" and not 9 <= d <= 64:
         pytest.skip("bf16x3 products serve 9 to 64 dimensions")
-    mode = bk.FUSED_BF16X3 if arithmetic == "bf16x3" else None
+    if mode == "mfma" or d > 64:
+        stage = {8: 256, 16: 256, 32: 128, 64: 64, 100: 32}[d]
+    else:
+        stage = {8: 128, 16: 128, 32: 64, 64: 32}[d]
     q = 130
     for stages in (1, 2, 3, 4, 5):
         for n in (stages * stage - 1, stages * stage, stages * stage + 1):
             p, s = oracle.generate(1000 * stages + n + d, n, q, d)
-            gd, gl = _fused(bk, dev, p, s, 16, arithmetic=mode)
-            _check(oracle, p, s, 16, gd, gl)
+            gd, gl = _fused(bk, dev, p, s, 16, arithmetic=_arith(bk, mode))
+            _check(oracle, p, s, 16, gd, gl, bits=_bits(mode, d))
 
 
 @pytest.mark.parametrize("n,q,d,k", [(20000, 150, 8, 32), (70001, 300, 16, 16), (300000, 33, 32, 4),
@@ -132,9 +166,14 @@ def test_point_split_variant_with_workspace(bk, dev, oracle, n, q, d, k):
     need = bk.fused_workspace_bytes(q, n, k)
     assert need % (8 * q * k) == 0 and 0 < need <= 8 * q * 64 * k
     gd, gl = _fused(bk, dev, p, s, k, workspace="auto")
-    _check(oracle, p, s, k, gd, gl)
+    _check(oracle, p, s, k, gd, gl, bits=True)
     pd, pl = _fused(bk, dev, p, s, k)
     assert np.array_equal(gd, pd) and np.array_equal(gl, pl)
+    # the same through the fp32 matrix instructions (the kernel over ranges has another geometry there)
+    md, ml = _fused(bk, dev, p, s, k, workspace="auto", arithmetic=bk.FUSED_FP32)
+    _check(oracle, p, s, k, md, ml)
+    pd, pl = _fused(bk, dev, p, s, k, arithmetic=bk.FUSED_FP32)
+    assert np.array_equal(md, pd) and np.array_equal(ml, pl)
 
 
 def test_smaller_workspace_means_fewer_ranges(bk, dev, oracle):
@@ -155,14 +194,18 @@ def test_duplicate_points_are_ordered_by_index(bk, dev, oracle):
     # every point appears 4 times: equal distances must come out by ascending index
     base, s = oracle.generate(5, 500, 64, 8)
     p = np.concatenate([base, base, base, base])
-    gd, gl = _fused(bk, dev, p, s, 32)
     part = oracle.dist(s, p, "partial")
     ed, el = oracle.topk(part, 32)
-    assert np.array_equal(gl, el)
+    for arithmetic in (None, bk.FUSED_FP32):
+        gd, gl = _fused(bk, dev, p, s, 32, arithmetic=arithmetic)
+        assert np.array_equal(gl, el)
+        if arithmetic is None:
+            assert np.array_equal(gd.view(np.uint32), ed.view(np.uint32))
 
 
+@pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("d,k", [(8, 32), (16, 4), (16, 32), (32, 32), (64, 16), (16, 64), (100, 32)])
-def test_points_that_come_ever_closer(bk, dev, oracle, d, k):
+def test_points_that_come_ever_closer(bk, dev, oracle, d, k, mode):
     # Every point is nearer to every query than all points before it, so every tile brings each
     # query 32 candidates: more than a query buffer of 24 slots holds even when it is empty (the
     # geometries with three stages in LDS), which has such a tile appended in two halves.  Small
@@ -176,7 +219,7 @@ def test_points_that_come_ever_closer(bk, dev, oracle, d, k):
     p[:, 1:3] = rng.integers(-1, 2, size=(n, 2))  # (a step along it outweighs what these can add)
     part = oracle.dist(s, p, "partial")
     assert np.all(np.diff(part, axis=1) < 0), "the points must approach every query"
-    gd, gl = _fused(bk, dev, p, s, k)
+    gd, gl = _fused(bk, dev, p, s, k, arithmetic=_arith(bk, mode))
     ed, el = oracle.topk(part, k)
     assert np.array_equal(gd, ed) and np.array_equal(gl, el)
 
@@ -187,9 +230,55 @@ def test_exact_arithmetic_is_bit_exact(bk, dev, oracle):
     rng = np.random.default_rng(3)
     p = rng.integers(-8, 9, size=(4000, 12)).astype(np.float32)
     s = rng.integers(-8, 9, size=(100, 12)).astype(np.float32)
-    gd, gl = _fused(bk, dev, p, s, 64)
     ed, el = oracle.topk(oracle.dist(s, p, "partial"), 64)
-    assert np.array_equal(gd, ed) and np.array_equal(gl, el)
+    for arithmetic in (None, bk.FUSED_FP32, bk.FUSED_BF16X3):
+        gd, gl = _fused(bk, dev, p, s, 64, arithmetic=arithmetic)
+        assert np.array_equal(gd, ed) and np.array_equal(gl, el)
+
+
+@pytest.mark.parametrize("d", [5, 8, 16, 24, 32, 64])
+@pytest.mark.parametrize("kind", ["tiny", "huge", "signs", "near", "ranges-of-magnitude", "subnormal", "constant"])
+def test_the_filter_never_drops_a_neighbour(bk, dev, oracle, d, kind):
+    """The filter of the default arithmetic promises a lower bound of every distance (bf16 pieces,
+    an error budget relative to ||q||^2 + 2 ||p||^2): a neighbour it dropped would show as a
+    difference from the oracle.  Inputs chosen against that budget: values near the ends of the
+    fp32 range, mixed signs, points so near the queries that norm and dot product cancel almost
+    completely (nearly every value then ties within the slack and is looked at exactly), coordinates
+    spread over eight orders of magnitude, subnormal coordinates, and constant vectors.  Bit for bit
+    against the oracle."""
+    n, q, k = 6000, 140, 32
+    rng = np.random.default_rng(d * 7 + len(kind))
+    p = rng.random((n, d), dtype=np.float32)
+    s = rng.random((q, d), dtype=np.float32)
+    if kind == "tiny":
+        p, s = p * np.float32(1e-18), s * np.float32(1e-18)
+    elif kind == "huge":
+        p, s = p * np.float32(3e17), s * np.float32(3e17)
+    elif kind == "signs":
+        p, s = (p - 0.5) * 100, (s - 0.5) * 100
+    elif kind == "near":
+        centre = (rng.random(d, dtype=np.float32) * 2000 - 1000).astype(np.float32)
+        p = centre + (p - 0.5) * np.float32(0.01)
+        s = centre + (s - 0.5) * np.float32(0.01)
+    elif kind == "ranges-of-magnitude":
+        scale = np.float32(10.0) ** rng.integers(-4, 5, size=d).astype(np.float32)
+        p, s = (p - 0.3) * scale, (s - 0.3) * scale
+    elif kind == "subnormal":
+        p[:, ::2] *= np.float32(1e-41)
+        s[:, ::2] *= np.float32(1e-41)
+    else:
+        p[:] = np.float32(0.7)
+        s[:] = np.float32(0.3)
+        p[::3, 0] = np.float32(0.25)
+    p = np.ascontiguousarray(p, dtype=np.float32)
+    s = np.ascontiguousarray(s, dtype=np.float32)
+    gd, gl = _fused(bk, dev, p, s, k)
+    ed, el = oracle.topk(oracle.dist(s, p, "partial"), k)
+    assert np.array_equal(gd.view(np.uint32), ed.view(np.uint32)), "values differ from the oracle's"
+    assert np.array_equal(gl, el), "labels differ from the oracle's"
+    if kind in ("signs", "near"):
+        wd, wl = _fused(bk, dev, p, s, k, workspace="auto")
+        assert np.array_equal(gd, wd) and np.array_equal(gl, wl)
 
 
 # reference-held checksums of the fused runs (data/fused-*.err), query 0
@@ -205,7 +294,7 @@ def test_golden_fused_checksums(bk, dev, oracle, golden, n, q):
             k = rec["k"]
             gd, gl = _fused(bk, dev, p, s, k)
             assert str(oracle.checksum(gl[0])) in rec["checksums"], (rec, oracle.checksum(gl[0]))
-            _check(oracle, p, s[:64], k, gd[:64], gl[:64])
+            _check(oracle, p, s[:64], k, gd[:64], gl[:64], bits=True)
             checked += 1
     assert checked >= 18
 
@@ -259,16 +348,17 @@ def test_long_lists_stay_in_the_fused_kernel(bk, dev, oracle, k):
     points, queries = oracle.generate(77, n, q, d)
     assert 0 < bk.fused_workspace_bytes(q, n, k) <= 8 * q * 64 * k and bk.fused_workspace_bytes(q, n, k) < q * n * 4
     gd, gl = _fused(bk, dev, points, queries, k, workspace="auto")
-    _check(oracle, points, queries, k, gd, gl)
+    _check(oracle, points, queries, k, gd, gl, bits=True)
     fd, fl = _fused(bk, dev, points, queries, k)
     assert np.array_equal(gd, fd) and np.array_equal(gl, fl)
 
 
-def _sampled_points(n, d, split, scale):
+def _sampled_points(n, d, small_stages, scale):
     """Points the launch over a sample visits (on at least 2^17 points, lists of 128 and more,
     or of 64 and more when the points are cut into ranges, start from radii taken from
-    it): every `scale`-th stage, the one in the middle of its group."""
-    if split:
+    it): every `scale`-th stage, the one in the middle of its group.  small_stages: the stage sizes
+    of the exact arithmetic and of bf16x3 products."""
+    if small_stages:
         stage = 128 if d <= 16 else (64 if d <= 32 else 32)
     else:
         stage = 256 if d <= 16 else (128 if d <= 32 else (64 if d <= 64 else 32))
@@ -278,13 +368,17 @@ def _sampled_points(n, d, split, scale):
                            for s in range(stages)])
 
 
-@pytest.mark.parametrize("d,k,arithmetic,ranges", [(8, 128, "fp32", False), (8, 256, "fp32", False),
-                                                   (32, 256, "fp32", False), (100, 128, "fp32", False),
-                                                   (16, 256, "bf16x3", False), (48, 128, "bf16x3", False),
-                                                   (8, 64, "fp32", True), (8, 256, "fp32", True),
-                                                   (16, 128, "fp32", True), (32, 64, "fp32", True),
-                                                   (24, 128, "bf16x3", True)])
-def test_first_radius_from_a_sample(bk, dev, oracle, d, k, arithmetic, ranges):
+@pytest.mark.parametrize("d,k,mode,ranges", [(8, 128, "mfma", False), (8, 256, "mfma", False),
+                                             (32, 256, "mfma", False), (100, 128, "default", False),
+                                             (8, 128, "default", False), (8, 256, "default", False),
+                                             (32, 256, "default", False), (64, 128, "default", False),
+                                             (16, 256, "bf16x3", False), (48, 128, "bf16x3", False),
+                                             (8, 64, "mfma", True), (8, 256, "mfma", True),
+                                             (16, 128, "mfma", True), (32, 64, "mfma", True),
+                                             (8, 64, "default", True), (8, 256, "default", True),
+                                             (16, 128, "default", True), (32, 64, "default", True),
+                                             (24, 128, "bf16x3", True)])
+def test_first_radius_from_a_sample(bk, dev, oracle, d, k, mode, ranges):
     """Lists on many points start from radii that a launch over a sample of the points
     estimates, and workgroups with a query whose estimate proved too low repeat their pass; the
     result must not depend on either.  Uniform points (the estimates hold), and points whose
@@ -294,25 +388,27 @@ def test_first_radius_from_a_sample(bk, dev, oracle, d, k, arithmetic, ranges):
     rng = np.random.default_rng(d * k)
     queries = rng.random((q, d), dtype=np.float32)
     points = rng.random((n, d), dtype=np.float32)
-    arithmetic = bk.FUSED_BF16X3 if arithmetic == "bf16x3" else None
+    arithmetic = _arith(bk, mode)
+    bits = _bits(mode, d)
     workspace = "auto" if ranges else None
     if ranges:
         assert bk.fused_workspace_bytes(q, n, k) > 0
     gd, gl = _fused(bk, dev, points, queries, k, arithmetic=arithmetic, workspace=workspace)
-    _check(oracle, points, queries, k, gd, gl)
+    _check(oracle, points, queries, k, gd, gl, bits=bits)
     assert not np.isnan(gd).any()
-    sample = _sampled_points(n, d, arithmetic is not None, 256 if ranges else 64)
+    sample = _sampled_points(n, d, mode == "bf16x3" or bits, 256 if ranges else 64)
     assert sample.size >= 2 * 32
     points = rng.random((n, d), dtype=np.float32)
     points[:, :4] += 1.0                    # all points a step away in four dimensions ...
     points[sample] = rng.random((sample.size, d), dtype=np.float32)    # ... but the sampled ones
     queries[::2, :4] += 1.0                 # every other query sits among the far points
     gd, gl = _fused(bk, dev, points, queries, k, arithmetic=arithmetic, workspace=workspace)
-    _check(oracle, points, queries, k, gd, gl, bar_dim=8)   # norms twice those of uniform points
+    _check(oracle, points, queries, k, gd, gl, bar_dim=8, bits=bits)   # norms twice those of uniform points
     assert not np.isnan(gd).any()
 
 
-def test_random_shapes_against_the_oracle(bk, dev, oracle):
+@pytest.mark.parametrize("mode", MODES)
+def test_random_shapes_against_the_oracle(bk, dev, oracle, mode):
     """40 random problems over dimensions on both sides of every padded size, all list lengths,
     ragged point and query counts, with the plain entry point, the workspace the library asks for
     and a workspace that only holds partial lists."""
@@ -332,9 +428,12 @@ def test_random_shapes_against_the_oracle(bk, dev, oracle):
         elif kind == 2:
             workspace = torch.empty(max(8, 8 * q * 64 * k), dtype=torch.uint8, device=dev)
         p, s = oracle.generate(3000 + case, n, q, d)
-        gd, gl = _fused(bk, dev, p, s, k, (2, 4, 1), 1, 1, workspace=workspace)
+        arithmetic = _arith(bk, mode)
+        if arithmetic is not None and workspace is None:
+            workspace = None  # (bitsknn_fused_l2_topk_f32_ex takes no workspace as well)
+        gd, gl = _fused(bk, dev, p, s, k, (2, 4, 1), 1, 1, workspace=workspace, arithmetic=arithmetic)
         try:
-            _check(oracle, p, s, k, gd, gl)
+            _check(oracle, p, s, k, gd, gl, bits=_bits(mode, d))
         except AssertionError as e:
             raise AssertionError((case, n, q, d, k, kind)) from e
 
