@@ -30,11 +30,15 @@ which did not do its work cannot produce a figure.
                with one fixed configuration and with the one the optima file names
   gemm         ||p||^2 - 2 q.p on fp32 MFMA for 1,048,576 points x 4,096 queries, d = 64 (a 16 GiB
                matrix), then bits top-k (k = 64) on it
-  fused        bits-fused, 1,048,576 points x 65,536 queries, d in {8,16,32} x k in {4,16,32}, priced
-               against the fp32 MFMA peak with 2*q*n*d flops; `fused` itself is the d = 32, k = 32
-               case (queries/s), `fused.grid` the nine cases; `fused.long_lists` the same shape at
-               k in {64,128,256}; `fused.few_queries` the reference's own fused shape (8192 queries,
-               131,072 points, d = 8) through the entry point that cuts the points into ranges
+  fused        bits-fused, 1,048,576 points x 65,536 queries, d in {8,16,32} x k in {4,16,32}, through
+               the plain entry points: distances in the reference's arithmetic for the pairs that
+               pass a filter on the bf16 matrix instructions.  Priced against the bf16 matrix peak
+               with the matrix flops the filter executes, with the algorithmic 2*q*n*d flops over the
+               fp32 matrix peak beside it; `fused` itself is the d = 32, k = 32 case (queries/s, also
+               with every distance from the fp32 matrix instructions and from bf16x3 products),
+               `fused.grid` the nine cases; `fused.long_lists` the same shape at k in {64,128,256};
+               `fused.few_queries` the reference's own fused shape (8192 queries, 131,072 points,
+               d = 8) through the entry point that cuts the points into ranges
   cpu          `cpu_baseline`: the CPU restatement of the reference's parallel top-k (reference
                src/topk/parallel_knn.cpp:30-65) on the host cores and of its serial top-k
                (src/topk/serial_knn.cpp:35-43) on one core, on a 1024 x 65,536 matrix
@@ -172,7 +176,9 @@ def verify_neighbours(np, points, queries, exp_d, exp_l, got_d, got_l, k):
     ascending = bool(np.all(got_d[:, 1:] >= got_d[:, :-1]))
     value_ok = bool(np.all(completed <= REL)) if dim >= 16 else bool(np.all((of_value <= REL) | excused))
     ok = bool(np.all(of_scale <= REL)) and value_ok and recall >= MIN_RECALL and ascending
-    return ok, {"kth_err_of_scale": float(of_scale.max()), "kth_err_of_completed_distance": float(completed.max()),
+    bit_exact = bool(np.array_equal(got_d.view(np.uint32), exp_d.view(np.uint32)) and np.array_equal(got_l, exp_l))
+    return ok, {"bit_exact_values_and_labels": bit_exact,
+                "kth_err_of_scale": float(of_scale.max()), "kth_err_of_completed_distance": float(completed.max()),
                 "kth_err_of_value": float(of_value.max()), "queries": int(queries.shape[0]),
                 "queries_excused_below_resolution": int(excused.sum()), "recall": recall}
 
@@ -301,13 +307,10 @@ def leg_gemm(bitsknn, torch, timer, oracle, dev, steps, check, q=4096, n=1 << 20
     alt_l = torch.empty((q, k), dtype=torch.int32, device=dev)
     _, t_fused = timer.run(lambda: bitsknn.fused_l2_topk(queries, points, k, out_dist=alt_d, out_label=alt_l,
                                                          workspace=space), steps, 2)
-    fused_tflops = 2.0 * q * n * d / t_fused / 1e12
     result["fused_alternative"] = {
         "workload": f"bits-fused over ranges of points (workspace of {space.numel()} bytes), same {n} points x "
                     f"{q} queries, d={d}, k={k}; no distance matrix",
-        "ms": t_fused * 1e3, "queries_per_s": q / t_fused,
-        "roofline": {"bound": "mfma", "achieved": fused_tflops, "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": fused_tflops / MFMA_F32_PEAK_TFLOPS}}
+        "ms": t_fused * 1e3, "queries_per_s": q / t_fused, "roofline": fused_roofline(q, n, d, t_fused)}
     if check:
         sample = sample_indices(q, 16)
         points_h = np.ascontiguousarray(points.cpu().numpy().T)
@@ -330,16 +333,39 @@ def leg_gemm(bitsknn, torch, timer, oracle, dev, steps, check, q=4096, n=1 << 20
         result["verification"] = detail
         ok_alt, detail_alt = verify_neighbours(np, points_h, queries_h, exp_d, exp_l, alt_d[sample].cpu().numpy(),
                                                alt_l[sample].cpu().numpy(), k)
-        result["fused_alternative"]["verified"] = bool(ok_alt)
+        result["fused_alternative"]["verified"] = bool(ok_alt and detail_alt["bit_exact_values_and_labels"])
         result["fused_alternative"]["verification"] = detail_alt
     return result
 
 
+def filter_flops_per_pair(d):
+    """bf16 matrix flops the default fused kernel executes per (query, point) pair: matrix
+    instructions of 32 x 32 x 16, two per tile up to 8 dimensions, else three per 16 dimensions
+    (two pieces per operand, the smallest product left out) and one for the norm"""
+    terms = 2 if d <= 8 else 3 * ((d + 15) // 16) + 1
+    return terms * 32.0
+
+
+def fused_roofline(q, n, d, seconds):
+    """The default fused kernel against the matrix unit it runs on: the bf16 matrix instructions of
+    its filter (executed flops, padding included) against the bf16 peak; next to it the
+    algorithmic 2*q*n*d flops of the distance over the time, and what fraction of the fp32 matrix
+    peak that is (above 1: the contraction does not run on the fp32 unit)."""
+    executed = filter_flops_per_pair(d) * q * n / seconds / 1e12
+    algorithmic = 2.0 * q * n * d / seconds / 1e12
+    return {"bound": "mfma", "achieved": executed, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": executed / MFMA_BF16_PEAK_TFLOPS,
+            "matrix_instructions": "v_mfma_f32_32x32x16_bf16, %d flops per pair executed" % filter_flops_per_pair(d),
+            "algorithmic_tflops": algorithmic, "algorithmic_over_fp32_matrix_peak": algorithmic / MFMA_F32_PEAK_TFLOPS}
+
+
 def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=65536, n=1 << 20, long_ks=(),
               workspace=False):
-    """Config 5: bits-fused at d x k; the d = 32, k = 32 case also with bf16x3 products.  long_ks:
-    list lengths beyond the configuration's, reported apart (`long_lists`).  workspace: through the
-    entry point that may cut the points into ranges (few queries)."""
+    """Config 5: bits-fused at d x k through the plain entry points (the reference's arithmetic
+    behind a filter on the bf16 matrix instructions); the d = 32, k = 32 case also with the
+    distances from the fp32 matrix instructions and from bf16x3 products.  long_ks: list lengths
+    beyond the configuration's, reported apart (`long_lists`).  workspace: through the entry point
+    that may cut the points into ranges (few queries)."""
     import numpy as np
     grid = []
     long_lists = []
@@ -358,10 +384,11 @@ def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=6553
             if workspace:
                 space = torch.empty(max(1, bitsknn.fused_workspace_bytes(q, n, k)), dtype=torch.uint8, device=dev)
             _, seconds = timer.run(lambda: bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l,
-                                                                 workspace=space), steps, 1)
-            tflops = 2.0 * q * n * d / seconds / 1e12
+                                                                 workspace=space), steps, 2)
+            roof = fused_roofline(q, n, d, seconds)
             entry = {"d": d, "k": k, "ms": seconds * 1e3, "queries_per_s": q / seconds,
-                     "pairs_per_s": q * n / seconds, "frac": tflops / MFMA_F32_PEAK_TFLOPS}
+                     "pairs_per_s": q * n / seconds, "frac": roof["frac"],
+                     "algorithmic_over_fp32_matrix_peak": roof["algorithmic_over_fp32_matrix_peak"]}
             if check:
                 if part is None:
                     points_h = np.ascontiguousarray(points.cpu().numpy().T)
@@ -370,32 +397,38 @@ def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=6553
                 exp_d, exp_l = oracle.topk(part, k)
                 ok, detail = verify_neighbours(np, points_h, queries_h, exp_d, exp_l, out_d[sample].cpu().numpy(),
                                                out_l[sample].cpu().numpy(), k)
-                entry["verified"] = bool(ok)
+                # the default arithmetic is the reference's: nothing but bit for bit counts
+                entry["verified"] = bool(ok and (detail["bit_exact_values_and_labels"] or d > 64))
                 entry["verification"] = detail
             (grid if k in ks else long_lists).append(entry)
             if d == 32 and k == 32 and not workspace:
                 headline = {"workload": f"bits-fused, {n} points x {q} queries, d={d}, k={k}, fp32 uniform[0,1)",
-                            "arithmetic": "fp32 matrix instructions", "launches_timed": steps,
+                            "arithmetic": "sequential fp32 fused multiply-adds in dimension order (the reference's) "
+                                          "for every pair that passes a guaranteed lower bound from bf16 matrix "
+                                          "instructions",
+                            "launches_timed": steps,
                             "queries_per_s": q / seconds, "ms": seconds * 1e3, "pairs_per_s": q * n / seconds,
-                            "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_F32_PEAK_TFLOPS,
-                                         "unit": "TFLOP/s", "frac": tflops / MFMA_F32_PEAK_TFLOPS}}
+                            "roofline": roof}
                 if check:
                     headline["verified"] = entry["verified"]
-                out_d.fill_(-1.0)
-                _, split_s = timer.run(
-                    lambda: bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l,
-                                                  arithmetic=bitsknn.FUSED_BF16X3), steps, 1)
-                split_tflops = 6 * 2.0 * q * n * d / split_s / 1e12
-                headline["bf16x3"] = {
-                    "arithmetic": "three bf16 pieces per fp32 operand, six bf16 matrix products per product, "
-                                  "fp32 accumulation",
-                    "queries_per_s": q / split_s, "ms": split_s * 1e3, "pairs_per_s": q * n / split_s,
-                    "roofline": {"bound": "mfma", "achieved": split_tflops, "peak": MFMA_BF16_PEAK_TFLOPS,
-                                 "unit": "TFLOP/s", "frac": split_tflops / MFMA_BF16_PEAK_TFLOPS}}
-                if check:
-                    ok, detail = verify_neighbours(np, points_h, queries_h, exp_d, exp_l,
-                                                   out_d[sample].cpu().numpy(), out_l[sample].cpu().numpy(), k)
-                    headline["bf16x3"]["verified"] = bool(ok)
+                for name, arithmetic, text, flops_per_pair, peak in (
+                        ("mfma_f32", bitsknn.FUSED_FP32, "every distance from fp32 matrix instructions", 2.0 * d,
+                         MFMA_F32_PEAK_TFLOPS),
+                        ("bf16x3", bitsknn.FUSED_BF16X3, "three bf16 pieces per fp32 operand, six bf16 matrix products "
+                         "per product, fp32 accumulation", 12.0 * d, MFMA_BF16_PEAK_TFLOPS)):
+                    out_d.fill_(-1.0)
+                    _, other_s = timer.run(
+                        lambda: bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l,
+                                                      arithmetic=arithmetic), steps, 1)
+                    tflops = flops_per_pair * q * n / other_s / 1e12
+                    headline[name] = {"arithmetic": text, "queries_per_s": q / other_s, "ms": other_s * 1e3,
+                                      "pairs_per_s": q * n / other_s,
+                                      "roofline": {"bound": "mfma", "achieved": tflops, "peak": peak, "unit": "TFLOP/s",
+                                                   "frac": tflops / peak}}
+                    if check:
+                        ok, detail = verify_neighbours(np, points_h, queries_h, exp_d, exp_l,
+                                                       out_d[sample].cpu().numpy(), out_l[sample].cpu().numpy(), k)
+                        headline[name]["verified"] = bool(ok)
         del points, queries
     result = headline if headline is not None else {"workload": f"bits-fused, {n} points x {q} queries"}
     result["grid"] = grid
@@ -487,19 +520,24 @@ def summarise(result):
                            "distance_ms": r3(g["distance_ms"]), "distance_bf16x3_ms": r3(g["distance_bf16x3"]["ms"]),
                            "selection_ms": r3(g["selection_ms"]), "end_to_end_ms": r3(g["end_to_end_ms"]),
                            "fused_alternative_ms": r3(g["fused_alternative"]["ms"]),
-                           "fused_alternative_frac_mfma": r3(g["fused_alternative"]["roofline"]["frac"])}
+                           "fused_alternative_frac_bf16_mfma": r3(g["fused_alternative"]["roofline"]["frac"])}
     if "fused" in result:
         f = result["fused"]
-        out["fused_grid_frac_mfma"] = {f"d{e['d']}_k{e['k']}": r3(e["frac"]) for e in f.get("grid", [])}
         out["fused_grid_ms"] = {f"d{e['d']}_k{e['k']}": r3(e["ms"]) for e in f.get("grid", [])}
+        out["fused_grid_frac_bf16_mfma"] = {f"d{e['d']}_k{e['k']}": r3(e["frac"]) for e in f.get("grid", [])}
+        out["fused_grid_algorithmic_over_fp32_mfma_peak"] = {
+            f"d{e['d']}_k{e['k']}": r3(e["algorithmic_over_fp32_matrix_peak"]) for e in f.get("grid", [])}
         if "long_lists" in f:
-            out["fused_long_lists_frac_mfma"] = {f"d{e['d']}_k{e['k']}": r3(e["frac"]) for e in f["long_lists"]}
+            out["fused_long_lists_ms"] = {f"d{e['d']}_k{e['k']}": r3(e["ms"]) for e in f["long_lists"]}
         if "queries_per_s" in f:
-            out["fused_d32_k32"] = {"queries_per_s": round(f["queries_per_s"]), "frac_mfma": r3(f["roofline"]["frac"]),
+            out["fused_d32_k32"] = {"queries_per_s": round(f["queries_per_s"]), "ms": r3(f["ms"]),
+                                    "frac_bf16_mfma": r3(f["roofline"]["frac"]),
+                                    "algorithmic_over_fp32_mfma_peak": r3(f["roofline"]["algorithmic_over_fp32_matrix_peak"]),
                                     "launches_timed": f.get("launches_timed")}
-            if "bf16x3" in f:
-                out["fused_d32_k32"]["bf16x3_queries_per_s"] = round(f["bf16x3"]["queries_per_s"])
-                out["fused_d32_k32"]["bf16x3_frac_bf16_mfma"] = r3(f["bf16x3"]["roofline"]["frac"])
+            for name in ("mfma_f32", "bf16x3"):
+                if name in f:
+                    out["fused_d32_k32"][name + "_queries_per_s"] = round(f[name]["queries_per_s"])
+                    out["fused_d32_k32"][name + "_frac"] = r3(f[name]["roofline"]["frac"])
         if "few_queries" in f:
             out["fused_few_queries_ms"] = {f"d{e['d']}_k{e['k']}": r3(e["ms"]) for e in f["few_queries"]["cases"]}
     if "bits_sq" in result:

@@ -429,6 +429,11 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         }
     }
     float radius = first_radius;     // k-th smallest distance of my query so far
+    if constexpr (EXACT)
+    {
+        // (a first radius from a sample gives the filter its threshold from the first tile on)
+        thr = radius + (filter_slack + 0x1.0p-22F * __builtin_fabsf(radius));
+    }
     int fill = 0;                    // used slots of my query's buffer (same in both lanes of a query)
     bool have_list = false;          // wave-uniform: the lists in the output arrays are valid
     bool merged = false;             // wave-uniform: this wave has merged during the current stage

@@ -170,12 +170,17 @@ def test_hard_rows_at_full_size(bk, dev, oracle, hard_matrices, kind, k):
 
 # ---- neighbours against the oracle on sampled queries ------------------------------------------
 
-def _check_neighbours(oracle, points_dm, queries_dm, sample, got_d, got_l, k, what):
-    """points_dm / queries_dm: dim-major device tensors; got_*: the results of the sampled queries."""
+def _check_neighbours(oracle, points_dm, queries_dm, sample, got_d, got_l, k, what, bits=False):
+    """points_dm / queries_dm: dim-major device tensors; got_*: the results of the sampled queries.
+    bits: the result must equal the oracle's bit for bit."""
     points = np.ascontiguousarray(points_dm.cpu().numpy().T)
     queries = np.ascontiguousarray(queries_dm[:, sample].cpu().numpy().T)
     part = oracle.dist(queries, points, "partial")
     exp_d, exp_l = oracle.topk(part, k)
+    if bits:
+        assert np.array_equal(got_d.view(np.uint32), exp_d.view(np.uint32)), (what, "values differ from the oracle's")
+        assert np.array_equal(got_l, exp_l), (what, "labels differ from the oracle's")
+        return
     assert np.all(got_d[:, 1:] >= got_d[:, :-1])
     assert got_l.min() >= 0 and got_l.max() < points.shape[0]
     for row in got_l:
@@ -200,17 +205,20 @@ def _check_neighbours(oracle, points_dm, queries_dm, sample, got_d, got_l, k, wh
     assert hits / (len(sample) * k) >= MIN_RECALL, (what, hits / (len(sample) * k))
 
 
-# config 5: 1,048,576 points x 65,536 queries (2^36 pairs per launch)
-@pytest.mark.parametrize("d,k", [(8, 4), (16, 16), (32, 32)])
-def test_fused_at_full_size(bk, dev, oracle, d, k):
+# config 5: 1,048,576 points x 65,536 queries (2^36 pairs per launch).  The default arithmetic
+# (the reference's, behind the filter) bit for bit against the oracle on the sampled queries; the
+# fp32 matrix instructions to the tolerance.
+@pytest.mark.parametrize("d,k,mode", [(8, 4, "default"), (16, 16, "default"), (32, 32, "default"),
+                                      (8, 32, "default"), (32, 4, "default"), (32, 32, "mfma"), (8, 4, "mfma")])
+def test_fused_at_full_size(bk, dev, oracle, d, k, mode):
     import torch
     q, n = 65536, 1 << 20
     g = torch.Generator(device=dev)
     g.manual_seed(100 + d)
     points = torch.rand((d, n), device=dev, generator=g)
     queries = torch.rand((d, q), device=dev, generator=g)
-    od, ol = bk.fused_l2_topk(queries, points, k)
-    torch.cuda.synchronize()
+    od, ol = bk.fused_l2_topk(queries, points, k, arithmetic=None if mode == "default" else bk.FUSED_FP32)
+    bk.fused_status()
     # whole result: ascending, labels in range and distinct per query
     assert bool((od[:, 1:] >= od[:, :-1]).all())
     assert int(ol.min()) >= 0 and int(ol.max()) < n
@@ -218,7 +226,7 @@ def test_fused_at_full_size(bk, dev, oracle, d, k):
     assert bool((sorted_labels[:, 1:] != sorted_labels[:, :-1]).all())
     sample = _sample(q, 64)
     _check_neighbours(oracle, points, queries, sample, od[sample].cpu().numpy(), ol[sample].cpu().numpy(), k,
-                      ("fused", d, k))
+                      ("fused", d, k, mode), bits=mode == "default")
 
 
 # config 4: 1,048,576 points x 4,096 queries, d = 64 -> a 16 GiB matrix, then bits top-k, k = 64
