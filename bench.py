@@ -28,6 +28,7 @@ which did not do its work cannot produce a figure.
                optima file names for each k
   hard         16,384 x 65,536 rows sorted ascending / descending / drawn from 256 values, k = 32, 256,
                with one fixed configuration and with the one the optima file names
+  sq           bits-sq: 64 and 256 rows of 524,288 values, every row cut into parts (k = 16, 64)
   gemm         ||p||^2 - 2 q.p on fp32 MFMA for 1,048,576 points x 4,096 queries, d = 64 (a 16 GiB
                matrix), then bits top-k (k = 64) on it
   fused        bits-fused, 1,048,576 points x 65,536 queries, d in {8,16,32} x k in {4,16,32}, through
@@ -59,7 +60,7 @@ sys.path.insert(0, PKG)
 HBM_PEAK_GBS = 8000.0       # MI355X published peak
 MFMA_F32_PEAK_TFLOPS = 157.3  # dense fp32 matrix peak
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 matrix peak
-LEGS = ("headline", "calibration", "sweep", "hard", "gemm", "fused", "cpu")
+LEGS = ("headline", "calibration", "sweep", "hard", "sq", "gemm", "fused", "cpu")
 # values per thread in the block-size sweep: the same 2048 values of a row in flight per iteration
 # whatever the workgroup size (fewer waves per row need more loads each), and the larger batches
 # that long lists need where few rows fit a compute unit
@@ -260,6 +261,35 @@ def leg_hard(bitsknn, torch, timer, oracle, dev, steps, check, rows=16384, cols=
                 if check:
                     entry["verified"] = verify_topk(oracle, cache, matrix, sample, k, out_d, out_l)
                 out.append(entry)
+    return out
+
+
+def leg_sq(bitsknn, torch, timer, oracle, dev, steps, check, cols=1 << 19):
+    """bits-sq: few long rows (64 and 256 rows of 2^19 values), every row cut into the parts the
+    optima file names, through bitsknn_topk_bits_parts_f32; against the HBM roofline with the bytes
+    of the rows."""
+    from bitsknn import tuning
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(24)
+    matrix = torch.rand((256, cols), device=dev, generator=gen)
+    out = []
+    for rows in (64, 256):
+        part = matrix[:rows]
+        sample = sample_indices(rows, 8)
+        cache = {}
+        for k in (16, 64):
+            block, parts, items, _, _ = tuning.config_algorithm("bits-sq", rows, k)
+            scratch = {}
+            out_d = torch.full((rows, k), -1.0, dtype=torch.float32, device=dev)
+            out_l = torch.empty((rows, k), dtype=torch.int32, device=dev)
+            _, seconds = timer.run(lambda: bitsknn.topk_bits_parts(part, k, parts, block, items, scratch=scratch,
+                                                                   out_dist=out_d, out_label=out_l), max(steps, 20), 5)
+            entry = {"rows": rows, "cols": cols, "k": k, "parts": parts, "block": block, "items_per_thread": items,
+                     "us": seconds * 1e6, "elements_per_s": rows * cols / seconds,
+                     "frac": (4.0 * rows * cols + 8.0 * rows * k) / seconds / 1e9 / HBM_PEAK_GBS}
+            if check:
+                entry["verified"] = verify_topk(oracle, cache, part, sample, k, out_d, out_l)
+            out.append(entry)
     return out
 
 
@@ -626,6 +656,9 @@ def main():
         torch.cuda.empty_cache()
     if "hard" in legs:
         result["hard_inputs"] = leg_hard(bitsknn, torch, timer, oracle, dev, few, check)
+        torch.cuda.empty_cache()
+    if "sq" in legs:
+        result["bits_sq"] = leg_sq(bitsknn, torch, timer, oracle, dev, few, check)
         torch.cuda.empty_cache()
     if "gemm" in legs:
         result["gemm_knn"] = leg_gemm(bitsknn, torch, timer, oracle, dev, few, check)

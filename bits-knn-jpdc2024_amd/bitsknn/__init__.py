@@ -20,6 +20,7 @@ EXPORTS = (
     "bitsknn_last_error",
     "bitsknn_version",
     "bitsknn_topk_bits_f32",
+    "bitsknn_topk_bits_parts_f32",
     "bitsknn_topk_partial_bitonic_f32",
     "bitsknn_label_offsets",
     "bitsknn_fill_f32",
@@ -65,6 +66,8 @@ def lib():
         L.bitsknn_topk_bits_f32.restype = ctypes.c_int
         L.bitsknn_topk_bits_f32.argtypes = [vp, sz, vp, sz, vp, sz, sz, vp, vp, sz, u32, u32, u32,
                                             ctypes.c_int, vp]
+        L.bitsknn_topk_bits_parts_f32.restype = ctypes.c_int
+        L.bitsknn_topk_bits_parts_f32.argtypes = [vp, sz, sz, u32, vp, vp, vp, vp, vp, sz, u32, u32, u32, vp]
         L.bitsknn_topk_partial_bitonic_f32.restype = ctypes.c_int
         L.bitsknn_topk_partial_bitonic_f32.argtypes = [vp, sz, sz, sz, vp, vp, sz, u32, u32, vp]
         L.bitsknn_label_offsets.restype = ctypes.c_int
@@ -145,6 +148,31 @@ def topk_bits(dist, k, block_size=256, items_per_thread=16, prefetch=False, in_l
                                        _ptr(in_label), label_stride, _ptr(label_offsets), rows, cols,
                                        _ptr(out_dist), _ptr(out_label), _row_stride(out_dist), k,
                                        block_size, items_per_thread, 1 if prefetch else 0, _stream()))
+    return out_dist, out_label
+
+
+def topk_bits_parts(dist, k, parts, block_size=256, items_per_thread=16, scratch=None, out_dist=None,
+                    out_label=None):
+    """bits-sq: bits top-k of every row of a contiguous 2-D float32 device tensor with the rows cut
+    into `parts` parts (bitsknn_topk_bits_parts_f32).  scratch: a dict that keeps the device memory
+    for the parts' results and the counters between calls.  Returns (values, labels), rows x k."""
+    import torch
+    assert dist.is_cuda and dist.dtype == torch.float32 and dist.dim() == 2 and dist.is_contiguous()
+    rows, cols = dist.shape
+    if out_dist is None:
+        out_dist = torch.empty((rows, k), dtype=torch.float32, device=dist.device)
+    if out_label is None:
+        out_label = torch.empty((rows, k), dtype=torch.int32, device=dist.device)
+    key = (rows, parts, k, str(dist.device))
+    scratch = scratch if scratch is not None else {}
+    if key not in scratch:
+        scratch[key] = (torch.empty(rows * parts * k, dtype=torch.float32, device=dist.device),
+                        torch.empty(rows * parts * k, dtype=torch.int32, device=dist.device),
+                        torch.zeros(rows, dtype=torch.int32, device=dist.device))
+    part_d, part_l, counters = scratch[key]
+    _check(lib().bitsknn_topk_bits_parts_f32(_ptr(dist), rows, cols, parts, _ptr(part_d), _ptr(part_l),
+                                             _ptr(counters), _ptr(out_dist), _ptr(out_label),
+                                             _row_stride(out_dist), k, block_size, items_per_thread, _stream()))
     return out_dist, out_label
 
 

@@ -152,26 +152,10 @@ def sweep(repeats=10, point_count=512 * 1024, query_counts=QUERY_COUNTS, k_value
 def bits_sq(rows, k, deg, block, batch, scratch=None):
     """`bits-sq` through the C ABI (reference src/topk/singlepass/bits_knn.cu:132-186): every row
     is cut into `deg` parts that are selected independently with their labels shifted by the part's
-    offset, then the deg*k partial results of a row are selected again with their labels."""
-    import torch
+    offset, then the deg*k partial results of a row are selected again with their labels -- in one
+    launch (bitsknn_topk_bits_parts_f32)."""
     import bitsknn
-    q, n = rows.shape
-    assert n % deg == 0
-    if scratch is None:
-        scratch = {}
-    key = (q, k, deg)
-    if key not in scratch:
-        scratch[key] = (torch.empty((q * deg, k), dtype=torch.float32, device=rows.device),
-                        torch.empty((q * deg, k), dtype=torch.int32, device=rows.device),
-                        bitsknn.label_offsets(q, deg, n // deg, rows.device),
-                        torch.empty((q, k), dtype=torch.float32, device=rows.device),
-                        torch.empty((q, k), dtype=torch.int32, device=rows.device))
-    part_d, part_l, offsets, out_d, out_l = scratch[key]
-    bitsknn.topk_bits(rows.view(q * deg, n // deg), k, block, batch, True, label_offsets=offsets,
-                      out_dist=part_d, out_label=part_l)
-    bitsknn.topk_bits(part_d.view(q, deg * k), k, block, batch, True, in_label=part_l.view(q, deg * k),
-                      out_dist=out_d, out_label=out_l)
-    return out_d, out_l
+    return bitsknn.topk_bits_parts(rows, k, deg, block, batch, scratch=scratch if scratch is not None else {})
 
 
 def sweep_bits_sq(repeats=10, point_count=512 * 1024, query_counts=SQ_QUERY_COUNTS, k_values=K_VALUES,

@@ -53,6 +53,17 @@ struct topk_args
     std::int32_t* out_label;
     size_t out_stride;
     u32 k;
+    // Rows cut into parts (the kernels instantiated with SQ only; parts <= 1 otherwise): rows
+    // i*parts .. i*parts + parts - 1 of the matrix are the parts of logical row i.  out_dist and
+    // out_label then take the k pairs of every part (row stride k), `done` holds one counter per
+    // logical row (zero before the launch, zero again after it), and the workgroup that finishes
+    // a logical row's last part selects the k smallest of its parts * k pairs, with their labels,
+    // into final_dist / final_label.
+    u32 parts;
+    int* done;
+    float* final_dist;
+    std::int32_t* final_label;
+    size_t final_stride;
 };
 
 // Merge the filled part of every wave's buffer slice into the ascending top-k list.  Slice w
@@ -116,8 +127,11 @@ __device__ __forceinline__ void keep_smallest(float (&lo)[KEEP], float value)
 }
 
 // BS threads, IPT list entries per thread, L 16-byte (or 4 x 4-byte when !VEC) loads in flight
-// per thread and iteration.
-template <int BS, int IPT, int L, bool VEC>
+// per thread and iteration.  SQ: rows cut into parts (topk_args::parts): the workgroup that
+// finishes the last part of a logical row goes through the kernel's body a second time, over the
+// pairs its parts have left (reference: the second pass of single_query_bits,
+// src/topk/singlepass/bits_knn.cu:132-186, there a launch of its own).
+template <int BS, int IPT, int L, bool VEC, bool SQ = false>
 __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
 {
     constexpr int NL = BS * IPT;     // length of the top-k list and of the whole buffer
@@ -147,18 +161,27 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
     __shared__ int s_flag;  // some wave wants a merge
     __shared__ int s_more;  // some wave still has values to process after this merge
     __shared__ u32 s_sample[W];
+    __shared__ int s_ticket;
 
     int t = static_cast<int>(threadIdx.x);
     const int lane = t & (WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(t / WAVE);
     const size_t row_idx = blockIdx.x;
-    const float* __restrict__ row = a.in + row_idx * a.in_stride;
-    const std::int32_t* __restrict__ lrow =
-        a.in_label != nullptr ? a.in_label + row_idx * a.label_stride : nullptr;
-    const u32 label_offset =
-        a.label_offsets != nullptr ? static_cast<u32>(a.label_offsets[row_idx]) : 0U;
-    const u32 n = a.cols;
+    // (with SQ the second turn of the loop below points these at the pairs of the row's parts)
+    const float* row = a.in + row_idx * a.in_stride;
+    const std::int32_t* lrow = a.in_label != nullptr ? a.in_label + row_idx * a.label_stride : nullptr;
+    u32 label_offset = a.label_offsets != nullptr ? static_cast<u32>(a.label_offsets[row_idx]) : 0U;
+    u32 n = a.cols;
+    float* out_d = a.out_dist + row_idx * a.out_stride;
+    std::int32_t* out_l = a.out_label + row_idx * a.out_stride;
+    if constexpr (SQ)
+    {
+        // part p of a logical row: its labels start at p * (values per part)
+        label_offset = static_cast<u32>(row_idx % a.parts) * a.cols;
+    }
     u64* const slice = buffer + wave * CAP;
+    for (int phase = 0; phase < (SQ ? 2 : 1); ++phase)
+    {
 
     auto label_of = [&](u32 col) -> std::int32_t {
         const u32 base = lrow != nullptr ? static_cast<u32>(lrow[col]) : col;
@@ -725,18 +748,62 @@ __global__ void __launch_bounds__(BS) bits_topk_kernel(const topk_args a)
         break;
     }
 
-    float* __restrict__ out_d = a.out_dist + row_idx * a.out_stride;
-    std::int32_t* __restrict__ out_l = a.out_label + row_idx * a.out_stride;
+    // (the pairs of a part are stored past the caches of this part of the chip, so that the workgroup
+    // that reduces the row, wherever it runs, finds them without a write-back of the whole cache)
+    const bool to_be_reduced = SQ && phase == 0 && a.parts > 1 && a.done != nullptr;
 #pragma unroll
     for (int r = 0; r < IPT; ++r)
     {
         const u32 e = static_cast<u32>(t * IPT + r);
         if (e < a.k)
         {
-            out_d[e] = key_value(topk[r]);
-            out_l[e] = key_label(topk[r]);
+            if (to_be_reduced)
+            {
+                __hip_atomic_store(out_d + e, key_value(topk[r]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(out_l + e, key_label(topk[r]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            else
+            {
+                out_d[e] = key_value(topk[r]);
+                out_l[e] = key_label(topk[r]);
+            }
         }
     }
+    if constexpr (SQ)
+    {
+        if (!to_be_reduced)
+        {
+            break;
+        }
+        // The barrier waits for the stores of every thread; then one thread counts the part in.
+        // The workgroup that counts in last sees the pairs of all parts of its logical row (it
+        // drops what its caches hold first) and selects from them.
+        __syncthreads();
+        const size_t logical = row_idx / a.parts;
+        if (t == 0)
+        {
+            s_ticket = __hip_atomic_fetch_add(a.done + logical, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (s_ticket != static_cast<int>(a.parts) - 1)
+        {
+            break;
+        }
+        if (t == 0)
+        {
+            a.done[logical] = 0; // for the next launch
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        const size_t first_part = logical * a.parts;
+        row = a.out_dist + first_part * a.out_stride;
+        lrow = a.out_label + first_part * a.out_stride;
+        label_offset = 0;
+        n = a.parts * a.k;
+        out_d = a.final_dist + logical * a.final_stride;
+        out_l = a.final_label + logical * a.final_stride;
+        __syncthreads();
+    }
+    } // phase
 }
 
 

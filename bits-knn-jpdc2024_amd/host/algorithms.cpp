@@ -344,7 +344,7 @@ public:
 
 // `bits-sq`: every row is cut into --deg parts that are selected independently (labels shifted
 // by the part offset), then the deg*k partial results of a row are selected again with their
-// labels.
+// labels (reference: single_query_bits, src/topk/singlepass/bits_knn.cu:116-186).
 class single_query_bits : public device_knn
 {
 public:
@@ -362,42 +362,27 @@ public:
             const std::size_t parts = query_count() * args_.deg;
             tmp_dist_ = device_buffer<float>{parts * k()};
             tmp_label_ = device_buffer<std::int32_t>{parts * k()};
-            offsets_ = device_buffer<std::int32_t>{parts};
-            BITSKNN_CHECK(bitsknn_label_offsets(offsets_.data(), query_count(), args_.deg,
-                                                point_count() / args_.deg, nullptr));
+            // one counter per row, zero between calls
+            counters_ = device_buffer<std::int32_t>{query_count()};
+            HIP_CHECK(hipMemsetAsync(counters_.data(), 0, query_count() * sizeof(std::int32_t), nullptr));
+            sync_default_stream();
         }
     }
 
     void selection() override
     {
-        const auto block = static_cast<std::uint32_t>(args_.selection_block_size);
-        const auto batch = static_cast<std::uint32_t>(args_.items_per_thread[0]);
-        const auto kk = static_cast<std::uint32_t>(k());
-        if (args_.deg <= 1)
-        {
-            BITSKNN_CHECK(bitsknn_topk_bits_f32(in_dist_gpu(), point_count(), nullptr, 0, nullptr,
-                                                query_count(), point_count(), out_dist_.data(),
-                                                out_label_.data(), k(), kk, block, batch, 1, nullptr));
-        }
-        else
-        {
-            const std::size_t cols = point_count() / args_.deg;
-            const std::size_t parts = query_count() * args_.deg;
-            BITSKNN_CHECK(bitsknn_topk_bits_f32(in_dist_gpu(), cols, nullptr, 0, offsets_.data(), parts,
-                                                cols, tmp_dist_.data(), tmp_label_.data(), k(), kk,
-                                                block, batch, 1, nullptr));
-            const std::size_t merged = k() * args_.deg;
-            BITSKNN_CHECK(bitsknn_topk_bits_f32(tmp_dist_.data(), merged, tmp_label_.data(), merged,
-                                                nullptr, query_count(), merged, out_dist_.data(),
-                                                out_label_.data(), k(), kk, block, batch, 1, nullptr));
-        }
+        BITSKNN_CHECK(bitsknn_topk_bits_parts_f32(
+            in_dist_gpu(), query_count(), point_count(), static_cast<std::uint32_t>(std::max<std::size_t>(args_.deg, 1)),
+            tmp_dist_.data(), tmp_label_.data(), counters_.data(), out_dist_.data(), out_label_.data(), k(),
+            static_cast<std::uint32_t>(k()), static_cast<std::uint32_t>(args_.selection_block_size),
+            static_cast<std::uint32_t>(args_.items_per_thread[0]), nullptr));
         sync_default_stream();
     }
 
 private:
     device_buffer<float> tmp_dist_;
     device_buffer<std::int32_t> tmp_label_;
-    device_buffer<std::int32_t> offsets_;
+    device_buffer<std::int32_t> counters_;
 };
 
 // ---------------------------------------------------------------------------------------------

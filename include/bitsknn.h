@@ -67,6 +67,32 @@ int bitsknn_topk_bits_f32(const float* in, size_t in_row_stride, const int32_t* 
                           void* stream);
 
 /*
+ * bits-sq: bits top-k for few, long rows.  Every row of the contiguous rows x cols matrix is cut
+ * into `parts` equal parts that are selected by separate workgroups (labels shifted by the part's
+ * first column), and the parts * k pairs of a row are selected again with their labels.  Same
+ * result as bitsknn_topk_bits_f32 on the whole rows, bit for bit.
+ *
+ * Replaces single_query_bits::selection (src/topk/singlepass/bits_knn.cu:132-186: two launches of
+ * the bits kernel, the prefetching form, and populate_label_offsets_kernel :67-76).  The labels of
+ * a part are shifted inside the kernel.  With up to 1024 parts in all it is one launch: the
+ * workgroup that finishes the last part of a row (a counter per row in device memory) selects from
+ * the row's pairs itself.  With more parts, or where the pairs of a row would not start on a
+ * 16-byte boundary (parts * k not a multiple of 4), the second pass is a launch of its own.
+ *
+ *  in                     rows x cols, row stride cols; cols a multiple of parts
+ *  parts                  parts per row (1: as bitsknn_topk_bits_f32 with prefetch)
+ *  part_dist, part_label  rows * parts * k pairs of device memory for the parts' results
+ *  counters               rows int32 in device memory, zero before the first call; every call
+ *                         leaves them zero
+ *  out_dist, out_label    rows x k outputs, row stride out_row_stride (>= k)
+ *  k, block_size, items_per_thread as for bitsknn_topk_bits_f32, with its messages.
+ */
+int bitsknn_topk_bits_parts_f32(const float* in, size_t rows, size_t cols, uint32_t parts,
+                                float* part_dist, int32_t* part_label, int32_t* counters,
+                                float* out_dist, int32_t* out_label, size_t out_row_stride, uint32_t k,
+                                uint32_t block_size, uint32_t items_per_thread, void* stream);
+
+/*
  * partial-bitonic-regs: top-k of every row by sorting the row block after block in registers and
  * merging each sorted block into the running result, with no filtering of the input (the
  * baseline that the bits kernel's buffer and filter are measured against).  Same matrix and

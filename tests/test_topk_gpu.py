@@ -287,6 +287,43 @@ def test_row_split_like_bits_sq(bk, dev, oracle):
     assert np.array_equal(fd.cpu().numpy(), ed) and np.array_equal(fl.cpu().numpy(), el)
 
 
+@pytest.mark.parametrize("rows,n,parts,k,block,batch", [
+    (1, 1 << 18, 8, 64, 256, 16), (3, 1 << 16, 16, 32, 128, 4), (64, 1 << 15, 4, 16, 128, 8),
+    (5, 40960, 5, 100, 256, 8), (7, 30000, 3, 7, 512, 4), (2, 1 << 17, 32, 256, 512, 12),
+    (4, 1 << 16, 2, 2048, 512, 4), (9, 9 * 1001, 7, 33, 256, 16), (130, 4096, 2, 4, 128, 16),
+    (2, 1 << 19, 32, 2, 128, 4), (300, 1 << 14, 4, 8, 128, 8), (512, 8192, 2, 16, 256, 4)])
+def test_rows_cut_into_parts_in_one_launch(bk, dev, oracle, rows, n, parts, k, block, batch):
+    """bitsknn_topk_bits_parts_f32 (bits-sq: reference src/topk/singlepass/bits_knn.cu:132-186) against
+    the oracle's top-k of the whole rows, bit for bit, three calls in a row on the same scratch
+    memory (the counters must come back to zero).  Shapes with 16-byte loads and one launch, with
+    parts * k not a multiple of four or more than 1024 parts in all (second pass as its own launch)
+    and with parts that are not a multiple of four values (4-byte loads)."""
+    import torch
+    m = oracle.uniform_matrix(rows + parts + k, rows, n)
+    m[:, ::97] = m[:, 5:6]     # ties across the parts
+    t = torch.from_numpy(m).to(dev)
+    ed, el = oracle.topk(m, k)
+    scratch = {}
+    for call in range(3):
+        od, ol = bk.topk_bits_parts(t, k, parts, block, batch, scratch=scratch)
+        torch.cuda.synchronize()
+        assert np.array_equal(od.cpu().numpy().view(np.uint32), ed.view(np.uint32)), call
+        assert np.array_equal(ol.cpu().numpy(), el), call
+    (_, _, counters), = scratch.values()
+    assert int(counters.abs().sum()) == 0
+
+
+def test_rows_cut_into_parts_validation(bk, dev):
+    import torch
+    t = torch.zeros((2, 1000), device=dev)
+    with pytest.raises(bk.BitsKnnError, match="multiple of the parts"):
+        bk.topk_bits_parts(t, 4, 3)
+    with pytest.raises(bk.BitsKnnError, match="Unsupported block size: 64"):
+        bk.topk_bits_parts(t, 4, 2, 64)
+    with pytest.raises(bk.BitsKnnError, match="Unsupported k value: 4096"):
+        bk.topk_bits_parts(t, 4096, 2)
+
+
 def test_strided_output(bk, dev, oracle):
     import torch
     m = oracle.uniform_matrix(31, 5, 10000)
