@@ -30,10 +30,16 @@ EXPORTS = (
     "bitsknn_fused_workspace_bytes",
     "bitsknn_fused_l2_topk_f32_ws",
     "bitsknn_fused_l2_topk_f32_ex",
+    "bitsknn_fused_l2_topk_f32_tuned",
     "bitsknn_fused_static_scratch_bytes",
     "bitsknn_fused_l2_topk_f32_static",
     "bitsknn_fused_status",
 )
+
+
+class FusedTuning(ctypes.Structure):
+    """bitsknn_fused_tuning of include/bitsknn.h"""
+    _fields_ = [("ranges", ctypes.c_int32), ("first_radius", ctypes.c_int32), ("reserved", ctypes.c_int32 * 6)]
 
 
 class BitsKnnError(RuntimeError):
@@ -96,6 +102,9 @@ def lib():
         L.bitsknn_fused_static_scratch_bytes.argtypes = []
         L.bitsknn_fused_l2_topk_f32_static.restype = ctypes.c_int
         L.bitsknn_fused_l2_topk_f32_static.argtypes = L.bitsknn_fused_l2_topk_f32.argtypes
+        L.bitsknn_fused_l2_topk_f32_tuned.restype = ctypes.c_int
+        L.bitsknn_fused_l2_topk_f32_tuned.argtypes = [vp, vp, ctypes.c_int, i32, i32, vp, vp, ctypes.c_int,
+                                                      ctypes.c_int, ctypes.POINTER(FusedTuning), vp, sz, vp]
         L.bitsknn_fused_status.restype = ctypes.c_int
         L.bitsknn_fused_status.argtypes = [vp]
         _lib = L
@@ -232,13 +241,14 @@ FUSED_FP32, FUSED_BF16X3, FUSED_EXACT = 0, 1, 2
 
 
 def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1, dim_mult=1,
-                  out_dist=None, out_label=None, workspace=None, arithmetic=None):
+                  out_dist=None, out_label=None, workspace=None, arithmetic=None, tuning=None):
     """bits-fused: top-k of ||p||^2 - 2 q.p without materialising the distance matrix.
     workspace: None -> the plain entry point; "auto" -> allocate what
     bitsknn_fused_workspace_bytes asks for; "static" -> the entry point that uses the library's own
     scratch memory and allocates nothing; or a uint8 device tensor.
-    arithmetic: None -> the entry points with fp32 matrix instructions; FUSED_FP32 / FUSED_BF16X3
-    -> bitsknn_fused_l2_topk_f32_ex with that arithmetic."""
+    arithmetic: None -> the plain entry points (FUSED_EXACT); FUSED_FP32 / FUSED_BF16X3 /
+    FUSED_EXACT -> bitsknn_fused_l2_topk_f32_ex with that arithmetic.
+    tuning: None, or (ranges, first_radius) -> bitsknn_fused_l2_topk_f32_tuned."""
     import torch
     d, q = queries_dm.shape
     d2, n = points_dm.shape
@@ -252,7 +262,13 @@ def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1,
                                 device=queries_dm.device)
     head = (_ptr(queries_dm), _ptr(points_dm), d, q, n, _ptr(out_dist), _ptr(out_label), k,
             params[0], params[1], params[2], block_query_dim, dim_mult)
-    if isinstance(workspace, str) and workspace == "static":
+    if tuning is not None:
+        assert not isinstance(workspace, str)
+        knobs = FusedTuning(int(tuning[0]), int(tuning[1]), (ctypes.c_int32 * 6)())
+        _check(lib().bitsknn_fused_l2_topk_f32_tuned(*head[:8], FUSED_EXACT if arithmetic is None else int(arithmetic),
+                                                     ctypes.byref(knobs), _ptr(workspace),
+                                                     workspace.numel() if workspace is not None else 0, _stream()))
+    elif isinstance(workspace, str) and workspace == "static":
         assert arithmetic is None
         _check(lib().bitsknn_fused_l2_topk_f32_static(*head, _stream()))
     elif arithmetic is not None:

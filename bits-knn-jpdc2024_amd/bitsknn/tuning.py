@@ -234,6 +234,113 @@ def sweep_fused(repeats=3, shapes=FUSED_SHAPES, dims=FUSED_DIMS, k_values=FUSED_
                 progress(q, dim)
 
 
+# ---- launch parameters of the fused kernels (bitsknn_fused_tuning) -------------------------------
+FUSED_TUNING_COLUMNS = ("hostname", "GPU", "point_count", "query_count", "dim", "k", "arithmetic", "ranges",
+                        "first_radius", "time", "time_with_the_librarys_choice")
+DEFAULT_FUSED_TUNING = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fused_tuning.csv")
+FUSED_TUNING_SHAPES = ((1024, 1 << 20), (8192, 1 << 17), (65536, 1 << 20))
+FUSED_RANGES = (1, 2, 4, 8, 16, 32, 64)
+FUSED_FIRST_RADII = (-1, 64, 256)
+ARITHMETIC_NAMES = {0: "fp32-matrix", 1: "bf16x3", 2: "exact"}
+
+
+def sweep_fused_tuning(repeats=3, shapes=FUSED_TUNING_SHAPES, dims=FUSED_DIMS, k_values=(4, 16, 32, 64, 128, 256),
+                       arithmetics=(2, 0), seed=17, progress=None):
+    """Time bits-fused on cuda:0 over what bitsknn_fused_l2_topk_f32_tuned lets a caller choose: the
+    number of ranges the points are cut into and whether (and how densely) a sample of the points
+    gives the first radii, per arithmetic.  The counterpart of the reference's sweep over the
+    register tiling of its fused kernel (scripts/run-fused-cache-params.sh).  Yields one dict per
+    measurement; `ranges` 0 and `first_radius` 0 are the library's own choice."""
+    import torch
+    import bitsknn
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    for q, n in shapes:
+        for dim in dims:
+            points = torch.rand((dim, n), device=dev, generator=gen)
+            queries = torch.rand((dim, q), device=dev, generator=gen)
+            for k in k_values:
+                out_d = torch.empty((q, k), dtype=torch.float32, device=dev)
+                out_l = torch.empty((q, k), dtype=torch.int32, device=dev)
+                workspace = torch.empty(8 * q * 64 * k, dtype=torch.uint8, device=dev)
+                for arithmetic in arithmetics:
+                    choices = [(0, 0)]
+                    for ranges in FUSED_RANGES:
+                        # more workgroups than eight per compute unit gain nothing
+                        if ranges > 1 and (q // 128) * ranges > 2048:
+                            continue
+                        for first_radius in FUSED_FIRST_RADII:
+                            choices.append((ranges, first_radius))
+                    for ranges, first_radius in choices:
+                        def run():
+                            bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l,
+                                                  workspace=workspace, arithmetic=arithmetic,
+                                                  tuning=(ranges, first_radius))
+                        run()
+                        start = torch.cuda.Event(enable_timing=True)
+                        end = torch.cuda.Event(enable_timing=True)
+                        start.record()
+                        for _ in range(repeats):
+                            run()
+                        end.record()
+                        end.synchronize()
+                        yield {"point_count": n, "query_count": q, "dim": dim, "k": k,
+                               "arithmetic": ARITHMETIC_NAMES[arithmetic], "ranges": ranges,
+                               "first_radius": first_radius, "time": start.elapsed_time(end) / 1e3 / repeats}
+            if progress is not None:
+                progress(q, dim)
+    bitsknn.fused_status()
+
+
+def fused_optima(rows):
+    """The fastest (ranges, first_radius) per problem and arithmetic, with the time of the library's
+    own choice beside it."""
+    best = {}
+    own = {}
+    for row in rows:
+        key = (row["point_count"], row["query_count"], row["dim"], row["k"], row["arithmetic"])
+        if row["ranges"] == 0 and row["first_radius"] == 0:
+            own[key] = row["time"]
+        elif key not in best or row["time"] < best[key]["time"]:
+            best[key] = row
+    return [dict(best[key], time_with_the_librarys_choice=own.get(key, float("nan"))) for key in sorted(best)]
+
+
+def write_fused_tuning(rows, path, hostname="mi355x", gpu="MI355X"):
+    with open(path, "w", newline="") as handle:
+        writer = csv.writer(handle, lineterminator="\n")
+        writer.writerow(FUSED_TUNING_COLUMNS)
+        for row in rows:
+            full = dict(row, hostname=hostname, GPU=gpu)
+            for name in ("time", "time_with_the_librarys_choice"):
+                if name in full:
+                    full[name] = f"{full[name]:.10g}"
+            writer.writerow([full.get(name, "") for name in FUSED_TUNING_COLUMNS])
+
+
+def config_fused(query_count, point_count, dim, k, arithmetic="exact", tuning_file=DEFAULT_FUSED_TUNING):
+    """(ranges, first_radius) for bitsknn_fused_l2_topk_f32_tuned from the shipped measurements: the
+    row of the arithmetic whose problem is nearest to the request (sum of the absolute log ratios
+    of queries, points, dimension and list length); (0, 0), the library's choice, without a file."""
+    import math
+    best, best_cost = (0, 0), None
+    try:
+        with open(tuning_file, newline="") as handle:
+            for row in csv.DictReader(handle):
+                if row["arithmetic"] != arithmetic:
+                    continue
+                cost = sum(abs(math.log(float(row[name]) / float(want)))
+                           for name, want in (("query_count", query_count), ("point_count", point_count),
+                                              ("dim", dim), ("k", k)))
+                if best_cost is None or cost < best_cost:
+                    best, best_cost = (int(row["ranges"]), int(row["first_radius"])), cost
+    except OSError:
+        pass
+    return best
+
+
 def sweep_partial_bitonic(repeats=5, problem_size=1 << 30, query_counts=(64, 256, 1024, 4096),
                           k_values=(32, 64, 128, 256, 512, 1024, 2048), block_sizes=(64, 128, 256, 512),
                           seed=17, progress=None):
@@ -293,13 +400,21 @@ def main(argv=None):
     ap.add_argument("--all", default=None, help="also write every measurement to this CSV")
     ap.add_argument("--repeats", type=int, default=10)
     ap.add_argument("--hostname", default="mi355x")
-    ap.add_argument("--only", choices=("bits", "bits-sq", "partial-bitonic-regs", "fused-cache"), default=None,
-                    help="time one family only (bits covers bits and bits-prefetch)")
+    ap.add_argument("--only", choices=("bits", "bits-sq", "partial-bitonic-regs", "fused-cache", "fused-tuning"),
+                    default=None, help="time one family only (bits covers bits and bits-prefetch; fused-tuning: the "
+                                       "launch parameters of the fused kernels, into --fused-out)")
+    ap.add_argument("--fused-out", default=DEFAULT_FUSED_TUNING, help="fused tuning CSV to write")
     args = ap.parse_args(argv)
 
     def progress(q, k):
         print(f"q={q} k={k} done", file=sys.stderr, flush=True)
 
+    if args.only == "fused-tuning":
+        measured = list(sweep_fused_tuning(progress=progress))
+        if args.all:
+            write_fused_tuning(measured, args.all, args.hostname)
+        write_fused_tuning(fused_optima(measured), args.fused_out, args.hostname)
+        return 0
     rows = []
     if args.only in (None, "bits"):
         rows += list(sweep(repeats=args.repeats, progress=progress))

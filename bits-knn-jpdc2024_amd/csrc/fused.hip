@@ -129,11 +129,18 @@ int choose_splits(int q, int n)
 // from the whole point set (q = 8192, n = 2^17, d = 8: 2.66 -> 1.56 ms at k = 256, 1.31 -> 1.05 ms at
 // k = 128, 0.88 -> 0.78 ms at k = 64; q = 1024, n = 2^20: 2.68 -> 1.04, 1.32 -> 0.88, 0.89 -> 0.76 ms).
 // The sample launch runs on the few workgroups the queries give (it is not cut into ranges), so it
-// takes every 256th stage only.
+// takes about 2048 points whatever the point count (the constants below).
+// The sweep over bitsknn_fused_tuning (bitsknn/tuning.py, fused_tuning.csv) is where these come
+// from: with one range lists of 64 gain 1.5-4 % too (65536 queries x 2^20 points, d = 8: 9.63 ->
+// 9.22 ms), and over ranges the sample wants about 2048 points whatever the point count (8192 queries
+// x 2^17 points, k = 256: every 256th stage 2.05 ms, every 64th 1.38 ms; 1024 queries x 2^20 points
+// are best served by every 256th).
 constexpr int SAMPLE_SCALE = 64;
-constexpr int SAMPLE_SCALE_RANGES = 256;
+constexpr int SAMPLE_SCALE_RANGES_MIN = 64;
+constexpr int SAMPLE_SCALE_RANGES_MAX = 256;
+constexpr int SAMPLE_POINTS_RANGES = 2048;
 constexpr int SAMPLE_MIN_POINTS = 1 << 17; // at least 8 (2 with ranges) sampled stages of any size
-constexpr int SAMPLE_MIN_K = 128;
+constexpr int SAMPLE_MIN_K = 64;
 constexpr int SAMPLE_MIN_K_RANGES = 64; // (k <= 32: the three extra launches cost what the merges save)
 
 int first_radius_rank(int k, int scale)
@@ -199,9 +206,32 @@ size_t partial_list_bytes(std::int32_t q, int splits, int k)
 int fused_impl(const float* queries_dim_major, const float* points_dim_major, int dim, std::int32_t q,
                std::int32_t n, float* out_dist, std::int32_t* out_label, int k, int query_reg,
                int db_reg, int dim_reg, int block_query_dim, int dim_mult, int arithmetic,
-               void* workspace, size_t workspace_bytes, bool use_workspace, void* stream)
+               void* workspace, size_t workspace_bytes, bool use_workspace, void* stream,
+               const bitsknn_fused_tuning* tuning = nullptr)
 {
     clear_error();
+    if (tuning != nullptr)
+    {
+        if (tuning->ranges < 0 || tuning->ranges > 64)
+        {
+            return fail(BITSKNN_ERR_INVALID, "bitsknn_fused_tuning: ranges must be 0 (the library's choice) or 1 .. 64, got %d",
+                        tuning->ranges);
+        }
+        if (tuning->first_radius < -1 || tuning->first_radius == 1 || tuning->first_radius > 4096)
+        {
+            return fail(BITSKNN_ERR_INVALID,
+                        "bitsknn_fused_tuning: first_radius must be 0 (the library's choice), -1 (never) or 2 .. 4096 "
+                        "(one stage in every so many), got %d",
+                        tuning->first_radius);
+        }
+        for (const std::int32_t word : tuning->reserved)
+        {
+            if (word != 0)
+            {
+                return fail(BITSKNN_ERR_INVALID, "bitsknn_fused_tuning: reserved words must be zero");
+            }
+        }
+    }
     // the reference's nested dispatch, outermost first (fused_cache_knn.cu:72-144).  Its tuning
     // parameters describe a register tiling for the fp32 vector unit; they are validated like
     // there and have no effect on the tiling for the matrix cores, which is fixed by the
@@ -263,8 +293,13 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
 
     int splits = use_workspace && workspace != nullptr &&
                          reinterpret_cast<std::uintptr_t>(workspace) % 4 == 0
-                     ? choose_splits(q, n)
+                     ? (tuning != nullptr && tuning->ranges > 0 ? tuning->ranges : choose_splits(q, n))
                      : 1;
+    // (ranges of at least one stage of the largest geometry)
+    while (splits > 1 && n / splits < 256)
+    {
+        splits /= 2;
+    }
 
     while (splits > 1 && partial_list_bytes(q, splits, k) > workspace_bytes)
     {
@@ -307,10 +342,21 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
                                      128, 4, 0, stream);
     };
     hipError_t status = hipSuccess;
-    const int scale = splits == 1 ? SAMPLE_SCALE : SAMPLE_SCALE_RANGES;
-    const int rank = n >= SAMPLE_MIN_POINTS && k >= (splits == 1 ? SAMPLE_MIN_K : SAMPLE_MIN_K_RANGES)
-                         ? first_radius_rank(k, scale)
-                         : 0;
+    int scale = SAMPLE_SCALE;
+    if (splits > 1)
+    {
+        scale = n / SAMPLE_POINTS_RANGES;
+        scale = scale < SAMPLE_SCALE_RANGES_MIN ? SAMPLE_SCALE_RANGES_MIN
+                                                : (scale > SAMPLE_SCALE_RANGES_MAX ? SAMPLE_SCALE_RANGES_MAX : scale);
+    }
+    bool sample = n >= SAMPLE_MIN_POINTS && k >= (splits == 1 ? SAMPLE_MIN_K : SAMPLE_MIN_K_RANGES);
+    if (tuning != nullptr && tuning->first_radius != 0)
+    {
+        // the caller's choice, as far as the sample has at least two stages of any geometry
+        sample = tuning->first_radius > 0 && n / tuning->first_radius >= 512;
+        scale = sample ? tuning->first_radius : scale;
+    }
+    const int rank = sample ? first_radius_rank(k, scale) : 0;
     if (rank > 0)
     {
         // lists of min(k, 32) nearest sample points into the first entries of the caller's output
@@ -396,6 +442,17 @@ extern "C" int bitsknn_fused_l2_topk_f32_ex(const float* queries_dim_major,
     return bitsknn::fused_impl(queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, k,
                                query_reg, db_reg, dim_reg, block_query_dim, dim_mult, arithmetic, workspace,
                                workspace_bytes, workspace != nullptr, stream);
+}
+
+extern "C" int bitsknn_fused_l2_topk_f32_tuned(const float* queries_dim_major,
+                                               const float* points_dim_major, int dim, int32_t q,
+                                               int32_t n, float* out_dist, int32_t* out_label, int k,
+                                               int arithmetic, const bitsknn_fused_tuning* tuning,
+                                               void* workspace, size_t workspace_bytes, void* stream)
+{
+    // (the reference's five parameters at the values of its fixed choice: they only have to be valid)
+    return bitsknn::fused_impl(queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, k, 2, 4, 1, 1,
+                               1, arithmetic, workspace, workspace_bytes, workspace != nullptr, stream, tuning);
 }
 
 extern "C" size_t bitsknn_fused_static_scratch_bytes(void) { return bitsknn::STATIC_SCRATCH_BYTES; }

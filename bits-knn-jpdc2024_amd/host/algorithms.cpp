@@ -3,6 +3,8 @@
 #include "knn.hpp"
 
 #include <algorithm>
+#include <cstdio>
+#include <cstdlib>
 #include <stdexcept>
 #include <utility>
 
@@ -392,12 +394,15 @@ private:
 class fused_cache_knn : public device_knn
 {
 public:
-    // arithmetic: BITSKNN_FUSED_FP32 (the reference's id) or BITSKNN_FUSED_BF16X3
-    explicit fused_cache_knn(int arithmetic = BITSKNN_FUSED_FP32) : arithmetic_(arithmetic) {}
+    // arithmetic: BITSKNN_FUSED_EXACT (the reference's id: its arithmetic), BITSKNN_FUSED_FP32 or
+    // BITSKNN_FUSED_BF16X3
+    explicit fused_cache_knn(int arithmetic = BITSKNN_FUSED_EXACT) : arithmetic_(arithmetic) {}
 
     std::string id() const override
     {
-        return arithmetic_ == BITSKNN_FUSED_BF16X3 ? "fused-cache-bf16x3" : "fused-cache";
+        return arithmetic_ == BITSKNN_FUSED_BF16X3 ? "fused-cache-bf16x3"
+               : arithmetic_ == BITSKNN_FUSED_FP32 ? "fused-cache-mfma"
+                                                   : "fused-cache";
     }
 
     void initialize(const knn_args& args) override
@@ -410,10 +415,28 @@ public:
         const auto queries = to_dim_major(args_.queries, query_count(), dim(), args_.queries_layout);
         points_ = device_buffer<float>{points.size()};
         queries_ = device_buffer<float>{queries.size()};
-        // partial lists of the point ranges when the queries alone do not fill the GPU
-        workspace_ = device_buffer<unsigned char>{bitsknn_fused_workspace_bytes(
-            static_cast<std::int32_t>(query_count()), static_cast<std::int32_t>(point_count()),
-            static_cast<int>(k()))};
+        // BITSKNN_FUSED_TUNING="ranges=R,first_radius=F" in the environment: the launch parameters a
+        // tuning sweep varies here (bitsknn_fused_tuning), in place of the library's own choice
+        tuned_ = false;
+        tuning_ = bitsknn_fused_tuning{};
+        if (const char* text = std::getenv("BITSKNN_FUSED_TUNING"); text != nullptr && *text != '\0')
+        {
+            int ranges = 0;
+            int first_radius = 0;
+            if (std::sscanf(text, "ranges=%d,first_radius=%d", &ranges, &first_radius) != 2)
+            {
+                throw std::runtime_error("BITSKNN_FUSED_TUNING must read ranges=R,first_radius=F");
+            }
+            tuning_.ranges = ranges;
+            tuning_.first_radius = first_radius;
+            tuned_ = true;
+        }
+        // partial lists of the point ranges when the queries alone do not fill the GPU (room for the
+        // 64 ranges a tuning may ask for)
+        workspace_ = device_buffer<unsigned char>{
+            tuned_ ? query_count() * 64 * k() * 8
+                   : bitsknn_fused_workspace_bytes(static_cast<std::int32_t>(query_count()),
+                                                   static_cast<std::int32_t>(point_count()), static_cast<int>(k()))};
         transfer_in_.start();
         points_.upload(points.data(), points.size());
         queries_.upload(queries.data(), queries.size());
@@ -425,13 +448,32 @@ public:
 
     void selection() override
     {
-        BITSKNN_CHECK(bitsknn_fused_l2_topk_f32_ex(
-            queries_.data(), points_.data(), static_cast<int>(dim()), static_cast<std::int32_t>(query_count()),
-            static_cast<std::int32_t>(point_count()), out_dist_.data(), out_label_.data(),
-            static_cast<int>(k()), static_cast<int>(args_.items_per_thread[0]),
-            static_cast<int>(args_.items_per_thread[1]), static_cast<int>(args_.items_per_thread[2]),
-            static_cast<int>(args_.selection_block_size), static_cast<int>(args_.deg), arithmetic_,
-            workspace_.size() != 0 ? workspace_.data() : nullptr, workspace_.size(), nullptr));
+        if (tuned_)
+        {
+            // the reference's parameters are validated with its messages (no queries: nothing runs),
+            // then the launch parameters of this implementation are the ones from the environment
+            BITSKNN_CHECK(bitsknn_fused_l2_topk_f32_ex(
+                queries_.data(), points_.data(), static_cast<int>(dim()), 0, static_cast<std::int32_t>(point_count()),
+                out_dist_.data(), out_label_.data(), static_cast<int>(k()), static_cast<int>(args_.items_per_thread[0]),
+                static_cast<int>(args_.items_per_thread[1]), static_cast<int>(args_.items_per_thread[2]),
+                static_cast<int>(args_.selection_block_size), static_cast<int>(args_.deg), arithmetic_, nullptr, 0,
+                nullptr));
+            BITSKNN_CHECK(bitsknn_fused_l2_topk_f32_tuned(
+                queries_.data(), points_.data(), static_cast<int>(dim()), static_cast<std::int32_t>(query_count()),
+                static_cast<std::int32_t>(point_count()), out_dist_.data(), out_label_.data(), static_cast<int>(k()),
+                arithmetic_, &tuning_, workspace_.size() != 0 ? workspace_.data() : nullptr, workspace_.size(),
+                nullptr));
+        }
+        else
+        {
+            BITSKNN_CHECK(bitsknn_fused_l2_topk_f32_ex(
+                queries_.data(), points_.data(), static_cast<int>(dim()), static_cast<std::int32_t>(query_count()),
+                static_cast<std::int32_t>(point_count()), out_dist_.data(), out_label_.data(),
+                static_cast<int>(k()), static_cast<int>(args_.items_per_thread[0]),
+                static_cast<int>(args_.items_per_thread[1]), static_cast<int>(args_.items_per_thread[2]),
+                static_cast<int>(args_.selection_block_size), static_cast<int>(args_.deg), arithmetic_,
+                workspace_.size() != 0 ? workspace_.data() : nullptr, workspace_.size(), nullptr));
+        }
         // synchronises, and fails if a wave of the kernel gave up a wait for a stage
         BITSKNN_CHECK(bitsknn_fused_status(nullptr));
     }
@@ -440,6 +482,8 @@ public:
 
 private:
     int arithmetic_;
+    bool tuned_ = false;
+    bitsknn_fused_tuning tuning_{};
     device_buffer<float> points_;
     device_buffer<float> queries_;
     device_buffer<unsigned char> workspace_;
@@ -507,6 +551,7 @@ std::vector<std::unique_ptr<knn>> make_algorithms()
     algorithms.push_back(std::make_unique<bits_knn>(true));
     algorithms.push_back(std::make_unique<single_query_bits>());
     algorithms.push_back(std::make_unique<partial_bitonic_regs>());
+    algorithms.push_back(std::make_unique<fused_cache_knn>(BITSKNN_FUSED_EXACT));
     algorithms.push_back(std::make_unique<fused_cache_knn>(BITSKNN_FUSED_FP32));
     algorithms.push_back(std::make_unique<fused_cache_knn>(BITSKNN_FUSED_BF16X3));
     algorithms.push_back(std::make_unique<two_pass_knn>());

@@ -174,7 +174,10 @@ int bitsknn_dist_f32(int op, int dim, size_t q, size_t n, const float* queries_d
  *                             messages; dim must be >= dim_mult*dim_reg as there.  Accepted for
  *                             compatibility only: they describe a register tiling for the fp32
  *                             vector unit and do not change the matrix-core kernel, so a sweep
- *                             over them measures the same kernel every time
+ *                             over them measures the same kernel every time (what a sweep can
+ *                             vary here: bitsknn_fused_l2_topk_f32_tuned)
+ * The distances are computed in the reference's arithmetic (BITSKNN_FUSED_EXACT below) for
+ * dim <= 64 and on the fp32 matrix instructions beyond.
  * A call enqueues one to three kernels on `stream` (long lists over many points are preceded by a
  * pass over a sample of the points, which gives every query a first radius, and followed by one
  * that repeats the queries whose first radius proved too low); until the last of them has run,
@@ -191,7 +194,7 @@ int bitsknn_fused_l2_topk_f32(const float* queries_dim_major, const float* point
  * still the fused kernel: no distance is written to memory.  When there are too few queries to
  * fill the GPU with one workgroup per 128 queries, the points are cut into ranges that are
  * searched by separate workgroups; their partial lists (k pairs per query and range) go to the
- * workspace and a bits pass (explicit labels) selects the final k.  Same distances bit for bit.
+ * workspace and a bits pass (explicit labels) selects the final k.  Same lists bit for bit.
  *
  * No counterpart in the reference, whose fused kernel always runs one thread block per query tile
  * (src/topk/singlepass/fused_cache_knn.cu:60-69); the host wrapper that owns the device memory
@@ -212,15 +215,25 @@ int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major, const float* po
  * bits-fused with the arithmetic of the products q.p chosen per call (nothing process-wide is
  * read); workspace may be NULL (then as bitsknn_fused_l2_topk_f32) or as for
  * bitsknn_fused_l2_topk_f32_ws.
- *   BITSKNN_FUSED_FP32    fp32 matrix instructions (v_mfma_f32_32x32x2_f32); what the two entry
- *                         points above use.
+ *   BITSKNN_FUSED_EXACT   what the entry points above use.  For dim <= 64 every reported distance
+ *                         is computed as the reference's kernel computes it -- norm and dot
+ *                         product by sequential fused multiply-adds over the dimensions in order,
+ *                         then norm - 2 dot (include/bits/topk/singlepass/
+ *                         fused_cache_kernel_structs.cuh:457-522, :622-631) -- so the lists equal
+ *                         the reference arithmetic's bit for bit, equal distances by lower index.
+ *                         Which pairs to compute is decided by a filter on the bf16 matrix
+ *                         instructions (v_mfma_f32_32x32x16_bf16, two bf16 pieces per operand, three
+ *                         products) whose value is a guaranteed lower bound of the distance less a
+ *                         slack of 2^-13 ||q||^2: no pair below a query's current k-th distance is
+ *                         ever dropped.  Larger dimensions use BITSKNN_FUSED_FP32.
+ *   BITSKNN_FUSED_FP32    every distance from fp32 matrix instructions (v_mfma_f32_32x32x2_f32):
+ *                         within 1e-5 of the reference arithmetic, not bit-identical to it.
  *   BITSKNN_FUSED_BF16X3  for 9 <= dim <= 64: every fp32 operand is cut exactly into three bf16
  *                         pieces and a product is the fp32 sum of six bf16 products on the bf16
- *                         matrix path (v_mfma_f32_32x32x16_bf16); what is left out is below 2^-23
- *                         of a product, the size of one fp32 rounding.  Other dimensions use
- *                         BITSKNN_FUSED_FP32.
- * No counterpart in the reference, whose fused kernel multiplies on the fp32 vector unit
- * (include/bits/topk/singlepass/fused_cache_kernel_structs.cuh:457-522).
+ *                         matrix path; what is left out is below 2^-23 of a product, the size of
+ *                         one fp32 rounding.  Other dimensions use BITSKNN_FUSED_FP32.
+ * The reference's fused kernel multiplies on the fp32 vector unit
+ * (fused_cache_kernel_structs.cuh:457-522); the last two have no counterpart there.
  * BITSKNN_ERR_INVALID for another value of `arithmetic`.
  */
 #define BITSKNN_FUSED_FP32 0
@@ -231,6 +244,39 @@ int bitsknn_fused_l2_topk_f32_ex(const float* queries_dim_major, const float* po
                                  int k, int query_reg, int db_reg, int dim_reg, int block_query_dim,
                                  int dim_mult, int arithmetic, void* workspace, size_t workspace_bytes,
                                  void* stream);
+
+/*
+ * bits-fused with the launch parameters of this implementation in the caller's hands: what a tuning
+ * sweep varies here.  The reference tunes its fused kernel over a register tiling (QUERY_REG,
+ * DB_REG, DIM_REG, BLOCK_QUERY_DIM, DIM_MULT: src/topk/singlepass/fused_cache_knn.cu:39-145,
+ * scripts/run-fused-cache-params.sh); the matrix-core kernels here have no such tiling to choose,
+ * and what does change their time is chosen per call by rules measured on one machine:
+ *   arithmetic    as for bitsknn_fused_l2_topk_f32_ex (the plain entry points take
+ *                 BITSKNN_FUSED_EXACT)
+ *   ranges        how many ranges the points are cut into (separate workgroups per range, partial
+ *                 lists of 8*q*ranges*k bytes in the workspace, one bits pass at the end); 0 = the
+ *                 library's choice (enough workgroups for two per compute unit, at most 64); fewer
+ *                 are used when the workspace is smaller or the ranges would fall below 256 points
+ *   first_radius  whether the lists start from radii taken from a launch over a sample of the points
+ *                 (one stage in every first_radius, 2 .. 4096; -1: never; 0: the library's choice,
+ *                 lists of 128 and more on at least 2^17 points, of 64 and more over ranges); a
+ *                 sample whose lists would not reach the rank the guarantee needs is not taken
+ * tuning == NULL: the library's choices.  Results do not depend on the tuning (for
+ * BITSKNN_FUSED_EXACT bit for bit; for the other arithmetics the distances of a point can differ in
+ * the last bit between one range and several).  bitsknn/tuning.py sweeps these and records the
+ * best per problem.  Errors as for bitsknn_fused_l2_topk_f32_ex, plus BITSKNN_ERR_INVALID for
+ * values outside the ranges above or non-zero reserved words.
+ */
+typedef struct bitsknn_fused_tuning
+{
+    int32_t ranges;
+    int32_t first_radius;
+    int32_t reserved[6];
+} bitsknn_fused_tuning;
+int bitsknn_fused_l2_topk_f32_tuned(const float* queries_dim_major, const float* points_dim_major,
+                                    int dim, int32_t q, int32_t n, float* out_dist, int32_t* out_label,
+                                    int k, int arithmetic, const bitsknn_fused_tuning* tuning,
+                                    void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * bitsknn_fused_l2_topk_f32_ws for callers that cannot allocate device memory (code under HIP

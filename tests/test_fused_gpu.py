@@ -368,7 +368,7 @@ def _sampled_points(n, d, small_stages, scale):
                            for s in range(stages)])
 
 
-@pytest.mark.parametrize("d,k,mode,ranges", [(8, 128, "mfma", False), (8, 256, "mfma", False),
+@pytest.mark.parametrize("d,k,mode,ranges", [(8, 64, "default", False), (8, 128, "mfma", False), (8, 256, "mfma", False),
                                              (32, 256, "mfma", False), (100, 128, "default", False),
                                              (8, 128, "default", False), (8, 256, "default", False),
                                              (32, 256, "default", False), (64, 128, "default", False),
@@ -396,7 +396,8 @@ def test_first_radius_from_a_sample(bk, dev, oracle, d, k, mode, ranges):
     gd, gl = _fused(bk, dev, points, queries, k, arithmetic=arithmetic, workspace=workspace)
     _check(oracle, points, queries, k, gd, gl, bits=bits)
     assert not np.isnan(gd).any()
-    sample = _sampled_points(n, d, mode == "bf16x3" or bits, 256 if ranges else 64)
+    # (over ranges the sample has about 2048 points: one stage in every 64 .. 256)
+    sample = _sampled_points(n, d, mode == "bf16x3" or bits, max(64, min(256, n // 2048)) if ranges else 64)
     assert sample.size >= 2 * 32
     points = rng.random((n, d), dtype=np.float32)
     points[:, :4] += 1.0                    # all points a step away in four dimensions ...
@@ -554,3 +555,33 @@ def test_a_wait_that_gives_up_is_reported(bk, dev):
     assert done.returncode == 0, (done.stdout, done.stderr)
     assert done.stdout.strip().endswith("ok"), done.stdout
     bk.fused_status()  # this process, with the default limit, has seen no wait give up
+
+
+def test_tuned_entry_point(bk, dev, oracle):
+    """bitsknn_fused_l2_topk_f32_tuned: the number of ranges and the sample for the first radii are
+    the caller's; the result is the same whatever they are (bit for bit in the default arithmetic),
+    and values outside their ranges are rejected."""
+    import torch
+    n, q, d, k = (1 << 17) + 300, 260, 12, 64
+    p, s = oracle.generate(404, n, q, d)
+    pd = torch.from_numpy(np.ascontiguousarray(p.T)).to(dev)
+    qd = torch.from_numpy(np.ascontiguousarray(s.T)).to(dev)
+    ed, el = oracle.topk(oracle.dist(s, p, "partial"), k)
+    space = torch.empty(8 * q * 64 * k, dtype=torch.uint8, device=dev)
+    for ranges, first_radius in [(0, 0), (1, -1), (1, 64), (2, -1), (8, 256), (64, 64), (3, 32), (64, 4096)]:
+        od, ol = bk.fused_l2_topk(qd, pd, k, workspace=space, tuning=(ranges, first_radius))
+        bk.fused_status()
+        assert np.array_equal(od.cpu().numpy().view(np.uint32), ed.view(np.uint32)), (ranges, first_radius)
+        assert np.array_equal(ol.cpu().numpy(), el), (ranges, first_radius)
+    # the fp32 matrix instructions through the same entry point, to the tolerance
+    od, ol = bk.fused_l2_topk(qd, pd, k, workspace=space, tuning=(4, 64), arithmetic=bk.FUSED_FP32)
+    bk.fused_status()
+    _check(oracle, p, s, k, od.cpu().numpy(), ol.cpu().numpy())
+    # without a workspace there is one range whatever is asked for
+    od, ol = bk.fused_l2_topk(qd, pd, k, tuning=(16, -1))
+    bk.fused_status()
+    assert np.array_equal(ol.cpu().numpy(), el)
+    for bad, message in (((65, 0), "ranges must be"), ((-1, 0), "ranges must be"), ((0, 1), "first_radius must be"),
+                         ((0, -2), "first_radius must be"), ((0, 5000), "first_radius must be")):
+        with pytest.raises(bk.BitsKnnError, match=message):
+            bk.fused_l2_topk(qd, pd, k, workspace=space, tuning=bad)

@@ -15,9 +15,9 @@ HEADER = ("algorithm,generator,preprocessor,iteration,point_count,query_count,di
 PHASES = ["prepare", "transfer-in", "distances", "selection", "postprocessing", "finish", "transfer-out"]
 
 
-def run(*args, timeout=300):
+def run(*args, timeout=300, env=None):
     assert os.path.exists(KNN), "build the driver with `make -C bits-knn-jpdc2024_amd knn`"
-    return subprocess.run([KNN, *args], capture_output=True, text=True, timeout=timeout)
+    return subprocess.run([KNN, *args], capture_output=True, text=True, timeout=timeout, env=env)
 
 
 def checksums(proc):
@@ -37,7 +37,7 @@ def test_help_lists_options_and_algorithms_on_stderr():
     p = run("--help")
     assert p.returncode == 0 and p.stdout == ""
     for token in ("--algorithm", "--items-per-thread", "--point-layout", "--deg", "--no-output",
-                  "Available algorithms:", "- bits", "- bits-prefetch", "- bits-sq", "- fused-cache", "- fused-cache-bf16x3",
+                  "Available algorithms:", "- bits", "- bits-prefetch", "- bits-sq", "- fused-cache", "- fused-cache-mfma", "- fused-cache-bf16x3",
                   "- magma-dist", "- magma-part-dist", "- magma-part-dist-bf16x3", "- cublas-dist", "- serial", "- parallel"):
         assert token in p.stderr
 
@@ -142,19 +142,40 @@ def test_golden_fused_checksums_end_to_end(golden):
 
 
 @pytest.mark.gpu
-def test_golden_fused_checksums_with_bf16x3_products(golden):
+@pytest.mark.parametrize("algorithm", ["fused-cache-bf16x3", "fused-cache-mfma"])
+def test_golden_fused_checksums_with_the_other_arithmetics(golden, algorithm):
     """The reference's own checksums for d = 16 (the dimension of its fused runs that takes the
-    bf16 pieces), reproduced with the other arithmetic of the products."""
+    bf16 pieces), reproduced with the other arithmetics of the products."""
     done = 0
     for rec in golden:
         if rec["family"] != "fused" or rec["d"] != 16 or (rec["n"], rec["q"]) != (131072, 8192) or rec["k"] not in (16, 32):
             continue
-        p = run("-a", "fused-cache-bf16x3", "-n", "128k", "-q", "8k", "-d", "16", "-k", str(rec["k"]),
+        p = run("-a", algorithm, "-n", "128k", "-q", "8k", "-d", "16", "-k", str(rec["k"]),
                 "--seed", "24", "--items-per-thread", "8,4,2", "--block-size", "1", "--deg", "1")
         assert p.returncode == 0, p.stderr
         assert str(checksums(p)[0]) in rec["checksums"], (rec, checksums(p))
         done += 1
     assert done == 2
+
+
+@pytest.mark.gpu
+def test_fused_launch_parameters_from_the_environment(golden):
+    """BITSKNN_FUSED_TUNING hands the driver's fused run the launch parameters a tuning sweep varies;
+    the checksum of the reference's run must come out whatever they are, and the reference's own
+    parameters are still validated."""
+    import os
+    rec = next(r for r in golden if r["family"] == "fused" and (r["n"], r["q"], r["d"], r["k"]) == (131072, 8192, 8, 64))
+    args = ("-a", "fused-cache", "-n", "128k", "-q", "8k", "-d", "8", "-k", "64", "--seed", "24",
+            "--items-per-thread", "8,4,2", "--block-size", "1", "--deg", "1")
+    for tuning in ("ranges=1,first_radius=-1", "ranges=16,first_radius=64", "ranges=0,first_radius=0"):
+        p = run(*args, env=dict(os.environ, BITSKNN_FUSED_TUNING=tuning))
+        assert p.returncode == 0, p.stderr
+        assert str(checksums(p)[0]) in rec["checksums"], (tuning, checksums(p))
+    p = run(*args[:-6], "--items-per-thread", "3,4,2", "--block-size", "1", "--deg", "1",
+            env=dict(os.environ, BITSKNN_FUSED_TUNING="ranges=2,first_radius=-1"))
+    assert p.returncode != 0 and "Unsupported queries_reg value: 3" in p.stderr
+    p = run(*args, env=dict(os.environ, BITSKNN_FUSED_TUNING="ranges=99,first_radius=0"))
+    assert p.returncode != 0 and "ranges must be" in p.stderr
 
 
 @pytest.mark.gpu
