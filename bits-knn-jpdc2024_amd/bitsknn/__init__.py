@@ -26,6 +26,8 @@ EXPORTS = (
     "bitsknn_fill_f32",
     "bitsknn_stream_read_f32",
     "bitsknn_dist_f32",
+    "bitsknn_dist_layout_workspace_bytes",
+    "bitsknn_dist_layout_f32",
     "bitsknn_fused_l2_topk_f32",
     "bitsknn_fused_workspace_bytes",
     "bitsknn_fused_l2_topk_f32_ws",
@@ -84,6 +86,11 @@ def lib():
         L.bitsknn_stream_read_f32.argtypes = [vp, sz, sz, sz, vp, vp]
         L.bitsknn_dist_f32.restype = ctypes.c_int
         L.bitsknn_dist_f32.argtypes = [ctypes.c_int, ctypes.c_int, sz, sz, vp, sz, vp, sz, vp, sz, vp]
+        L.bitsknn_dist_layout_workspace_bytes.restype = ctypes.c_size_t
+        L.bitsknn_dist_layout_workspace_bytes.argtypes = [ctypes.c_int, sz, sz, ctypes.c_int, ctypes.c_int]
+        L.bitsknn_dist_layout_f32.restype = ctypes.c_int
+        L.bitsknn_dist_layout_f32.argtypes = [ctypes.c_int, ctypes.c_int, sz, sz, vp, ctypes.c_int, sz, vp,
+                                              ctypes.c_int, sz, vp, sz, vp, sz, vp]
         L.bitsknn_fused_l2_topk_f32.restype = ctypes.c_int
         L.bitsknn_fused_l2_topk_f32.argtypes = [vp, vp, ctypes.c_int, i32, i32, vp, vp, ctypes.c_int,
                                                 ctypes.c_int, ctypes.c_int, ctypes.c_int,
@@ -234,6 +241,26 @@ def distances(queries_dm, points_dm, op=DIST_L2, out=None):
     _check(lib().bitsknn_dist_f32(op, d, q, n, _ptr(queries_dm), _row_stride(queries_dm),
                                   _ptr(points_dm), _row_stride(points_dm), _ptr(out),
                                   _row_stride(out), _stream()))
+    return out
+
+
+LAYOUT_ROW_MAJOR, LAYOUT_COLUMN_MAJOR = 0, 1
+
+
+def distances_layout(queries, queries_layout, points, points_layout, op=DIST_L2, out=None):
+    """Distance matrix q x n from 2-D float32 device tensors in the caller's layout: LAYOUT_ROW_MAJOR
+    (count x dim, the vectors one after the other) or LAYOUT_COLUMN_MAJOR (dim x count)."""
+    import torch
+    q, d = queries.shape if queries_layout == LAYOUT_ROW_MAJOR else queries.shape[::-1]
+    n, d2 = points.shape if points_layout == LAYOUT_ROW_MAJOR else points.shape[::-1]
+    assert d == d2
+    if out is None:
+        out = torch.empty((q, n), dtype=torch.float32, device=queries.device)
+    need = int(lib().bitsknn_dist_layout_workspace_bytes(d, q, n, queries_layout, points_layout))
+    workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=queries.device)
+    _check(lib().bitsknn_dist_layout_f32(op, d, q, n, _ptr(queries), queries_layout, _row_stride(queries),
+                                         _ptr(points), points_layout, _row_stride(points), _ptr(out),
+                                         _row_stride(out), _ptr(workspace), need, _stream()))
     return out
 
 

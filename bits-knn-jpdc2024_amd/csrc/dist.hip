@@ -16,6 +16,8 @@
 
 #include <type_traits>
 
+#include <initializer_list>
+
 #include "common.hpp"
 #include "dist_split.hpp"
 
@@ -887,8 +889,138 @@ bool launch_resident(int dim, size_t q, size_t n, const float* queries, size_t q
     return plain(0, q_full, n_full) && plain(q_full, q, 0);
 }
 
+// Vectors given one after the other (component t of vector v at in[v * in_stride + t]) into the
+// dim-major form the distance kernels read (out[t * out_stride + v]): 32 x 32 tiles through LDS, so
+// that both sides are accessed in runs of consecutive addresses.
+__global__ void __launch_bounds__(256) to_dim_major_kernel(const float* __restrict__ in, size_t in_stride,
+                                                           float* __restrict__ out, size_t out_stride,
+                                                           size_t count, int dim)
+{
+    __shared__ float tile[32][33];
+    const int tx = static_cast<int>(threadIdx.x) & 31;
+    const int ty = static_cast<int>(threadIdx.x) >> 5; // 0 .. 7
+    const size_t v0 = static_cast<size_t>(blockIdx.x) * 32;
+    const int t0 = static_cast<int>(blockIdx.y) * 32;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+    {
+        const size_t v = v0 + ty + 8 * i;
+        const int t = t0 + tx;
+        tile[ty + 8 * i][tx] = v < count && t < dim ? in[v * in_stride + t] : 0.0F;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+    {
+        const int t = t0 + ty + 8 * i;
+        const size_t v = v0 + tx;
+        if (t < dim && v < count)
+        {
+            out[static_cast<size_t>(t) * out_stride + v] = tile[tx][ty + 8 * i];
+        }
+    }
+}
+
+// row stride of a dim-major copy in the workspace: the count rounded up to whole 16-byte pieces
+size_t padded_count(size_t count) { return (count + 3) / 4 * 4; }
+
 } // namespace
 } // namespace bitsknn
+
+extern "C" size_t bitsknn_dist_layout_workspace_bytes(int dim, size_t q, size_t n, int queries_layout,
+                                                      int points_layout)
+{
+    using namespace bitsknn;
+    if (dim <= 0)
+    {
+        return 0;
+    }
+    size_t floats = 0;
+    if (queries_layout == BITSKNN_LAYOUT_ROW_MAJOR)
+    {
+        floats += static_cast<size_t>(dim) * padded_count(q);
+    }
+    if (points_layout == BITSKNN_LAYOUT_ROW_MAJOR)
+    {
+        floats += static_cast<size_t>(dim) * padded_count(n);
+    }
+    return floats * sizeof(float);
+}
+
+extern "C" int bitsknn_dist_layout_f32(int op, int dim, size_t q, size_t n, const float* queries,
+                                       int queries_layout, size_t query_stride, const float* points,
+                                       int points_layout, size_t point_stride, float* dist,
+                                       size_t dist_row_stride, void* workspace, size_t workspace_bytes,
+                                       void* stream)
+{
+    using namespace bitsknn;
+    clear_error();
+    for (const int layout : {queries_layout, points_layout})
+    {
+        if (layout != BITSKNN_LAYOUT_ROW_MAJOR && layout != BITSKNN_LAYOUT_COLUMN_MAJOR)
+        {
+            return fail(BITSKNN_ERR_INVALID, "bitsknn_dist_layout_f32: unknown layout %d", layout);
+        }
+    }
+    if (dim <= 0)
+    {
+        return fail(BITSKNN_ERR_INVALID, "bitsknn_dist_f32: dimension must be positive, got %d", dim);
+    }
+    if (q == 0 || n == 0)
+    {
+        return BITSKNN_OK;
+    }
+    if (queries == nullptr || points == nullptr)
+    {
+        return fail(BITSKNN_ERR_INVALID, "bitsknn_dist_f32: null pointer");
+    }
+    const size_t need = bitsknn_dist_layout_workspace_bytes(dim, q, n, queries_layout, points_layout);
+    if (need != 0 && (workspace == nullptr || workspace_bytes < need ||
+                      reinterpret_cast<std::uintptr_t>(workspace) % 16 != 0))
+    {
+        return fail(BITSKNN_ERR_INVALID,
+                    "bitsknn_dist_layout_f32: vectors given one after the other need a 16-byte aligned workspace of "
+                    "%zu bytes (bitsknn_dist_layout_workspace_bytes), got %zu",
+                    need, workspace_bytes);
+    }
+    auto* hip_stream = static_cast<hipStream_t>(stream);
+    auto* next = static_cast<float*>(workspace);
+    // the dim-major operand of the kernels: the caller's array as it is, or its copy in the workspace
+    auto dim_major = [&](const float*& base, int layout, size_t& stride, size_t count) -> int {
+        if (layout == BITSKNN_LAYOUT_COLUMN_MAJOR)
+        {
+            return BITSKNN_OK;
+        }
+        if (stride < static_cast<size_t>(dim))
+        {
+            return fail(BITSKNN_ERR_INVALID, "bitsknn_dist_layout_f32: stride smaller than the dimension");
+        }
+        const size_t tiles = (count + 31) / 32;
+        if (tiles > 0x7FFFFFFFULL || (dim + 31) / 32 > 65535)
+        {
+            return fail(BITSKNN_ERR_INVALID, "bitsknn_dist_layout_f32: too many vectors for one launch: %zu", count);
+        }
+        const size_t out_stride = padded_count(count);
+        hipLaunchKernelGGL(to_dim_major_kernel, dim3(static_cast<unsigned>(tiles), static_cast<unsigned>((dim + 31) / 32)),
+                           dim3(256), 0, hip_stream, base, stride, next, out_stride, count, dim);
+        BITSKNN_HIP_CHECK(hipGetLastError());
+        base = next;
+        stride = out_stride;
+        next += static_cast<size_t>(dim) * out_stride;
+        return BITSKNN_OK;
+    };
+    int status = dim_major(queries, queries_layout, query_stride, q);
+    if (status != BITSKNN_OK)
+    {
+        return status;
+    }
+    status = dim_major(points, points_layout, point_stride, n);
+    if (status != BITSKNN_OK)
+    {
+        return status;
+    }
+    return bitsknn_dist_f32(op, dim, q, n, queries, query_stride, points, point_stride, dist, dist_row_stride, stream);
+}
 
 extern "C" int bitsknn_dist_f32(int op, int dim, size_t q, size_t n, const float* queries_dim_major,
                                 size_t query_stride, const float* points_dim_major,

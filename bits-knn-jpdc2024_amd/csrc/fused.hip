@@ -286,10 +286,8 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     {
         return fail(BITSKNN_ERR_INVALID, "bitsknn_fused_l2_topk_f32: null pointer");
     }
-    if (static_cast<size_t>(q) > 65535U * FQ_QB)
-    {
-        return fail(BITSKNN_ERR_INVALID, "bitsknn_fused_l2_topk_f32: too many queries: %d", q);
-    }
+    // (any int32 query count, as in the reference, fused_cache_kernel_structs.cuh:698-702: the
+    // workgroups of 128 queries are the x dimension of the grid, which takes 2^31 - 1 of them)
 
     int splits = use_workspace && workspace != nullptr &&
                          reinterpret_cast<std::uintptr_t>(workspace) % 4 == 0

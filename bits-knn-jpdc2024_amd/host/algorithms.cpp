@@ -34,6 +34,11 @@ std::vector<float> to_dim_major(const float* data, std::size_t count, std::size_
     return out;
 }
 
+int layout_code(matrix_layout layout)
+{
+    return layout == matrix_layout::row_major ? BITSKNN_LAYOUT_ROW_MAJOR : BITSKNN_LAYOUT_COLUMN_MAJOR;
+}
+
 float component(const float* data, std::size_t count, std::size_t dim, matrix_layout layout,
                 std::size_t v, std::size_t t)
 {
@@ -53,24 +58,30 @@ void device_distance::prepare(const knn_args& args)
     {
         throw std::runtime_error{"Only the row-major layout of the distance matrix is supported."};
     }
-    const auto points = to_dim_major(args_.points, args_.point_count, args_.dim, args_.points_layout);
-    const auto queries = to_dim_major(args_.queries, args_.query_count, args_.dim, args_.queries_layout);
+    // the vectors go to the device in the caller's layout (reference: cuda_distance::prepare,
+    // src/distance/cuda_distance.cpp; the layouts are resolved on the device)
     points_ = device_buffer<float>{args_.dim * args_.point_count};
     queries_ = device_buffer<float>{args_.dim * args_.query_count};
     dist_ = device_buffer<float>{args_.query_count * args_.point_count};
+    workspace_ = device_buffer<unsigned char>{bitsknn_dist_layout_workspace_bytes(
+        static_cast<int>(args_.dim), args_.query_count, args_.point_count, layout_code(args_.queries_layout),
+        layout_code(args_.points_layout))};
     transfer_.start();
-    points_.upload(points.data(), points.size());
-    queries_.upload(queries.data(), queries.size());
+    points_.upload(args_.points, points_.size());
+    queries_.upload(args_.queries, queries_.size());
     sync_default_stream();
     transfer_.stop();
 }
 
 void device_distance::compute()
 {
-    BITSKNN_CHECK(bitsknn_dist_f32(op_, static_cast<int>(args_.dim), args_.query_count,
-                                   args_.point_count, queries_.data(), args_.query_count,
-                                   points_.data(), args_.point_count, dist_.data(), args_.point_count,
-                                   nullptr));
+    const bool q_rows = args_.queries_layout == matrix_layout::row_major;
+    const bool p_rows = args_.points_layout == matrix_layout::row_major;
+    BITSKNN_CHECK(bitsknn_dist_layout_f32(
+        op_, static_cast<int>(args_.dim), args_.query_count, args_.point_count, queries_.data(),
+        layout_code(args_.queries_layout), q_rows ? args_.dim : args_.query_count, points_.data(),
+        layout_code(args_.points_layout), p_rows ? args_.dim : args_.point_count, dist_.data(), args_.point_count,
+        workspace_.size() != 0 ? workspace_.data() : nullptr, workspace_.size(), nullptr));
 }
 
 const std::vector<float>& device_distance::matrix_cpu()

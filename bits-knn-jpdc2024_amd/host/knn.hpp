@@ -64,9 +64,10 @@ protected:
     int op_;
     std::string name_;
     knn_args args_{};
-    knn_host::device_buffer<float> points_;  // dim x point_count
-    knn_host::device_buffer<float> queries_; // dim x query_count
+    knn_host::device_buffer<float> points_;  // in the caller's layout
+    knn_host::device_buffer<float> queries_; // in the caller's layout
     knn_host::device_buffer<float> dist_;    // query_count x point_count
+    knn_host::device_buffer<unsigned char> workspace_; // dim-major copies of row-major inputs
     std::vector<float> dist_host_;
     knn_host::transfer_timer transfer_;
 };

@@ -159,6 +159,31 @@ int bitsknn_dist_f32(int op, int dim, size_t q, size_t n, const float* queries_d
                      float* dist, size_t dist_row_stride, void* stream);
 
 /*
+ * bitsknn_dist_f32 for vectors in the caller's layout.  The reference's distance classes take the
+ * points and the queries in either matrix layout of knn_args, four combinations
+ * (src/distance/cublas_distance.cu:122-149: the transposition flags of the SGEMM and the
+ * row_major / column_major forms of squared_length_kernel :23-60; include/bits/layout.hpp:4):
+ *   BITSKNN_LAYOUT_ROW_MAJOR     the vectors one after the other: component t of vector v at
+ *                                base[v*stride + t], stride >= dim (matrix_layout::row_major)
+ *   BITSKNN_LAYOUT_COLUMN_MAJOR  dim-major as for bitsknn_dist_f32: base[t*stride + v], stride >=
+ *                                the vector count (matrix_layout::column_major)
+ * A set of vectors given one after the other is first brought into dim-major form on the device
+ * (a copy in `workspace`, 16-byte aligned, bitsknn_dist_layout_workspace_bytes() bytes: dim x the
+ * count rounded up to a multiple of four floats per such set; nothing for dim-major sets), then
+ * the kernels of bitsknn_dist_f32 run: same values bit for bit in every combination.
+ * Errors as for bitsknn_dist_f32, plus BITSKNN_ERR_INVALID for an unknown layout or a workspace
+ * that is missing, misaligned or too small.
+ */
+#define BITSKNN_LAYOUT_ROW_MAJOR 0
+#define BITSKNN_LAYOUT_COLUMN_MAJOR 1
+size_t bitsknn_dist_layout_workspace_bytes(int dim, size_t q, size_t n, int queries_layout,
+                                           int points_layout);
+int bitsknn_dist_layout_f32(int op, int dim, size_t q, size_t n, const float* queries,
+                            int queries_layout, size_t query_stride, const float* points,
+                            int points_layout, size_t point_stride, float* dist, size_t dist_row_stride,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * bits-fused: partial squared L2 distance (||p||^2 - 2 q.p) and top-k in one kernel; the
  * q x n distance matrix is never written to memory.  Outputs q x k, row stride k, ascending,
  * equal distances ordered by lower point index.

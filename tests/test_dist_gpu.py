@@ -262,3 +262,42 @@ def test_bf16x3_distances_views_and_ragged_ends(bk, dev, oracle):
         exp = oracle.dist(s, p, "partial")
         scale = (p.astype(np.float64) ** 2).sum(1)[None, :] * 2 + (s.astype(np.float64) ** 2).sum(1)[:, None]
         assert np.max(np.abs(out[:, off:off + n].cpu().numpy() - exp) / scale) < 1e-5, (n, q, d, opad, off)
+
+
+@pytest.mark.parametrize("op", ["l2", "partial", "expanded"])
+@pytest.mark.parametrize("q,n,d", [(37, 1000, 5), (130, 4097, 32), (64, 300, 100), (1, 1, 1), (33, 129, 64)])
+def test_the_four_layout_combinations(bk, dev, oracle, op, q, n, d):
+    """bitsknn_dist_layout_f32: points and queries in either layout of the reference's knn_args
+    (src/distance/cublas_distance.cu:122-149 serves the four combinations); every combination must
+    give the matrix of the dim-major entry point bit for bit."""
+    import torch
+    code = {"l2": bk.DIST_L2, "partial": bk.DIST_PARTIAL_L2, "expanded": bk.DIST_EXPANDED}[op]
+    points, queries = oracle.generate(q + n + d, n, q, d)
+    p_rows = torch.from_numpy(points).to(dev)
+    q_rows = torch.from_numpy(queries).to(dev)
+    p_dm = p_rows.t().contiguous()
+    q_dm = q_rows.t().contiguous()
+    want = bk.distances(q_dm, p_dm, code)
+    torch.cuda.synchronize()
+    for q_layout, q_in in ((bk.LAYOUT_ROW_MAJOR, q_rows), (bk.LAYOUT_COLUMN_MAJOR, q_dm)):
+        for p_layout, p_in in ((bk.LAYOUT_ROW_MAJOR, p_rows), (bk.LAYOUT_COLUMN_MAJOR, p_dm)):
+            got = bk.distances_layout(q_in, q_layout, p_in, p_layout, code)
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), (q_layout, p_layout)
+    if op == "l2":
+        assert np.array_equal(want.cpu().numpy(), oracle.dist(queries, points, "l2"))
+
+
+def test_layout_entry_point_validation(bk, dev):
+    import torch
+    a = torch.zeros((10, 4), device=dev)
+    square = torch.zeros((4, 4), device=dev)
+    with pytest.raises(bk.BitsKnnError, match="unknown layout 7"):
+        bk.distances_layout(square, 7, square, bk.LAYOUT_ROW_MAJOR)
+    L = bk.lib()
+    assert L.bitsknn_dist_layout_workspace_bytes(4, 10, 10, bk.LAYOUT_COLUMN_MAJOR, bk.LAYOUT_COLUMN_MAJOR) == 0
+    assert L.bitsknn_dist_layout_workspace_bytes(4, 10, 13, bk.LAYOUT_ROW_MAJOR, bk.LAYOUT_ROW_MAJOR) == 4 * (12 + 16) * 4
+    out = torch.empty((10, 10), device=dev)
+    status = L.bitsknn_dist_layout_f32(bk.DIST_L2, 4, 10, 10, a.data_ptr(), bk.LAYOUT_ROW_MAJOR, 4, a.data_ptr(),
+                                       bk.LAYOUT_ROW_MAJOR, 4, out.data_ptr(), 10, None, 0, None)
+    assert status == bk.ERR_INVALID and b"workspace" in L.bitsknn_last_error()
