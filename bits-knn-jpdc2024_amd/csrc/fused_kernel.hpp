@@ -333,7 +333,8 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             qq = __builtin_fmaf(qx[dd], qx[dd], qq);
         }
         filter_slack = FILTER_REL * qq * (1.0F + 0x1.0p-20F) + FILTER_ABS * (1.0F + qq);
-        const vuint4 ones{0x3F803F80U, 0, 0, 0};
+        // (the norm cell holds two pieces per share of the norm, at most four shares)
+        const vuint4 ones{0x3F803F80U, 0x3F803F80U, 0x3F803F80U, 0x3F803F80U};
         const vuint4 zeros{0, 0, 0, 0};
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
@@ -709,8 +710,13 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     // are neighbouring lanes, which add up their shares of the norm among themselves
     // SPLIT: thread t carries the 8 dimensions 8*(t % TPP) .. + 7 of point t / TPP (neighbouring
     // lanes as well)
-    const int sp = SPLIT || EXACT || G::PAIRED ? t / TPP : t % PT;
-    const int sd0 = SPLIT || EXACT ? VPT * (t % TPP) : (G::PAIRED ? t % TPP : t / PT);
+    // EXACT: thread t carries the VPT dimensions VPT * (t / PT) .. of point t % PT, so that the
+    // threads of a wave write neighbouring words, rows and cells of a stage (no two of them meet in
+    // a bank of LDS); every group of VPT dimensions has its own share of the norm
+    const int sp = EXACT ? t % PT : (SPLIT || G::PAIRED ? t / TPP : t % PT);
+    const int sd0 = EXACT ? VPT * (t / PT) : (SPLIT ? VPT * (t % TPP) : (G::PAIRED ? t % TPP : t / PT));
+    // EXACT: the word of a point's norm cell that takes this thread's share of the norm
+    const int norm_slot = DP == 64 ? wave : t / PT;
     auto dim_of = [&](int i) -> int { return SPLIT || EXACT ? sd0 + i : sd0 + TPP * i; };
     float pre[VPT];
     // Point values are read with buffer loads: a constant byte offset per value and lane (beyond
@@ -810,10 +816,10 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             constexpr int PIECE2 = DP <= 8 ? 1 : KS; // first cell of the second pieces
             if constexpr (VPT == 8)
             {
+                // (the cell of dimension group t / PT of point t % PT is cell t)
                 vuint4* const cells = reinterpret_cast<vuint4*>(stage + DP * PT);
-                const int ks = sd0 / 8;
-                cells[ks * PT + sp] = piece[0];
-                cells[(PIECE2 + ks) * PT + sp] = piece[1];
+                cells[t] = piece[0];
+                cells[PIECE2 * PT + t] = piece[1];
             }
             else
             {
@@ -824,31 +830,23 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 halves[2 * sp + h] = vuint2{piece[0][0], piece[0][1]};
                 halves[2 * (PIECE2 * PT + sp) + h] = vuint2{piece[1][0], piece[1][1]};
             }
-            // the threads of a point are TPP neighbouring lanes
-            if constexpr (TPP >= 2)
+            if constexpr (DP == 64)
             {
-                share += __builtin_bit_cast(float, lane_xor32<1>(__builtin_bit_cast(u32, share)));
-            }
-            if constexpr (TPP >= 4)
-            {
-                share += __builtin_bit_cast(float, lane_xor32<2>(__builtin_bit_cast(u32, share)));
-            }
-            if constexpr (TPP == 8)
-            {
-                share += __builtin_bit_cast(float, lane_xor32<4>(__builtin_bit_cast(u32, share)));
+                // two groups of dimensions per wave: one share
+                share += __builtin_bit_cast(float, lane_xor32<32>(__builtin_bit_cast(u32, share)));
             }
             {
-                // the lowered norm in two pieces, written by every thread of the point (same
-                // value: no branch in the staging code, which is scheduled between the matrix
-                // instructions of the stage being filtered); points beyond the end only pass an
+                // the lowered share of the norm in two pieces, one word of the point's norm cell per
+                // share (the matrix instruction adds them up); points beyond the end only pass an
                 // infinite radius
                 const float lowered = __builtin_fmaf(-NORM_LOWER, share, share);
                 const vfloat2 whole{lowered, 0.0F};
                 const u32 first = __builtin_bit_cast(u32, __builtin_convertvector(whole, vbf16x2)) & 0xFFFFU;
                 const vfloat2 rest{lowered - __builtin_bit_cast(float, first << 16U), 0.0F};
                 const u32 second = __builtin_bit_cast(u32, __builtin_convertvector(rest, vbf16x2)) & 0xFFFFU;
-                const vuint4 cell{base + sp < n ? first | (second << 16U) : BF16_HUGE, 0, 0, 0};
-                reinterpret_cast<vuint4*>(stage + DP * PT)[(G::CELLS - 1) * PT + sp] = cell;
+                u32* const norm_cell =
+                    reinterpret_cast<u32*>(reinterpret_cast<vuint4*>(stage + DP * PT) + (G::CELLS - 1) * PT + sp);
+                norm_cell[norm_slot] = base + sp < n ? first | (second << 16U) : BF16_HUGE;
             }
         }
         else if constexpr (SPLIT)
@@ -1081,7 +1079,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         __builtin_amdgcn_sched_barrier(0);
         // staging state
         constexpr int PAIRS_OF_VALUES = VPT / 2;
-        constexpr int CHUNKS = PAIRS_OF_VALUES + 4;
+        constexpr int CHUNKS = PAIRS_OF_VALUES + 3;
         static_assert(!EXACT || CHUNKS <= MT * TERMS, "a piece of staging per matrix instruction");
         float share = 0.0F;
         u32 piece1[4] = {0, 0, 0, 0};
@@ -1109,9 +1107,8 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             {
                 if constexpr (VPT == 8)
                 {
-                    const int ks = sd0 / 8;
-                    into_cells[ks * PT + sp] = vuint4{piece1[0], piece1[1], piece1[2], piece1[3]};
-                    into_cells[(PIECE2 + ks) * PT + sp] = vuint4{piece2[0], piece2[1], piece2[2], piece2[3]};
+                    into_cells[t] = vuint4{piece1[0], piece1[1], piece1[2], piece1[3]};
+                    into_cells[PIECE2 * PT + t] = vuint4{piece2[0], piece2[1], piece2[2], piece2[3]};
                 }
                 else
                 {
@@ -1125,22 +1122,10 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             }
             else if constexpr (c == PAIRS_OF_VALUES + 1)
             {
-                // the threads of a point are TPP neighbouring lanes
-                if constexpr (TPP >= 2)
+                if constexpr (DP == 64)
                 {
-                    share += __builtin_bit_cast(float, lane_xor32<1>(__builtin_bit_cast(u32, share)));
+                    share += __builtin_bit_cast(float, lane_xor32<32>(__builtin_bit_cast(u32, share)));
                 }
-                if constexpr (TPP >= 4)
-                {
-                    share += __builtin_bit_cast(float, lane_xor32<2>(__builtin_bit_cast(u32, share)));
-                }
-                if constexpr (TPP == 8)
-                {
-                    share += __builtin_bit_cast(float, lane_xor32<4>(__builtin_bit_cast(u32, share)));
-                }
-            }
-            else if constexpr (c == PAIRS_OF_VALUES + 2)
-            {
                 const float lowered = __builtin_fmaf(-NORM_LOWER, share, share);
                 const vfloat2 whole{lowered, 0.0F};
                 const u32 first = __builtin_bit_cast(u32, __builtin_convertvector(whole, vbf16x2)) & 0xFFFFU;
@@ -1150,7 +1135,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             }
             else
             {
-                into_cells[(G::CELLS - 1) * PT + sp] = vuint4{norm_word, 0, 0, 0};
+                reinterpret_cast<u32*>(into_cells + (G::CELLS - 1) * PT + sp)[norm_slot] = norm_word;
             }
         };
         static_for<0, TERMS>([&](auto j_tag) {
