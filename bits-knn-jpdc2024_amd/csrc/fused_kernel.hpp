@@ -1024,13 +1024,14 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         static_for<0, TERMS>([&](auto j_tag) {
             constexpr int j = decltype(j_tag)::value;
             // term j: which cell of the point against which operand of the query (up to 8
-            // dimensions: the two cells in turn; else the norm cell first, then per 16 dimensions
-            // piece 2 x piece 1, piece 1 x piece 2, piece 1 x piece 1)
-            constexpr int kb = DP <= 8 ? 0 : (j - 1) / 3;
-            constexpr int which = DP <= 8 ? j : (j - 1) % 3;
-            constexpr int a_at = DP <= 8 ? j : (j == 0 ? 2 * KB : (which == 0 ? KB + kb : kb));
-            constexpr int b_piece = DP <= 8 ? j : (j == 0 ? 2 : (which == 1 ? 1 : 0));
-            constexpr int b_kb = DP <= 8 || j == 0 ? 0 : kb;
+            // dimensions: the two cells in turn; else per 16 dimensions piece 2 x piece 1,
+            // piece 1 x piece 2, piece 1 x piece 1, and the norm cell last)
+            constexpr bool norm_term = DP > 8 && j == 3 * KB;
+            constexpr int kb = DP <= 8 || norm_term ? 0 : j / 3;
+            constexpr int which = DP <= 8 ? j : j % 3;
+            constexpr int a_at = DP <= 8 ? j : (norm_term ? 2 * KB : (which == 0 ? KB + kb : kb));
+            constexpr int b_piece = DP <= 8 ? j : (norm_term ? 2 : (which == 1 ? 1 : 0));
+            constexpr int b_kb = kb;
 #pragma unroll
             for (int t = 0; t < MT; ++t)
             {
@@ -1045,7 +1046,10 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     // instructions that are placed one after each of the first matrix instructions, where they
     // execute next to it.  The staging code has no branch (every thread of a point writes the norm
     // cell); scheduling barriers keep the order written here.
-    auto filter_values_and_stage = [&](const float* stage, vfloat16 (&w)[MT], float* into, int next_base) __attribute__((always_inline)) {
+    auto filter_values_and_stage = [&](const float* stage, vfloat16 (&w)[MT], float* into, int next_base, auto early_tag) __attribute__((always_inline)) {
+        constexpr bool EARLY_FETCH = decltype(early_tag)::value;
+        // (the cells are read in the order in which the matrix instructions take them, the norm
+        // cell last, so that the first instruction waits for the first read only)
         const vuint4* const cells = reinterpret_cast<const vuint4*>(stage + DP * PT);
         vfloat16 zero;
 #pragma unroll
@@ -1056,24 +1060,39 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         constexpr int TERMS = DP <= 8 ? 2 : 3 * KB + 1;
         constexpr int NCELL = DP <= 8 ? 2 : 2 * KB + 1;
         vuint4 cell[MT][NCELL];
-#pragma unroll
-        for (int t = 0; t < MT; ++t)
+        const vuint4* const mine = cells + ql;
+        if constexpr (DP <= 8)
         {
-            const vuint4* const mine = cells + 32 * t + ql;
-            if constexpr (DP <= 8)
-            {
-                cell[t][0] = mine[(half != 0 ? 1 : 0) * PT];
-                cell[t][1] = mine[(half != 0 ? 2 : 0) * PT];
-            }
-            else
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
             {
 #pragma unroll
-                for (int kb = 0; kb < KB; ++kb)
+                for (int t = 0; t < MT; ++t)
                 {
-                    cell[t][kb] = mine[(2 * kb + half) * PT];
-                    cell[t][KB + kb] = mine[(KS + 2 * kb + half) * PT];
+                    cell[t][c] = mine[32 * t + (half != 0 ? 1 + c : 0) * PT];
                 }
-                cell[t][2 * KB] = mine[2 * KS * PT];
+            }
+        }
+        else
+        {
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+            {
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+                {
+                    cell[t][KB + kb] = mine[32 * t + (KS + 2 * kb + half) * PT];
+                }
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+                {
+                    cell[t][kb] = mine[32 * t + (2 * kb + half) * PT];
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+            {
+                cell[t][2 * KB] = mine[32 * t + 2 * KS * PT];
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -1119,6 +1138,22 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                     halves[2 * sp + h] = vuint2{piece1[0], piece1[1]};
                     halves[2 * (PIECE2 * PT + sp) + h] = vuint2{piece2[0], piece2[1]};
                 }
+                // the registers of the values are free: the stage after the next one is requested
+                // now, so that its loads have the rest of this stage and the start of the next one
+                // (buffer loads without a branch: beyond the matrix they read zero, and points
+                // from n on, whatever their values, carry the norm that only passes an infinite
+                // radius and are dropped by their labels)
+                if constexpr (EARLY_FETCH)
+                {
+                    const int stage_off =
+                        ((next_base + PT) * a.sample_scale + a.sample_offset) * static_cast<int>(sizeof(float));
+#pragma unroll
+                    for (int i = 0; i < VPT; ++i)
+                    {
+                        pre[i] = __builtin_bit_cast(
+                            float, __builtin_amdgcn_raw_buffer_load_b32(point_rsrc, load_off[i], stage_off, 0));
+                    }
+                }
             }
             else if constexpr (c == PAIRS_OF_VALUES + 1)
             {
@@ -1140,11 +1175,12 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         };
         static_for<0, TERMS>([&](auto j_tag) {
             constexpr int j = decltype(j_tag)::value;
-            constexpr int kb = DP <= 8 ? 0 : (j - 1) / 3;
-            constexpr int which = DP <= 8 ? j : (j - 1) % 3;
-            constexpr int a_at = DP <= 8 ? j : (j == 0 ? 2 * KB : (which == 0 ? KB + kb : kb));
-            constexpr int b_piece = DP <= 8 ? j : (j == 0 ? 2 : (which == 1 ? 1 : 0));
-            constexpr int b_kb = DP <= 8 || j == 0 ? 0 : kb;
+            constexpr bool norm_term = DP > 8 && j == 3 * KB;
+            constexpr int kb = DP <= 8 || norm_term ? 0 : j / 3;
+            constexpr int which = DP <= 8 ? j : j % 3;
+            constexpr int a_at = DP <= 8 ? j : (norm_term ? 2 * KB : (which == 0 ? KB + kb : kb));
+            constexpr int b_piece = DP <= 8 ? j : (norm_term ? 2 : (which == 1 ? 1 : 0));
+            constexpr int b_kb = kb;
             static_for<0, MT>([&](auto t_tag) {
                 constexpr int t = decltype(t_tag)::value;
                 constexpr int m = j * MT + t; // number of this matrix instruction
@@ -1531,25 +1567,40 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         {
             // The next stage is written while the matrix instructions of this one run (see
             // filter_values_and_stage).  (The stage after the last one is "written" from whatever
-            // the registers hold, into a slot that nobody reads any more.)
-            for (int base = n_begin; base < n; base += PT)
-            {
-                wait_for(slot, round + 1);
-                BITSKNN_FT_LAP(0);
-                const int next = slot + 1 == NB ? 0 : slot + 1;
-                const float* const stage = stages + slot * STAGE_FLOATS;
-                vfloat16 w[MT];
-                __builtin_amdgcn_sched_barrier(0);
-                filter_values_and_stage(stage, w, stages + next * STAGE_FLOATS, base + PT);
-                count_in(next);
-                if (base + 2 * PT < n)
+            // the registers hold, into a slot that nobody reads any more.)  Point matrices below
+            // 2 GiB request the stage after the next one in the middle of those instructions.
+            auto pass = [&](auto early_tag) __attribute__((always_inline)) {
+                constexpr bool EARLY_FETCH = decltype(early_tag)::value;
+                for (int base = n_begin; base < n; base += PT)
                 {
-                    fetch(base + 2 * PT);
+                    wait_for(slot, round + 1);
+                    BITSKNN_FT_LAP(0);
+                    const int next = slot + 1 == NB ? 0 : slot + 1;
+                    const float* const stage = stages + slot * STAGE_FLOATS;
+                    vfloat16 w[MT];
+                    __builtin_amdgcn_sched_barrier(0);
+                    filter_values_and_stage(stage, w, stages + next * STAGE_FLOATS, base + PT, early_tag);
+                    count_in(next);
+                    if constexpr (!EARLY_FETCH)
+                    {
+                        if (base + 2 * PT < n)
+                        {
+                            fetch(base + 2 * PT);
+                        }
+                    }
+                    BITSKNN_FT_LAP(2);
+                    filter_and_append(w, stage, base);
+                    slot = next;
+                    round += slot == 0 ? 1 : 0;
                 }
-                BITSKNN_FT_LAP(2);
-                filter_and_append(w, stage, base);
-                slot = next;
-                round += slot == 0 ? 1 : 0;
+            };
+            if (small_points)
+            {
+                pass(std::true_type{});
+            }
+            else
+            {
+                pass(std::false_type{});
             }
         }
         else
