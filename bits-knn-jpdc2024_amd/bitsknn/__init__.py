@@ -30,6 +30,7 @@ EXPORTS = (
     "bitsknn_dist_layout_f32",
     "bitsknn_fused_l2_topk_f32",
     "bitsknn_fused_workspace_bytes",
+    "bitsknn_fused_image_bytes",
     "bitsknn_fused_l2_topk_f32_ws",
     "bitsknn_fused_l2_topk_f32_ex",
     "bitsknn_fused_l2_topk_f32_tuned",
@@ -41,7 +42,8 @@ EXPORTS = (
 
 class FusedTuning(ctypes.Structure):
     """bitsknn_fused_tuning of include/bitsknn.h"""
-    _fields_ = [("ranges", ctypes.c_int32), ("first_radius", ctypes.c_int32), ("reserved", ctypes.c_int32 * 6)]
+    _fields_ = [("ranges", ctypes.c_int32), ("first_radius", ctypes.c_int32), ("image", ctypes.c_int32),
+                ("reserved", ctypes.c_int32 * 5)]
 
 
 class BitsKnnError(RuntimeError):
@@ -101,6 +103,8 @@ def lib():
                                                    ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, sz, vp]
         L.bitsknn_fused_workspace_bytes.restype = ctypes.c_size_t
         L.bitsknn_fused_workspace_bytes.argtypes = [i32, i32, ctypes.c_int]
+        L.bitsknn_fused_image_bytes.restype = ctypes.c_size_t
+        L.bitsknn_fused_image_bytes.argtypes = [ctypes.c_int, i32]
         L.bitsknn_fused_l2_topk_f32_ws.restype = ctypes.c_int
         L.bitsknn_fused_l2_topk_f32_ws.argtypes = [vp, vp, ctypes.c_int, i32, i32, vp, vp, ctypes.c_int,
                                                    ctypes.c_int, ctypes.c_int, ctypes.c_int,
@@ -271,11 +275,12 @@ def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1,
                   out_dist=None, out_label=None, workspace=None, arithmetic=None, tuning=None):
     """bits-fused: top-k of ||p||^2 - 2 q.p without materialising the distance matrix.
     workspace: None -> the plain entry point; "auto" -> allocate what
-    bitsknn_fused_workspace_bytes asks for; "static" -> the entry point that uses the library's own
+    bitsknn_fused_workspace_bytes asks for; "image" -> that plus room for the stage image
+    (fused_workspace_with_image_bytes); "static" -> the entry point that uses the library's own
     scratch memory and allocates nothing; or a uint8 device tensor.
     arithmetic: None -> the plain entry points (FUSED_EXACT); FUSED_FP32 / FUSED_BF16X3 /
     FUSED_EXACT -> bitsknn_fused_l2_topk_f32_ex with that arithmetic.
-    tuning: None, or (ranges, first_radius) -> bitsknn_fused_l2_topk_f32_tuned."""
+    tuning: None, or (ranges, first_radius[, image]) -> bitsknn_fused_l2_topk_f32_tuned."""
     import torch
     d, q = queries_dm.shape
     d2, n = points_dm.shape
@@ -287,11 +292,15 @@ def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1,
     if isinstance(workspace, str) and workspace == "auto":
         workspace = torch.empty(max(1, fused_workspace_bytes(q, n, k)), dtype=torch.uint8,
                                 device=queries_dm.device)
+    if isinstance(workspace, str) and workspace == "image":
+        workspace = torch.empty(max(1, fused_workspace_with_image_bytes(d, q, n, k)), dtype=torch.uint8,
+                                device=queries_dm.device)
     head = (_ptr(queries_dm), _ptr(points_dm), d, q, n, _ptr(out_dist), _ptr(out_label), k,
             params[0], params[1], params[2], block_query_dim, dim_mult)
     if tuning is not None:
         assert not isinstance(workspace, str)
-        knobs = FusedTuning(int(tuning[0]), int(tuning[1]), (ctypes.c_int32 * 6)())
+        knobs = FusedTuning(int(tuning[0]), int(tuning[1]), int(tuning[2]) if len(tuning) > 2 else 0,
+                            (ctypes.c_int32 * 5)())
         _check(lib().bitsknn_fused_l2_topk_f32_tuned(*head[:8], FUSED_EXACT if arithmetic is None else int(arithmetic),
                                                      ctypes.byref(knobs), _ptr(workspace),
                                                      workspace.numel() if workspace is not None else 0, _stream()))
@@ -311,6 +320,15 @@ def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1,
 
 def fused_workspace_bytes(q, n, k):
     return int(lib().bitsknn_fused_workspace_bytes(q, n, k))
+
+
+def fused_image_bytes(dim, n):
+    return int(lib().bitsknn_fused_image_bytes(dim, n))
+
+
+def fused_workspace_with_image_bytes(dim, q, n, k):
+    """Partial lists, rounded up to a multiple of 256 bytes, then the stage image."""
+    return (fused_workspace_bytes(q, n, k) + 255) // 256 * 256 + fused_image_bytes(dim, n)
 
 
 def fused_static_scratch_bytes():

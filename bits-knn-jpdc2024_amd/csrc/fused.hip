@@ -142,6 +142,10 @@ constexpr int SAMPLE_POINTS_RANGES = 2048;
 constexpr int SAMPLE_MIN_POINTS = 1 << 17; // at least 8 (2 with ranges) sampled stages of any size
 constexpr int SAMPLE_MIN_K = 64;
 constexpr int SAMPLE_MIN_K_RANGES = 64; // (k <= 32: the three extra launches cost what the merges save)
+// fewest queries for which the stage image of the exact arithmetic is built when the workspace has
+// room for it (its launch reads and writes the points once, about 0.1 ms for 2^20 points in 32
+// dimensions; every workgroup of 128 queries saves the cutting of all its points)
+constexpr int IMAGE_MIN_QUERIES = 4096;
 
 int first_radius_rank(int k, int scale)
 {
@@ -223,6 +227,13 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
                         "bitsknn_fused_tuning: first_radius must be 0 (the library's choice), -1 (never) or 2 .. 4096 "
                         "(one stage in every so many), got %d",
                         tuning->first_radius);
+        }
+        if (tuning->image < -1 || tuning->image > 1)
+        {
+            return fail(BITSKNN_ERR_INVALID,
+                        "bitsknn_fused_tuning: image must be 0 (the library's choice), -1 (never) or 1 (whenever the "
+                        "workspace has room for it), got %d",
+                        tuning->image);
         }
         for (const std::int32_t word : tuning->reserved)
         {
@@ -327,6 +338,8 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
         a.splits = splits;
     }
     a.split_points = ((n + splits - 1) / splits + 255) / 256 * 256;
+    a.image = nullptr;
+    a.image_bytes = 0;
 
     auto* hip_stream = static_cast<hipStream_t>(stream);
     const int split = arithmetic == BITSKNN_FUSED_BF16X3 ? FUSED_ARITH_BF16X3
@@ -340,6 +353,26 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
                                      128, 4, 0, stream);
     };
     hipError_t status = hipSuccess;
+    // The stage image: with room for it in the workspace behind the partial lists, the points are
+    // cut into the stages of the exact arithmetic once, by a launch of their own, instead of by
+    // every workgroup of the fused kernel again.  That pays from a few thousand queries on.
+    if (split == FUSED_ARITH_EXACT && use_workspace && workspace != nullptr && dim <= 64 &&
+        (tuning == nullptr || tuning->image >= 0))
+    {
+        const size_t image_bytes = fused_image_bytes(dim, n);
+        const size_t lists = splits > 1 ? partial_list_bytes(q, splits, k) : 0;
+        const size_t offset = (lists + 255) / 256 * 256;
+        const bool wanted = (tuning != nullptr && tuning->image == 1) || q >= IMAGE_MIN_QUERIES;
+        if (wanted && image_bytes > 0 && image_bytes < (1ULL << 31) && offset + image_bytes <= workspace_bytes &&
+            reinterpret_cast<std::uintptr_t>(workspace) % 16 == 0)
+        {
+            void* const image = static_cast<char*>(workspace) + offset;
+            status = launch_fused_image(points_dim_major, dim, n, image, hip_stream);
+            BITSKNN_HIP_CHECK(status);
+            a.image = image;
+            a.image_bytes = static_cast<int>(image_bytes);
+        }
+    }
     int scale = SAMPLE_SCALE;
     if (splits > 1)
     {
@@ -406,6 +439,12 @@ extern "C" int bitsknn_fused_l2_topk_f32(const float* queries_dim_major,
     return bitsknn::fused_impl(queries_dim_major, points_dim_major, dim, q, n, out_dist, out_label, k,
                                query_reg, db_reg, dim_reg, block_query_dim, dim_mult, BITSKNN_FUSED_EXACT,
                                nullptr, 0, false, stream);
+}
+
+extern "C" size_t bitsknn_fused_image_bytes(int dim, int32_t n)
+{
+    const size_t bytes = bitsknn::fused_image_bytes(dim, n);
+    return bytes < (1ULL << 31) ? bytes : 0;
 }
 
 extern "C" size_t bitsknn_fused_workspace_bytes(int32_t q, int32_t n, int k)

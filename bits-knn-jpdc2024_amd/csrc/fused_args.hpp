@@ -64,6 +64,11 @@ struct fused_args
     // end and overwrites the k-th distances of its queries with NaN.
     int* fault;
     int poll_limit;
+    // FUSED_ARITH_EXACT: the stages of the whole point matrix as they stand in LDS, one after the
+    // other, written by launch_fused_image (null: the kernel cuts the points itself); image_bytes
+    // below 2^31
+    const void* image;
+    int image_bytes;
 #ifdef BITSKNN_FUSED_TIMING
     // instrumented build: cycles of all waves per phase of the stage loop, added up here
     unsigned long long* timing;
@@ -72,6 +77,10 @@ struct fused_args
 
 // one per compiled list length K (fused_inst.hip); arith: one of FUSED_ARITH_*, used where the
 // dimension allows it (fp32 matrix instructions otherwise)
+// the stage image of FUSED_ARITH_EXACT (stage_image.hip): its size for a point matrix of up to 64
+// dimensions (0 otherwise), and the launch that writes it
+size_t fused_image_bytes(int dim, int n);
+hipError_t launch_fused_image(const float* points, int dim, int n, void* image, hipStream_t stream);
 hipError_t launch_fused_k_4(const fused_args& a, int arith, hipStream_t stream);
 hipError_t launch_fused_k_8(const fused_args& a, int arith, hipStream_t stream);
 hipError_t launch_fused_k_16(const fused_args& a, int arith, hipStream_t stream);

@@ -787,6 +787,37 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             }
         }
     };
+    // EXACT with a stage image (fused_args::image): the stages as they stand in LDS were written to
+    // global memory by fused_image_kernel, one after the other; staging is then a copy of 16-byte
+    // units, IU per thread, through registers -- no arithmetic in this kernel.
+    constexpr int UNITS = EXACT ? STAGE_FLOATS / 4 : 1;
+    constexpr int IU = EXACT ? (UNITS + FQ_THREADS - 1) / FQ_THREADS : 1;
+    vuint4 img[IU];
+    int img_off[IU];
+    const auto image_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<void*>(EXACT ? a.image : nullptr), 0, EXACT ? a.image_bytes : 0, 0x00020000);
+#pragma unroll
+    for (int j = 0; j < IU; ++j)
+    {
+        img[j] = vuint4{0, 0, 0, 0};
+        img_off[j] = t + FQ_THREADS * j < UNITS ? (t + FQ_THREADS * j) * 16 : OUTSIDE;
+    }
+    // (base is a multiple of PT, and so is the offset of a sample; beyond the image the loads read zero)
+    auto fetch_image = [&](int base) __attribute__((always_inline)) {
+        const int stage_off = (base * a.sample_scale + a.sample_offset) * (STAGE_FLOATS * 4 / PT);
+#pragma unroll
+        for (int j = 0; j < IU; ++j)
+        {
+            img[j] = __builtin_bit_cast(vuint4, __builtin_amdgcn_raw_buffer_load_b128(image_rsrc, img_off[j], stage_off, 0));
+        }
+    };
+    auto deposit_image_unit = [&](float* stage, auto j_tag) __attribute__((always_inline)) {
+        constexpr int j = decltype(j_tag)::value;
+        if (FQ_THREADS * (j + 1) <= UNITS || t + FQ_THREADS * j < UNITS)
+        {
+            reinterpret_cast<vuint4*>(stage)[t + FQ_THREADS * j] = img[j];
+        }
+    };
     auto deposit = [&](float* stage, int base) {
         if constexpr (G::STAGERS < FQ_THREADS)
         {
@@ -1046,8 +1077,11 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     // instructions that are placed one after each of the first matrix instructions, where they
     // execute next to it.  The staging code has no branch (every thread of a point writes the norm
     // cell); scheduling barriers keep the order written here.
-    auto filter_values_and_stage = [&](const float* stage, vfloat16 (&w)[MT], float* into, int next_base, auto early_tag) __attribute__((always_inline)) {
-        constexpr bool EARLY_FETCH = decltype(early_tag)::value;
+    auto filter_values_and_stage = [&](const float* stage, vfloat16 (&w)[MT], float* into, int next_base, auto mode_tag) __attribute__((always_inline)) {
+        constexpr int MODE = decltype(mode_tag)::value; // 0: the values of the stage after the next
+                                                        // one are requested after this call, 1: in
+                                                        // the middle of it, 2: stages from an image
+        constexpr bool EARLY_FETCH = MODE == 1;
         // (the cells are read in the order in which the matrix instructions take them, the norm
         // cell last, so that the first instruction waits for the first read only)
         const vuint4* const cells = reinterpret_cast<const vuint4*>(stage + DP * PT);
@@ -1098,7 +1132,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         __builtin_amdgcn_sched_barrier(0);
         // staging state
         constexpr int PAIRS_OF_VALUES = VPT / 2;
-        constexpr int CHUNKS = PAIRS_OF_VALUES + 3;
+        constexpr int CHUNKS = MODE == 2 ? IU + 1 : PAIRS_OF_VALUES + 3;
         static_assert(!EXACT || CHUNKS <= MT * TERMS, "a piece of staging per matrix instruction");
         float share = 0.0F;
         u32 piece1[4] = {0, 0, 0, 0};
@@ -1108,7 +1142,19 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         constexpr int PIECE2 = DP <= 8 ? 1 : KS; // first cell of the second pieces
         auto chunk = [&](auto c_tag) __attribute__((always_inline)) {
             constexpr int c = decltype(c_tag)::value;
-            if constexpr (c < PAIRS_OF_VALUES)
+            if constexpr (MODE == 2)
+            {
+                // one unit of the image per matrix instruction, then the request for the next stage
+                if constexpr (c < IU)
+                {
+                    deposit_image_unit(into, c_tag);
+                }
+                else
+                {
+                    fetch_image(next_base + PT);
+                }
+            }
+            else if constexpr (c < PAIRS_OF_VALUES)
             {
                 // two values: pieces, share of the norm, fp32 rows
                 const vfloat2 pair{pre[2 * c], pre[2 * c + 1]};
@@ -1551,14 +1597,24 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 __builtin_amdgcn_s_sleep(1);
             }
         };
-        fetch(n_begin);
-        // the query fragment and the first stage have arrived (nothing else is in flight yet)
-        __builtin_amdgcn_s_waitcnt(0x0F70);
-        deposit(stages, n_begin);
-        count_in(0);
-        if (n_begin + PT < n)
+        if (EXACT && a.image != nullptr)
         {
-            fetch(n_begin + PT);
+            fetch_image(n_begin);
+            static_for<0, IU>([&](auto j_tag) { deposit_image_unit(stages, j_tag); });
+            count_in(0);
+            fetch_image(n_begin + PT);
+        }
+        else
+        {
+            fetch(n_begin);
+            // the query fragment and the first stage have arrived (nothing else is in flight yet)
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            deposit(stages, n_begin);
+            count_in(0);
+            if (n_begin + PT < n)
+            {
+                fetch(n_begin + PT);
+            }
         }
         int slot = 0;  // of the stage being multiplied
         int round = 0; // how often that slot has been used before
@@ -1569,8 +1625,8 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             // filter_values_and_stage).  (The stage after the last one is "written" from whatever
             // the registers hold, into a slot that nobody reads any more.)  Point matrices below
             // 2 GiB request the stage after the next one in the middle of those instructions.
-            auto pass = [&](auto early_tag) __attribute__((always_inline)) {
-                constexpr bool EARLY_FETCH = decltype(early_tag)::value;
+            auto pass = [&](auto mode_tag) __attribute__((always_inline)) {
+                constexpr int MODE = decltype(mode_tag)::value;
                 for (int base = n_begin; base < n; base += PT)
                 {
                     wait_for(slot, round + 1);
@@ -1579,9 +1635,9 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                     const float* const stage = stages + slot * STAGE_FLOATS;
                     vfloat16 w[MT];
                     __builtin_amdgcn_sched_barrier(0);
-                    filter_values_and_stage(stage, w, stages + next * STAGE_FLOATS, base + PT, early_tag);
+                    filter_values_and_stage(stage, w, stages + next * STAGE_FLOATS, base + PT, mode_tag);
                     count_in(next);
-                    if constexpr (!EARLY_FETCH)
+                    if constexpr (MODE == 0)
                     {
                         if (base + 2 * PT < n)
                         {
@@ -1594,13 +1650,17 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                     round += slot == 0 ? 1 : 0;
                 }
             };
-            if (small_points)
+            if (a.image != nullptr)
             {
-                pass(std::true_type{});
+                pass(std::integral_constant<int, 2>{});
+            }
+            else if (small_points)
+            {
+                pass(std::integral_constant<int, 1>{});
             }
             else
             {
-                pass(std::false_type{});
+                pass(std::integral_constant<int, 0>{});
             }
         }
         else

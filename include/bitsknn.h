@@ -228,9 +228,19 @@ int bitsknn_fused_l2_topk_f32(const float* queries_dim_major, const float* point
  * bitsknn_fused_workspace_bytes returns the size the call wants: 8*q*ranges*k bytes, at most 64
  * ranges; 0 when the queries fill the GPU by themselves.  A smaller workspace (4-byte aligned) is
  * not an error: the call uses as many ranges as fit, down to the single kernel without any.
+ *
+ * The stage image.  In the exact arithmetic (dim <= 64) every workgroup cuts every point into bf16
+ * pieces again.  With bitsknn_fused_image_bytes(dim, n) more bytes in the workspace, behind the
+ * partial lists rounded up to a multiple of 256 bytes (and the workspace 16-byte aligned), a launch
+ * of its own writes the stages of the whole point matrix there once per call and the fused kernel
+ * copies them (65536 queries x 2^20 points, d = 32, k = 32: a quarter of the kernel's time).  It is
+ * written from 4096 queries on (bitsknn_fused_tuning::image overrides that); the results are the
+ * same bit for bit with and without it.  bitsknn_fused_image_bytes is 0 where no image is used
+ * (dim > 64, or an image of 2 GiB and more).
  * Errors as for bitsknn_fused_l2_topk_f32.
  */
 size_t bitsknn_fused_workspace_bytes(int32_t q, int32_t n, int k);
+size_t bitsknn_fused_image_bytes(int dim, int32_t n);
 int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major, const float* points_dim_major,
                                  int dim, int32_t q, int32_t n, float* out_dist, int32_t* out_label,
                                  int k, int query_reg, int db_reg, int dim_reg, int block_query_dim,
@@ -286,6 +296,10 @@ int bitsknn_fused_l2_topk_f32_ex(const float* queries_dim_major, const float* po
  *                 (one stage in every first_radius, 2 .. 4096; -1: never; 0: the library's choice,
  *                 lists of 128 and more on at least 2^17 points, of 64 and more over ranges); a
  *                 sample whose lists would not reach the rank the guarantee needs is not taken
+ *   image         whether the points are cut into the stages of BITSKNN_FUSED_EXACT once, into the
+ *                 workspace behind the partial lists (bitsknn_fused_image_bytes), instead of by
+ *                 every workgroup again: 1 = whenever the workspace has room, -1 = never, 0 = the
+ *                 library's choice (from 4096 queries on)
  * tuning == NULL: the library's choices.  Results do not depend on the tuning (for
  * BITSKNN_FUSED_EXACT bit for bit; for the other arithmetics the distances of a point can differ in
  * the last bit between one range and several).  bitsknn/tuning.py sweeps these and records the
@@ -296,7 +310,8 @@ typedef struct bitsknn_fused_tuning
 {
     int32_t ranges;
     int32_t first_radius;
-    int32_t reserved[6];
+    int32_t image;
+    int32_t reserved[5];
 } bitsknn_fused_tuning;
 int bitsknn_fused_l2_topk_f32_tuned(const float* queries_dim_major, const float* points_dim_major,
                                     int dim, int32_t q, int32_t n, float* out_dist, int32_t* out_label,
