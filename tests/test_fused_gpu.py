@@ -30,22 +30,30 @@ def _fused(bk, dev, points, queries, k, params=(8, 4, 2), bqd=1, dim_mult=1, wor
     import torch
     pd = _dm(points, dev).reshape(points.shape[1], points.shape[0])
     qd = _dm(queries, dev).reshape(queries.shape[1], queries.shape[0])
+    if arithmetic == "image":
+        # the default arithmetic with the stages cut once into the workspace (forced: the library
+        # itself only does it from a few thousand queries on), ranges as the library chooses
+        od, ol = bk.fused_l2_topk(qd, pd, k, workspace="image", tuning=(0, 0, 1))
+        bk.fused_status()
+        return od.cpu().numpy(), ol.cpu().numpy()
     od, ol = bk.fused_l2_topk(qd, pd, k, params, bqd, dim_mult, workspace=workspace, arithmetic=arithmetic)
     bk.fused_status()  # synchronises; raises if a wave gave up a wait for a stage
     return od.cpu().numpy(), ol.cpu().numpy()
 
 
 MODES = ["default", "mfma"]
+MODES_AND_IMAGE = ["default", "mfma", "image"]
 
 
 def _arith(bk, mode):
-    """C-ABI arithmetic of a test mode: None = the plain entry points"""
-    return {"default": None, "mfma": bk.FUSED_FP32, "bf16x3": bk.FUSED_BF16X3}[mode]
+    """C-ABI arithmetic of a test mode: None = the plain entry points; "image" = the default
+    arithmetic through bitsknn_fused_l2_topk_f32_tuned with the stage image (see _fused)"""
+    return {"default": None, "mfma": bk.FUSED_FP32, "bf16x3": bk.FUSED_BF16X3, "image": "image"}[mode]
 
 
 def _bits(mode, dim):
     """whether the result of this mode must equal the oracle's bit for bit"""
-    return mode == "default" and dim <= 64
+    return mode in ("default", "image") and dim <= 64
 
 
 def _check(oracle, points, queries, k, gd, gl, min_recall=0.999, bar_dim=None, bits=False):
@@ -104,7 +112,7 @@ def test_reference_unit_test_shapes(bk, dev, oracle, d, k, n, q, mode):
     _check(oracle, p, s, k, gd, gl, bits=_bits(mode, d))
 
 
-@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("mode", MODES_AND_IMAGE)
 @pytest.mark.parametrize("k", [4, 8, 16, 32, 64, 128, 256])
 @pytest.mark.parametrize("d", [4, 8, 16, 32, 64])
 def test_all_k_values(bk, dev, oracle, k, d, mode):
@@ -113,7 +121,7 @@ def test_all_k_values(bk, dev, oracle, k, d, mode):
     _check(oracle, p, s, k, gd, gl, bits=_bits(mode, d))
 
 
-@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("mode", MODES_AND_IMAGE)
 @pytest.mark.parametrize("d", [1, 2, 3, 5, 7, 9, 15, 17, 31, 33, 48, 49, 63, 64, 65, 100, 113, 200, 256])
 def test_dimensions(bk, dev, oracle, d, mode):
     p, s = oracle.generate(d, 3000, 70, d)
@@ -121,7 +129,7 @@ def test_dimensions(bk, dev, oracle, d, mode):
     _check(oracle, p, s, 16, gd, gl, bits=_bits(mode, d))
 
 
-@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("mode", MODES_AND_IMAGE)
 @pytest.mark.parametrize("n,q", [(1, 1), (31, 5), (32, 33), (33, 127), (255, 128), (257, 129), (1000, 300), (5001, 1)])
 def test_ragged_counts(bk, dev, oracle, n, q, mode):
     for d in (8, 24):
@@ -134,12 +142,14 @@ def test_ragged_counts(bk, dev, oracle, n, q, mode):
 # points per stage by padded dimension.  fp32 matrix instructions: 256 up to 16 dimensions, 128 / 64
 # / 32 for 32 / 64 / 128; the exact arithmetic and bf16x3: 128 up to 16 dimensions, 64 / 32 for 32 / 64
 @pytest.mark.parametrize("d", [8, 16, 32, 64, 100])
-@pytest.mark.parametrize("mode", ["default", "mfma", "bf16x3"])
+@pytest.mark.parametrize("mode", ["default", "mfma", "bf16x3", "image"])
 def test_point_counts_around_whole_stages(bk, dev, oracle, d, mode):
     # one to five stages, each count one short of, at and one past a whole stage: the ring of three
     # stage buffers starts, wraps around and ends at every position
     if mode == "bf16x3" and not 9 <= d <= 64:
         pytest.skip("bf16x3 products serve 9 to 64 dimensions")
+    if mode == "image" and d > 64:
+        pytest.skip("the stage image serves up to 64 dimensions")
     if mode == "mfma" or d > 64:
         stage = {8: 256, 16: 256, 32: 128, 64: 64, 100: 32}[d]
     else:
@@ -203,7 +213,7 @@ def test_duplicate_points_are_ordered_by_index(bk, dev, oracle):
             assert np.array_equal(gd.view(np.uint32), ed.view(np.uint32))
 
 
-@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("mode", MODES_AND_IMAGE)
 @pytest.mark.parametrize("d,k", [(8, 32), (16, 4), (16, 32), (32, 32), (64, 16), (16, 64), (100, 32)])
 def test_points_that_come_ever_closer(bk, dev, oracle, d, k, mode):
     # Every point is nearer to every query than all points before it, so every tile brings each
@@ -279,6 +289,9 @@ def test_the_filter_never_drops_a_neighbour(bk, dev, oracle, d, kind):
     if kind in ("signs", "near"):
         wd, wl = _fused(bk, dev, p, s, k, workspace="auto")
         assert np.array_equal(gd, wd) and np.array_equal(gl, wl)
+    # the same through the stage image (the launch that writes it cuts the points the same way)
+    wd, wl = _fused(bk, dev, p, s, k, arithmetic="image")
+    assert np.array_equal(gd.view(np.uint32), wd.view(np.uint32)) and np.array_equal(gl, wl)
 
 
 # reference-held checksums of the fused runs (data/fused-*.err), query 0
@@ -585,3 +598,40 @@ def test_tuned_entry_point(bk, dev, oracle):
                          ((0, -2), "first_radius must be"), ((0, 5000), "first_radius must be")):
         with pytest.raises(bk.BitsKnnError, match=message):
             bk.fused_l2_topk(qd, pd, k, workspace=space, tuning=bad)
+
+
+def test_stage_image(bk, dev, oracle):
+    """The stage image: bitsknn_fused_image_bytes more bytes in the workspace, behind the partial
+    lists, and the points are cut into the stages of the default arithmetic once per call.  Same
+    result bit for bit with one range and several, with first radii from a sample, with a workspace
+    that is too small for it (no image then) and through the plain workspace entry point, which
+    writes it from 4096 queries on."""
+    import torch
+    assert bk.fused_image_bytes(32, 1 << 20) == (1 << 20) // 64 * (32 * 64 * 4 + 9 * 64 * 16)
+    assert bk.fused_image_bytes(8, 1000) == 8 * (8 * 128 * 4 + 3 * 128 * 16)
+    assert bk.fused_image_bytes(65, 1000) == 0 and bk.fused_image_bytes(64, 1 << 23) == 0
+    n, q, d, k = (1 << 17) + 300, 260, 24, 64
+    p, s = oracle.generate(405, n, q, d)
+    pd = torch.from_numpy(np.ascontiguousarray(p.T)).to(dev)
+    qd = torch.from_numpy(np.ascontiguousarray(s.T)).to(dev)
+    ed, el = oracle.topk(oracle.dist(s, p, "partial"), k)
+    lists = 8 * q * 64 * k
+    space = torch.empty((lists + 255) // 256 * 256 + bk.fused_image_bytes(d, n), dtype=torch.uint8, device=dev)
+    for tuning in [(1, -1, 1), (1, 64, 1), (8, -1, 1), (64, 64, 1), (3, 32, 1), (0, 0, 1), (0, 0, 0), (4, 0, -1)]:
+        space.fill_(0xFF)
+        od, ol = bk.fused_l2_topk(qd, pd, k, workspace=space, tuning=tuning)
+        bk.fused_status()
+        assert np.array_equal(od.cpu().numpy().view(np.uint32), ed.view(np.uint32)), tuning
+        assert np.array_equal(ol.cpu().numpy(), el), tuning
+    # a workspace with room for the lists of 4 ranges only: ranges, no image
+    od, ol = bk.fused_l2_topk(qd, pd, k, workspace=space[:8 * q * 4 * k + 1000], tuning=(4, 0, 1))
+    bk.fused_status()
+    assert np.array_equal(ol.cpu().numpy(), el)
+    # many queries: the plain workspace entry point writes the image by itself
+    n, q, d, k = 30000, 4500, 8, 16
+    p, s = oracle.generate(406, n, q, d)
+    ed, el = oracle.topk(oracle.dist(s, p, "partial"), k)
+    gd, gl = _fused(bk, dev, p, s, k, workspace="image")
+    assert np.array_equal(gd.view(np.uint32), ed.view(np.uint32)) and np.array_equal(gl, el)
+    with pytest.raises(bk.BitsKnnError, match="image must be"):
+        bk.fused_l2_topk(qd, pd, 64, workspace=space, tuning=(0, 0, 2))
