@@ -391,11 +391,14 @@ def fused_roofline(q, n, d, seconds):
 
 def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=65536, n=1 << 20, long_ks=(),
               workspace=False):
-    """Config 5: bits-fused at d x k through the plain entry points (the reference's arithmetic
-    behind a filter on the bf16 matrix instructions); the d = 32, k = 32 case also with the
-    distances from the fp32 matrix instructions and from bf16x3 products.  long_ks: list lengths
-    beyond the configuration's, reported apart (`long_lists`).  workspace: through the entry point
-    that may cut the points into ranges (few queries)."""
+    """Config 5: bits-fused at d x k in the default arithmetic (the reference's, behind a filter on
+    the bf16 matrix instructions) through the workspace entry point, as the knn driver calls it: the
+    workspace has room for the stage image, so the points are cut into bf16 pieces once per call
+    (that launch is inside the timed call); `ms_plain_entry_point` is the entry point without a
+    workspace beside it.  The d = 32, k = 32 case also with the distances from the fp32 matrix
+    instructions and from bf16x3 products.  long_ks: list lengths beyond the configuration's,
+    reported apart (`long_lists`).  workspace: room for partial lists as well, so that few queries
+    search the points in ranges."""
     import numpy as np
     grid = []
     long_lists = []
@@ -410,15 +413,23 @@ def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=6553
         for k in tuple(ks) + tuple(long_ks):
             out_d = torch.full((q, k), -1.0, dtype=torch.float32, device=dev)
             out_l = torch.empty((q, k), dtype=torch.int32, device=dev)
-            space = None
-            if workspace:
-                space = torch.empty(max(1, bitsknn.fused_workspace_bytes(q, n, k)), dtype=torch.uint8, device=dev)
+            lists = bitsknn.fused_workspace_bytes(q, n, k) if workspace else 0
+            space = torch.empty(max(1, (lists + 255) // 256 * 256 + bitsknn.fused_image_bytes(d, n)),
+                                dtype=torch.uint8, device=dev)
+            plain_s = None
+            if not workspace:
+                _, plain_s = timer.run(lambda: bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d,
+                                                                     out_label=out_l), steps, 2)
+                out_d.fill_(-1.0)
             _, seconds = timer.run(lambda: bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l,
                                                                  workspace=space), steps, 2)
             roof = fused_roofline(q, n, d, seconds)
             entry = {"d": d, "k": k, "ms": seconds * 1e3, "queries_per_s": q / seconds,
                      "pairs_per_s": q * n / seconds, "frac": roof["frac"],
                      "algorithmic_over_fp32_matrix_peak": roof["algorithmic_over_fp32_matrix_peak"]}
+            if plain_s is not None:
+                entry["ms_plain_entry_point"] = plain_s * 1e3
+            del space
             if check:
                 if part is None:
                     points_h = np.ascontiguousarray(points.cpu().numpy().T)
@@ -436,8 +447,11 @@ def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=6553
                             "arithmetic": "sequential fp32 fused multiply-adds in dimension order (the reference's) "
                                           "for every pair that passes a guaranteed lower bound from bf16 matrix "
                                           "instructions",
+                            "entry_point": "bitsknn_fused_l2_topk_f32_ws with room for the stage image in the "
+                                           "workspace (one launch that cuts the points, one fused launch)",
                             "launches_timed": steps,
                             "queries_per_s": q / seconds, "ms": seconds * 1e3, "pairs_per_s": q * n / seconds,
+                            "ms_plain_entry_point": plain_s * 1e3,
                             "roofline": roof}
                 if check:
                     headline["verified"] = entry["verified"]
@@ -554,6 +568,8 @@ def summarise(result):
     if "fused" in result:
         f = result["fused"]
         out["fused_grid_ms"] = {f"d{e['d']}_k{e['k']}": r3(e["ms"]) for e in f.get("grid", [])}
+        out["fused_grid_ms_plain_entry_point"] = {f"d{e['d']}_k{e['k']}": r3(e["ms_plain_entry_point"])
+                                                  for e in f.get("grid", []) if "ms_plain_entry_point" in e}
         out["fused_grid_frac_bf16_mfma"] = {f"d{e['d']}_k{e['k']}": r3(e["frac"]) for e in f.get("grid", [])}
         out["fused_grid_algorithmic_over_fp32_mfma_peak"] = {
             f"d{e['d']}_k{e['k']}": r3(e["algorithmic_over_fp32_matrix_peak"]) for e in f.get("grid", [])}

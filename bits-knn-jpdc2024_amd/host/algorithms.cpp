@@ -426,28 +426,37 @@ public:
         const auto queries = to_dim_major(args_.queries, query_count(), dim(), args_.queries_layout);
         points_ = device_buffer<float>{points.size()};
         queries_ = device_buffer<float>{queries.size()};
-        // BITSKNN_FUSED_TUNING="ranges=R,first_radius=F" in the environment: the launch parameters a
-        // tuning sweep varies here (bitsknn_fused_tuning), in place of the library's own choice
+        // BITSKNN_FUSED_TUNING="ranges=R,first_radius=F[,image=I]" in the environment: the launch
+        // parameters a tuning sweep varies here (bitsknn_fused_tuning), in place of the library's own
+        // choice
         tuned_ = false;
         tuning_ = bitsknn_fused_tuning{};
         if (const char* text = std::getenv("BITSKNN_FUSED_TUNING"); text != nullptr && *text != '\0')
         {
             int ranges = 0;
             int first_radius = 0;
-            if (std::sscanf(text, "ranges=%d,first_radius=%d", &ranges, &first_radius) != 2)
+            int image = 0;
+            if (std::sscanf(text, "ranges=%d,first_radius=%d,image=%d", &ranges, &first_radius, &image) < 2)
             {
-                throw std::runtime_error("BITSKNN_FUSED_TUNING must read ranges=R,first_radius=F");
+                throw std::runtime_error("BITSKNN_FUSED_TUNING must read ranges=R,first_radius=F[,image=I]");
             }
             tuning_.ranges = ranges;
             tuning_.first_radius = first_radius;
+            tuning_.image = image;
             tuned_ = true;
         }
         // partial lists of the point ranges when the queries alone do not fill the GPU (room for the
-        // 64 ranges a tuning may ask for)
-        workspace_ = device_buffer<unsigned char>{
+        // 64 ranges a tuning may ask for), then, from the next multiple of 256 bytes on, room for the
+        // stages of the exact arithmetic cut once per call
+        const std::size_t lists =
             tuned_ ? query_count() * 64 * k() * 8
                    : bitsknn_fused_workspace_bytes(static_cast<std::int32_t>(query_count()),
-                                                   static_cast<std::int32_t>(point_count()), static_cast<int>(k()))};
+                                                   static_cast<std::int32_t>(point_count()), static_cast<int>(k()));
+        const std::size_t image =
+            arithmetic_ == BITSKNN_FUSED_EXACT
+                ? bitsknn_fused_image_bytes(static_cast<int>(dim()), static_cast<std::int32_t>(point_count()))
+                : 0;
+        workspace_ = device_buffer<unsigned char>{(lists + 255) / 256 * 256 + image};
         transfer_in_.start();
         points_.upload(points.data(), points.size());
         queries_.upload(queries.data(), queries.size());
