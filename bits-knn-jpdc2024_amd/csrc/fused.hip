@@ -142,10 +142,14 @@ constexpr int SAMPLE_POINTS_RANGES = 2048;
 constexpr int SAMPLE_MIN_POINTS = 1 << 17; // at least 8 (2 with ranges) sampled stages of any size
 constexpr int SAMPLE_MIN_K = 64;
 constexpr int SAMPLE_MIN_K_RANGES = 64; // (k <= 32: the three extra launches cost what the merges save)
-// fewest queries for which the stage image of the exact arithmetic is built when the workspace has
-// room for it (its launch reads and writes the points once, about 0.1 ms for 2^20 points in 32
-// dimensions; every workgroup of 128 queries saves the cutting of all its points)
+// The stage image of the exact arithmetic is built, when the workspace has room for it, from this
+// many queries on (its launch reads and writes the points once, about 0.1 ms for 2^20 points in 32
+// dimensions; every workgroup of 128 queries saves the cutting of all its points) in up to this many
+// dimensions (65536 queries x 2^20 points, k = 32: d = 8 7.4 -> 7.1 ms, d = 16 9.9 -> 9.6 ms, but
+// d = 32 16.9 -> 17.3 ms and d = 64 33.2 -> 33.7 ms: the copy moves twice the bytes that the cutting
+// reads, and there the vector instructions of the cutting hide behind the matrix instructions)
 constexpr int IMAGE_MIN_QUERIES = 4096;
+constexpr int IMAGE_MAX_DIM = 16;
 
 int first_radius_rank(int k, int scale)
 {
@@ -362,7 +366,8 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
         const size_t image_bytes = fused_image_bytes(dim, n);
         const size_t lists = splits > 1 ? partial_list_bytes(q, splits, k) : 0;
         const size_t offset = (lists + 255) / 256 * 256;
-        const bool wanted = (tuning != nullptr && tuning->image == 1) || q >= IMAGE_MIN_QUERIES;
+        const bool wanted =
+            (tuning != nullptr && tuning->image == 1) || (q >= IMAGE_MIN_QUERIES && dim <= IMAGE_MAX_DIM);
         if (wanted && image_bytes > 0 && image_bytes < (1ULL << 31) && offset + image_bytes <= workspace_bytes &&
             reinterpret_cast<std::uintptr_t>(workspace) % 16 == 0)
         {

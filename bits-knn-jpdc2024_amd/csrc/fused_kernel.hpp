@@ -1072,16 +1072,17 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             }
         });
     };
-    // EXACT: the filter values of a stage as above, with the staging of the next stage (`into`,
-    // first point `next_base`; the values are in `pre`) cut into pieces of a few vector and LDS
-    // instructions that are placed one after each of the first matrix instructions, where they
-    // execute next to it.  The staging code has no branch (every thread of a point writes the norm
-    // cell); scheduling barriers keep the order written here.
-    auto filter_values_and_stage = [&](const float* stage, vfloat16 (&w)[MT], float* into, int next_base, auto mode_tag) __attribute__((always_inline)) {
-        constexpr int MODE = decltype(mode_tag)::value; // 0: the values of the stage after the next
-                                                        // one are requested after this call, 1: in
-                                                        // the middle of it, 2: stages from an image
-        constexpr bool EARLY_FETCH = MODE == 1;
+    // EXACT: the filter values of a stage as above, with the cutting of the values in `pre` (a stage
+    // further on) into bf16 pieces placed between the matrix instructions, a few vector instructions
+    // after each of the first ones, where they execute next to it; scheduling barriers keep the
+    // order written here.  The pieces stay in registers (cut1, cut2, cut_norm) until write_cut puts
+    // them into a stage.  `cut_base`: first point of the stage the values belong to.  MODE 2 (stages
+    // from an image): nothing to cut.
+    u32 cut1[4] = {0, 0, 0, 0};
+    u32 cut2[4] = {0, 0, 0, 0};
+    u32 cut_norm = 0;
+    auto filter_values_and_cut = [&](const float* stage, vfloat16 (&w)[MT], int cut_base, auto mode_tag) __attribute__((always_inline)) {
+        constexpr int MODE = decltype(mode_tag)::value;
         // (the cells are read in the order in which the matrix instructions take them, the norm
         // cell last, so that the first instruction waits for the first read only)
         const vuint4* const cells = reinterpret_cast<const vuint4*>(stage + DP * PT);
@@ -1130,78 +1131,25 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             }
         }
         __builtin_amdgcn_sched_barrier(0);
-        // staging state
         constexpr int PAIRS_OF_VALUES = VPT / 2;
-        constexpr int CHUNKS = MODE == 2 ? IU + 1 : PAIRS_OF_VALUES + 3;
-        static_assert(!EXACT || CHUNKS <= MT * TERMS, "a piece of staging per matrix instruction");
+        constexpr int CHUNKS = MODE == 2 ? 0 : PAIRS_OF_VALUES + 1;
+        static_assert(!EXACT || CHUNKS <= MT * TERMS, "a piece of the cutting per matrix instruction");
         float share = 0.0F;
-        u32 piece1[4] = {0, 0, 0, 0};
-        u32 piece2[4] = {0, 0, 0, 0};
-        u32 norm_word = 0;
-        vuint4* const into_cells = reinterpret_cast<vuint4*>(into + DP * PT);
-        constexpr int PIECE2 = DP <= 8 ? 1 : KS; // first cell of the second pieces
         auto chunk = [&](auto c_tag) __attribute__((always_inline)) {
             constexpr int c = decltype(c_tag)::value;
-            if constexpr (MODE == 2)
+            if constexpr (c < PAIRS_OF_VALUES)
             {
-                // one unit of the image per matrix instruction, then the request for the next stage
-                if constexpr (c < IU)
-                {
-                    deposit_image_unit(into, c_tag);
-                }
-                else
-                {
-                    fetch_image(next_base + PT);
-                }
-            }
-            else if constexpr (c < PAIRS_OF_VALUES)
-            {
-                // two values: pieces, share of the norm, fp32 rows
+                // two values: pieces, share of the norm
                 const vfloat2 pair{pre[2 * c], pre[2 * c + 1]};
                 const u32 first = __builtin_bit_cast(u32, __builtin_convertvector(pair, vbf16x2));
                 const vfloat2 rest{pair.x - __builtin_bit_cast(float, first << 16U),
                                    pair.y - __builtin_bit_cast(float, first & 0xFFFF0000U)};
-                piece1[c] = first;
-                piece2[c] = __builtin_bit_cast(u32, __builtin_convertvector(rest, vbf16x2));
+                cut1[c] = first;
+                cut2[c] = __builtin_bit_cast(u32, __builtin_convertvector(rest, vbf16x2));
                 share = __builtin_fmaf(pair.x, pair.x, share);
                 share = __builtin_fmaf(pair.y, pair.y, share);
-                into[(sd0 + 2 * c) * PT + sp] = pair.x;
-                into[(sd0 + 2 * c + 1) * PT + sp] = pair.y;
             }
-            else if constexpr (c == PAIRS_OF_VALUES)
-            {
-                if constexpr (VPT == 8)
-                {
-                    into_cells[t] = vuint4{piece1[0], piece1[1], piece1[2], piece1[3]};
-                    into_cells[PIECE2 * PT + t] = vuint4{piece2[0], piece2[1], piece2[2], piece2[3]};
-                }
-                else
-                {
-                    // half a cell per thread
-                    typedef u32 vuint2 __attribute__((ext_vector_type(2)));
-                    vuint2* const halves = reinterpret_cast<vuint2*>(into + DP * PT);
-                    const int h = sd0 / 4;
-                    halves[2 * sp + h] = vuint2{piece1[0], piece1[1]};
-                    halves[2 * (PIECE2 * PT + sp) + h] = vuint2{piece2[0], piece2[1]};
-                }
-                // the registers of the values are free: the stage after the next one is requested
-                // now, so that its loads have the rest of this stage and the start of the next one
-                // (buffer loads without a branch: beyond the matrix they read zero, and points
-                // from n on, whatever their values, carry the norm that only passes an infinite
-                // radius and are dropped by their labels)
-                if constexpr (EARLY_FETCH)
-                {
-                    const int stage_off =
-                        ((next_base + PT) * a.sample_scale + a.sample_offset) * static_cast<int>(sizeof(float));
-#pragma unroll
-                    for (int i = 0; i < VPT; ++i)
-                    {
-                        pre[i] = __builtin_bit_cast(
-                            float, __builtin_amdgcn_raw_buffer_load_b32(point_rsrc, load_off[i], stage_off, 0));
-                    }
-                }
-            }
-            else if constexpr (c == PAIRS_OF_VALUES + 1)
+            else
             {
                 if constexpr (DP == 64)
                 {
@@ -1212,11 +1160,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 const u32 first = __builtin_bit_cast(u32, __builtin_convertvector(whole, vbf16x2)) & 0xFFFFU;
                 const vfloat2 rest{lowered - __builtin_bit_cast(float, first << 16U), 0.0F};
                 const u32 second = __builtin_bit_cast(u32, __builtin_convertvector(rest, vbf16x2)) & 0xFFFFU;
-                norm_word = next_base + sp < n ? first | (second << 16U) : BF16_HUGE;
-            }
-            else
-            {
-                reinterpret_cast<u32*>(into_cells + (G::CELLS - 1) * PT + sp)[norm_slot] = norm_word;
+                cut_norm = cut_base + sp < n ? first | (second << 16U) : BF16_HUGE;
             }
         };
         static_for<0, TERMS>([&](auto j_tag) {
@@ -1240,6 +1184,40 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 __builtin_amdgcn_sched_barrier(0);
             });
         });
+    };
+    // EXACT: the stage cut by filter_values_and_cut (fp32 rows from `pre`, cells from the pieces), or
+    // the units of the image, into LDS; a handful of LDS writes.
+    auto write_cut = [&](float* into, auto mode_tag) __attribute__((always_inline)) {
+        constexpr int MODE = decltype(mode_tag)::value;
+        if constexpr (MODE == 2)
+        {
+            static_for<0, IU>([&](auto j_tag) { deposit_image_unit(into, j_tag); });
+        }
+        else
+        {
+#pragma unroll
+            for (int i = 0; i < VPT; ++i)
+            {
+                into[(sd0 + i) * PT + sp] = pre[i];
+            }
+            vuint4* const into_cells = reinterpret_cast<vuint4*>(into + DP * PT);
+            constexpr int PIECE2 = DP <= 8 ? 1 : KS; // first cell of the second pieces
+            if constexpr (VPT == 8)
+            {
+                into_cells[t] = vuint4{cut1[0], cut1[1], cut1[2], cut1[3]};
+                into_cells[PIECE2 * PT + t] = vuint4{cut2[0], cut2[1], cut2[2], cut2[3]};
+            }
+            else
+            {
+                // half a cell per thread
+                typedef u32 vuint2 __attribute__((ext_vector_type(2)));
+                vuint2* const halves = reinterpret_cast<vuint2*>(into + DP * PT);
+                const int h = sd0 / 4;
+                halves[2 * sp + h] = vuint2{cut1[0], cut1[1]};
+                halves[2 * (PIECE2 * PT + sp) + h] = vuint2{cut2[0], cut2[1]};
+            }
+            reinterpret_cast<u32*>(into_cells + (G::CELLS - 1) * PT + sp)[norm_slot] = cut_norm;
+        }
     };
     // EXACT, second half of a stage.  First every tile is filtered without a branch: the smallest
     // filter value of every lane per tile and over the stage.  Only if some lane's is not above its
@@ -1597,14 +1575,7 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 __builtin_amdgcn_s_sleep(1);
             }
         };
-        if (EXACT && a.image != nullptr)
-        {
-            fetch_image(n_begin);
-            static_for<0, IU>([&](auto j_tag) { deposit_image_unit(stages, j_tag); });
-            count_in(0);
-            fetch_image(n_begin + PT);
-        }
-        else
+        if constexpr (!EXACT)
         {
             fetch(n_begin);
             // the query fragment and the first stage have arrived (nothing else is in flight yet)
@@ -1621,33 +1592,95 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
         BITSKNN_FT_LAP(5);
         if constexpr (EXACT)
         {
-            // The next stage is written while the matrix instructions of this one run (see
-            // filter_values_and_stage).  (The stage after the last one is "written" from whatever
-            // the registers hold, into a slot that nobody reads any more.)  Point matrices below
-            // 2 GiB request the stage after the next one in the middle of those instructions.
-            auto pass = [&](auto mode_tag) __attribute__((always_inline)) {
-                constexpr int MODE = decltype(mode_tag)::value;
-                for (int base = n_begin; base < n; base += PT)
+            // The default arithmetic writes two stages ahead, at the end of an iteration.  Step k
+            // writes stage k and counts at ready[k % 3]: steps 0 and 1 before the loop, step i + 2 at
+            // the end of iteration i, which reads stage i.  Before it overwrites the slot of stage
+            // i - 1 with stage i + 2, a wave waits until every wave has counted step i + 1, that is,
+            // has finished iteration i - 1 (and written stage i + 1 at its end): the one wait of an
+            // iteration also is what the next iteration's reads need.  So a wave may be a whole
+            // iteration ahead of the slowest one of its workgroup -- the work on candidates differs
+            // from wave to wave and stage to stage, and with less slack every wave pays for the
+            // slowest one of every stage.  Every wave counts every step whatever its tiles hold,
+            // and a wait is for counts that the other waves reach without waiting for this one.
+            // The values of a stage are requested an iteration before they are cut (during the
+            // matrix instructions) and written.  Past the last stage the waves write stages that
+            // nobody reads (same waits, same counts).
+            auto count_step = [&](int counter) __attribute__((always_inline)) {
+                // (LDS executes the instructions of a wave in order: the count follows the writes
+                // without a wait in between; the fence keeps the compiler from moving them)
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                if (lane == 0)
                 {
-                    wait_for(slot, round + 1);
-                    BITSKNN_FT_LAP(0);
-                    const int next = slot + 1 == NB ? 0 : slot + 1;
-                    const float* const stage = stages + slot * STAGE_FLOATS;
-                    vfloat16 w[MT];
-                    __builtin_amdgcn_sched_barrier(0);
-                    filter_values_and_stage(stage, w, stages + next * STAGE_FLOATS, base + PT, mode_tag);
-                    count_in(next);
-                    if constexpr (MODE == 0)
+                    __hip_atomic_fetch_add(ready + counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+            };
+            auto pass = [&](auto mode_tag) __attribute__((always_inline)) {
+                constexpr int MODE = decltype(mode_tag)::value; // 0: point matrices of 2 GiB and more,
+                                                                // 1: buffer loads, 2: stages from an image
+                auto request = [&](int base) __attribute__((always_inline)) {
+                    if constexpr (MODE == 2)
                     {
-                        if (base + 2 * PT < n)
+                        fetch_image(base);
+                    }
+                    else if constexpr (MODE == 1)
+                    {
+                        // (buffer loads without a branch: beyond the matrix they read zero, and
+                        // points from n on, whatever their values, carry the norm that only passes an
+                        // infinite radius and are dropped by their labels)
+                        const int stage_off = (base * a.sample_scale + a.sample_offset) * static_cast<int>(sizeof(float));
+#pragma unroll
+                        for (int i = 0; i < VPT; ++i)
                         {
-                            fetch(base + 2 * PT);
+                            pre[i] = __builtin_bit_cast(
+                                float, __builtin_amdgcn_raw_buffer_load_b32(point_rsrc, load_off[i], stage_off, 0));
                         }
                     }
+                    else
+                    {
+                        fetch(base < n ? base : n_begin);
+                    }
+                };
+                auto write_whole = [&](float* into, int base) __attribute__((always_inline)) {
+                    if constexpr (MODE == 2)
+                    {
+                        write_cut(into, mode_tag);
+                    }
+                    else
+                    {
+                        deposit(into, base);
+                    }
+                };
+                request(n_begin);
+                write_whole(stages, n_begin);
+                count_step(0);
+                request(n_begin + PT);
+                wait_for(0, 1);
+                write_whole(stages + STAGE_FLOATS, n_begin + PT);
+                count_step(1);
+                request(n_begin + 2 * PT);
+                int reads = 0;   // slot of the stage being read (i % 3); its stage is complete
+                int waits = 1;   // counter of step i + 1
+                int writes = 2;  // slot of stage i + 2, counter of step i + 2
+                int uses = 1;    // how often the counter `waits` has been used, this use included
+                for (int base = n_begin; base < n; base += PT)
+                {
+                    BITSKNN_FT_LAP(0);
+                    const float* const stage = stages + reads * STAGE_FLOATS;
+                    vfloat16 w[MT];
+                    __builtin_amdgcn_sched_barrier(0);
+                    filter_values_and_cut(stage, w, base + 2 * PT, mode_tag);
                     BITSKNN_FT_LAP(2);
                     filter_and_append(w, stage, base);
-                    slot = next;
-                    round += slot == 0 ? 1 : 0;
+                    wait_for(waits, uses);
+                    BITSKNN_FT_LAP(1);
+                    write_cut(stages + writes * STAGE_FLOATS, mode_tag);
+                    count_step(writes);
+                    request(base + 3 * PT);
+                    const int next = writes;
+                    writes = reads;
+                    reads = waits;
+                    waits = next;
+                    uses += waits == 0 ? 1 : 0;
                 }
             };
             if (a.image != nullptr)

@@ -233,9 +233,9 @@ int bitsknn_fused_l2_topk_f32(const float* queries_dim_major, const float* point
  * pieces again.  With bitsknn_fused_image_bytes(dim, n) more bytes in the workspace, behind the
  * partial lists rounded up to a multiple of 256 bytes (and the workspace 16-byte aligned), a launch
  * of its own writes the stages of the whole point matrix there once per call and the fused kernel
- * copies them (65536 queries x 2^20 points, d = 32, k = 32: a quarter of the kernel's time).  It is
- * written from 4096 queries on (bitsknn_fused_tuning::image overrides that); the results are the
- * same bit for bit with and without it.  bitsknn_fused_image_bytes is 0 where no image is used
+ * copies them (65536 queries x 2^20 points, k = 32: d = 8 7.4 -> 7.1 ms, d = 16 9.9 -> 9.6 ms).  It is
+ * written from 4096 queries on in up to 16 dimensions (bitsknn_fused_tuning::image overrides that);
+ * the results are the same bit for bit with and without it.  bitsknn_fused_image_bytes is 0 where no image is used
  * (dim > 64, or an image of 2 GiB and more).
  * Errors as for bitsknn_fused_l2_topk_f32.
  */
@@ -299,7 +299,7 @@ int bitsknn_fused_l2_topk_f32_ex(const float* queries_dim_major, const float* po
  *   image         whether the points are cut into the stages of BITSKNN_FUSED_EXACT once, into the
  *                 workspace behind the partial lists (bitsknn_fused_image_bytes), instead of by
  *                 every workgroup again: 1 = whenever the workspace has room, -1 = never, 0 = the
- *                 library's choice (from 4096 queries on)
+ *                 library's choice (from 4096 queries on, up to 16 dimensions)
  * tuning == NULL: the library's choices.  Results do not depend on the tuning (for
  * BITSKNN_FUSED_EXACT bit for bit; for the other arithmetics the distances of a point can differ in
  * the last bit between one range and several).  bitsknn/tuning.py sweeps these and records the

@@ -14,13 +14,37 @@ What a wave does, as in the kernel:
 A count is the number of waves that have written their part, added up over the uses of a slot, as in
 LDS.  The model also runs two variants that must fail, to show that the check can tell: a ring of
 two slots, and the write placed before the wait.
+
+The kernels of the default arithmetic write two stages ahead, at the end of an iteration, so that a
+wave may run a whole iteration ahead of the slowest one of its workgroup (`late=True` below):
+
+    write its part of stage 0, count step 0
+    wait for step 0, write its part of stage 1, count step 1
+    for i = 0, 1, ...:
+        read stage i (the multiply, the candidates)
+        wait until all waves have counted step i + 1            (all have finished iteration i - 1)
+        write its part of stage i + 2 (slot (i + 2) % 3; past the last stage a write nobody reads)
+        count step i + 2                                         (counter (i + 2) % 3)
 """
 import pytest
 
 SLOTS = 3
 
 
-def wave_program(stages, write_before_wait=False):
+def late_program(stages, write_before_wait=False):
+    """steps k = 0, 1, ...: step k writes stage k; ("wait", k) / ("count", k) name steps here"""
+    program = [("write", 0), ("count", 0), ("wait", 0), ("write", 1), ("count", 1)]
+    for i in range(stages):
+        steps = [("wait", i + 1), ("write", i + 2), ("count", i + 2)]
+        if write_before_wait:
+            steps = [steps[1], steps[0], steps[2]]
+        program += [("read", i)] + steps
+    return program
+
+
+def wave_program(stages, write_before_wait=False, late=False):
+    if late:
+        return late_program(stages, write_before_wait)
     program = [("write", 0), ("count", 0)]
     for i in range(stages):
         steps = [("wait", i)]
@@ -32,12 +56,14 @@ def wave_program(stages, write_before_wait=False):
     return program
 
 
-def explore(waves, stages, slots=SLOTS, write_before_wait=False):
+def explore(waves, stages, slots=SLOTS, write_before_wait=False, late=False):
     """Breadth-first search over all interleavings.  A wave's program is a list of steps; the state
     is the tuple of program counters (everything else follows from them).  Returns the set of
     reachable states, or raises AssertionError with the offending state."""
-    program = wave_program(stages, write_before_wait)
+    program = wave_program(stages, write_before_wait, late)
     length = len(program)
+    # (the late protocol also writes the two stages past the last one, which nobody reads)
+    counts = stages + 2 if late else stages
 
     def counted(pcs, stage):
         """waves that have counted in for `stage`"""
@@ -66,7 +92,7 @@ def explore(waves, stages, slots=SLOTS, write_before_wait=False):
                 if kind == "wait":
                     # the counter of the slot holds the counts of all its uses so far
                     slot = stage % slots
-                    total = sum(counted(pcs, s) for s in range(stages) if s % slots == slot)
+                    total = sum(counted(pcs, s) for s in range(counts) if s % slots == slot)
                     if total < waves * (stage // slots + 1):
                         continue  # this wave cannot move now
                 elif kind == "write":
@@ -77,7 +103,7 @@ def explore(waves, stages, slots=SLOTS, write_before_wait=False):
                     assert written(pcs, stage), ("reads an incomplete stage", pcs, w, stage)
                     # and no wave has started to overwrite it
                     later = stage + slots
-                    if later < stages:
+                    if later < counts:
                         at = program.index(("write", later))
                         assert all(p <= at for p in pcs), ("reads a stage being overwritten", pcs, w, stage)
                 moved = True
@@ -120,3 +146,37 @@ def test_the_check_catches_a_ring_that_is_too_short():
 def test_the_check_catches_a_write_before_the_wait():
     with pytest.raises(AssertionError, match="being read|being overwritten"):
         explore(3, 6, write_before_wait=True)
+
+
+# ---- the protocol of the default arithmetic: two stages ahead, written at the end of an iteration
+
+@pytest.mark.parametrize("waves,stages", [(2, 9), (3, 6), (4, 4)])
+def test_late_writes_every_interleaving_is_safe_and_finishes(waves, stages):
+    assert len(explore(waves, stages, late=True)) > stages
+
+
+@pytest.mark.parametrize("stages", [1, 2, 3])
+def test_late_writes_short_runs(stages):
+    assert len(explore(4, stages, late=True)) > 0
+
+
+def test_late_writes_let_a_wave_run_an_iteration_ahead():
+    # one wave may have read stage i + 1 completely and be at the end of that iteration while another
+    # has only just started to read stage i; it never starts to read stage i + 2 before the other is
+    # done with stage i
+    stages = 6
+    program = wave_program(stages, late=True)
+    read_at = {s: program.index(("read", s)) for s in range(stages)}
+    states = explore(2, stages, late=True)
+    assert any(a > read_at[3] and b <= read_at[2] for a, b in states)
+    assert not any(a > read_at[4] and b <= read_at[2] for a, b in states)
+
+
+def test_late_writes_the_check_catches_a_ring_that_is_too_short():
+    with pytest.raises(AssertionError, match="being read|being overwritten"):
+        explore(3, 6, slots=2, late=True)
+
+
+def test_late_writes_the_check_catches_a_write_before_the_wait():
+    with pytest.raises(AssertionError, match="being read|being overwritten"):
+        explore(3, 6, write_before_wait=True, late=True)
