@@ -167,7 +167,8 @@ def test_fused_launch_parameters_from_the_environment(golden):
     rec = next(r for r in golden if r["family"] == "fused" and (r["n"], r["q"], r["d"], r["k"]) == (131072, 8192, 8, 64))
     args = ("-a", "fused-cache", "-n", "128k", "-q", "8k", "-d", "8", "-k", "64", "--seed", "24",
             "--items-per-thread", "8,4,2", "--block-size", "1", "--deg", "1")
-    for tuning in ("ranges=1,first_radius=-1", "ranges=16,first_radius=64", "ranges=0,first_radius=0"):
+    for tuning in ("ranges=1,first_radius=-1", "ranges=16,first_radius=64", "ranges=0,first_radius=0",
+                   "ranges=4,first_radius=0,image=1", "ranges=0,first_radius=0,image=-1"):
         p = run(*args, env=dict(os.environ, BITSKNN_FUSED_TUNING=tuning))
         assert p.returncode == 0, p.stderr
         assert str(checksums(p)[0]) in rec["checksums"], (tuning, checksums(p))
@@ -176,6 +177,8 @@ def test_fused_launch_parameters_from_the_environment(golden):
     assert p.returncode != 0 and "Unsupported queries_reg value: 3" in p.stderr
     p = run(*args, env=dict(os.environ, BITSKNN_FUSED_TUNING="ranges=99,first_radius=0"))
     assert p.returncode != 0 and "ranges must be" in p.stderr
+    p = run(*args, env=dict(os.environ, BITSKNN_FUSED_TUNING="ranges=0,first_radius=0,image=3"))
+    assert p.returncode != 0 and "image must be" in p.stderr
 
 
 @pytest.mark.gpu
