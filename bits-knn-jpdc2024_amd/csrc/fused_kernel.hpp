@@ -117,8 +117,9 @@ __device__ __forceinline__ void cut_bf16x2(const float (&x)[8], vuint4& p1, vuin
 //   accumulation in W    <= 17 * 2^-23 per matrix instruction, at most 13     (2.7e-5 S, allowing
 //                           for truncating adds of every term)
 // together below FILTER_REL = 2^-13 (1.22e-4) of S with a factor of 1.5 to spare.  The norm pieces
-// hold at most N (1 - NORM_LOWER) (1 + 2^-15.3) (cutting, the order of the staging threads' sums, one
-// rounding), and NORM_LOWER = 2^-12 + 2^-14 >= 2 FILTER_REL + 2^-15.3, so that
+// (one share per group of 8 dimensions, each lowered and cut by itself and added up by the matrix
+// instruction of the norm cell) hold at most N (1 - NORM_LOWER) (1 + 2^-15.3) (cutting, the sums of
+// a share, one rounding), and NORM_LOWER = 2^-12 + 2^-14 >= 2 FILTER_REL + 2^-15.3, so that
 //   W <= V + FILTER_REL * Q        whenever V is finite,
 // and a pair can only have V < radius if W < radius + FILTER_REL * Q.  The compare is written so
 // that a NaN in W passes; FILTER_ABS covers products of pieces that underflow.
