@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only LEG,...] [--skip LEG,...]
                     [--k 32] [--block-size 256] [--items-per-thread 8] [--prefetch]
-                    [--fused-d D] [--fused-k K] [--no-verify]
+                    [--fused-d D] [--fused-k K] [--fused-workspace-only] [--no-verify]
 
 A step is one bits top-k pass (through the C ABI) over a resident 1024 x 1,048,576 fp32 matrix
 of i.i.d. uniform [0,1) values (4 GiB, generated on the device).  The printed JSON line follows
@@ -390,7 +390,7 @@ def fused_roofline(q, n, d, seconds):
 
 
 def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=65536, n=1 << 20, long_ks=(),
-              workspace=False):
+              workspace=False, plain_too=True):
     """Config 5: bits-fused at d x k in the default arithmetic (the reference's, behind a filter on
     the bf16 matrix instructions) through the workspace entry point, as the knn driver calls it: the
     workspace has room for the stage image, so the points are cut into bf16 pieces once per call
@@ -417,7 +417,7 @@ def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=6553
             space = torch.empty(max(1, (lists + 255) // 256 * 256 + bitsknn.fused_image_bytes(d, n)),
                                 dtype=torch.uint8, device=dev)
             plain_s = None
-            if not workspace:
+            if not workspace and plain_too:
                 _, plain_s = timer.run(lambda: bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d,
                                                                      out_label=out_l), steps, 2)
                 out_d.fill_(-1.0)
@@ -451,8 +451,9 @@ def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=6553
                                            "workspace (one launch that cuts the points, one fused launch)",
                             "launches_timed": steps,
                             "queries_per_s": q / seconds, "ms": seconds * 1e3, "pairs_per_s": q * n / seconds,
-                            "ms_plain_entry_point": plain_s * 1e3,
                             "roofline": roof}
+                if plain_s is not None:
+                    headline["ms_plain_entry_point"] = plain_s * 1e3
                 if check:
                     headline["verified"] = entry["verified"]
                 for name, arithmetic, text, flops_per_pair, peak in (
@@ -609,6 +610,8 @@ def main():
     ap.add_argument("--skip", default="", help="comma-separated legs to leave out")
     ap.add_argument("--fused-d", type=int, default=0, help="restrict the fused grid to this dimension")
     ap.add_argument("--fused-k", type=int, default=0, help="restrict the fused grid to this list length")
+    ap.add_argument("--fused-workspace-only", action="store_true",
+                    help="time the fused grid through the workspace entry point only (counter passes)")
     ap.add_argument("--no-verify", action="store_true", help="leave out the comparison with the oracle")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -684,7 +687,8 @@ def main():
         ks = (args.fused_k,) if args.fused_k else (4, 16, 32)
         whole = not args.fused_d and not args.fused_k
         result["fused"] = leg_fused(bitsknn, torch, timer, oracle, dev, max(5, args.steps // 4), check, dims, ks,
-                                    long_ks=(64, 128, 256) if whole else ())
+                                    long_ks=(64, 128, 256) if whole else (),
+                                    plain_too=not args.fused_workspace_only)
         if whole:
             # the reference's own fused shape with few queries (its plots: 8192 queries, 2^17 points):
             # the entry point with a workspace, which cuts the points into ranges
