@@ -43,7 +43,7 @@ EXPORTS = (
 class FusedTuning(ctypes.Structure):
     """bitsknn_fused_tuning of include/bitsknn.h"""
     _fields_ = [("ranges", ctypes.c_int32), ("first_radius", ctypes.c_int32), ("image", ctypes.c_int32),
-                ("reserved", ctypes.c_int32 * 5)]
+                ("workgroup", ctypes.c_int32), ("reserved", ctypes.c_int32 * 4)]
 
 
 class BitsKnnError(RuntimeError):
@@ -280,7 +280,7 @@ def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1,
     scratch memory and allocates nothing; or a uint8 device tensor.
     arithmetic: None -> the plain entry points (FUSED_EXACT); FUSED_FP32 / FUSED_BF16X3 /
     FUSED_EXACT -> bitsknn_fused_l2_topk_f32_ex with that arithmetic.
-    tuning: None, or (ranges, first_radius[, image]) -> bitsknn_fused_l2_topk_f32_tuned."""
+    tuning: None, or (ranges, first_radius[, image[, workgroup]]) -> bitsknn_fused_l2_topk_f32_tuned."""
     import torch
     d, q = queries_dm.shape
     d2, n = points_dm.shape
@@ -300,7 +300,7 @@ def fused_l2_topk(queries_dm, points_dm, k, params=(8, 4, 2), block_query_dim=1,
     if tuning is not None:
         assert not isinstance(workspace, str)
         knobs = FusedTuning(int(tuning[0]), int(tuning[1]), int(tuning[2]) if len(tuning) > 2 else 0,
-                            (ctypes.c_int32 * 5)())
+                            int(tuning[3]) if len(tuning) > 3 else 0, (ctypes.c_int32 * 4)())
         _check(lib().bitsknn_fused_l2_topk_f32_tuned(*head[:8], FUSED_EXACT if arithmetic is None else int(arithmetic),
                                                      ctypes.byref(knobs), _ptr(workspace),
                                                      workspace.numel() if workspace is not None else 0, _stream()))

@@ -150,6 +150,9 @@ constexpr int SAMPLE_MIN_K_RANGES = 64; // (k <= 32: the three extra launches co
 // reads, and there the vector instructions of the cutting hide behind the matrix instructions)
 constexpr int IMAGE_MIN_QUERIES = 4096;
 constexpr int IMAGE_MAX_DIM = 16;
+// fewest workgroups of 256 queries (times the ranges of points) that are launched as such: nearly
+// one for each of the 256 compute units
+constexpr int BIG_MIN_WORKGROUPS = 224;
 
 int first_radius_rank(int k, int scale)
 {
@@ -238,6 +241,12 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
                         "bitsknn_fused_tuning: image must be 0 (the library's choice), -1 (never) or 1 (whenever the "
                         "workspace has room for it), got %d",
                         tuning->image);
+        }
+        if (tuning->workgroup != 0 && tuning->workgroup != 128 && tuning->workgroup != 256)
+        {
+            return fail(BITSKNN_ERR_INVALID,
+                        "bitsknn_fused_tuning: workgroup must be 0 (the library's choice), 128 or 256 queries, got %d",
+                        tuning->workgroup);
         }
         for (const std::int32_t word : tuning->reserved)
         {
@@ -344,6 +353,16 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     a.split_points = ((n + splits - 1) / splits + 255) / 256 * 256;
     a.image = nullptr;
     a.image_bytes = 0;
+    // Workgroups of 256 queries (eight waves sharing stages of twice the points: half the staging,
+    // LDS writes and hand-overs per pair) where the kernel has them and they fill the chip: one per
+    // compute unit, ranges of points included.  65536 queries x 2^20 points, k = 32: d = 8 7.65 ->
+    // 6.40 ms, d = 16 10.1 -> 8.86 ms, d = 32 16.8 -> 14.3 ms (the stage image, which only the
+    // workgroups of 128 queries take, gives 7.10 / 9.82 / 17.2 ms).
+    const bool has_big = arithmetic == BITSKNN_FUSED_EXACT && dim <= 32 && k <= 32;
+    const long long big_workgroups = (static_cast<long long>(q) + 255) / 256 * splits;
+    const bool big = has_big && (tuning != nullptr && tuning->workgroup != 0 ? tuning->workgroup == 256
+                                                                              : big_workgroups >= BIG_MIN_WORKGROUPS);
+    a.workgroup = big ? 1 : 0;
 
     auto* hip_stream = static_cast<hipStream_t>(stream);
     const int split = arithmetic == BITSKNN_FUSED_BF16X3 ? FUSED_ARITH_BF16X3
@@ -360,7 +379,7 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     // The stage image: with room for it in the workspace behind the partial lists, the points are
     // cut into the stages of the exact arithmetic once, by a launch of their own, instead of by
     // every workgroup of the fused kernel again.  That pays from a few thousand queries on.
-    if (split == FUSED_ARITH_EXACT && use_workspace && workspace != nullptr && dim <= 64 &&
+    if (split == FUSED_ARITH_EXACT && use_workspace && workspace != nullptr && dim <= 64 && !big &&
         (tuning == nullptr || tuning->image >= 0))
     {
         const size_t image_bytes = fused_image_bytes(dim, n);

@@ -152,11 +152,19 @@ constexpr u32 BF16_HUGE = 0x7F7FU;
 constexpr int RING_MAX_DP = 128; // largest padded dimension that takes the ring of stages
 constexpr int FQ_XCHG = 96;      // words a wave has for the exchange at a merge: 32 radii, fills, labels
 
-template <int DP, int ARITH, int K, bool WIDE_OK = false>
+template <int DP, int ARITH, int K, bool WIDE_OK = false, bool BIG_OK = false>
 struct fused_geometry
 {
     static constexpr bool SPLIT = ARITH == FUSED_ARITH_BF16X3;
     static constexpr bool EXACT = ARITH == FUSED_ARITH_EXACT;
+    // BIG: workgroups of eight waves (256 queries) that share stages of twice the points, one
+    // workgroup per compute unit -- the same two waves per SIMD, but half the staging, LDS writes
+    // and hand-overs per pair.  The exact arithmetic in 32 dimensions on the ring of stages; worth
+    // it where the queries alone give every compute unit such a workgroup (launch_fused).
+    static constexpr bool BIG = BIG_OK && ARITH == FUSED_ARITH_EXACT && DP <= 32 && K <= FQ_CAP;
+    static constexpr int WAVES = BIG ? 2 * FQ_WAVES : FQ_WAVES;
+    static constexpr int THREADS = WAVES * WAVE;
+    static constexpr int QB = FQ_QW * WAVES; // queries per workgroup
     static constexpr bool WIDE = WIDE_OK && K >= 128 && DP <= 16 && ARITH == FUSED_ARITH_MFMA_F32;
     static constexpr int CAP = WIDE ? 2 * FQ_CAP : FQ_CAP; // buffer slots per query
     static constexpr int DK = DP < 16 ? 16 : DP;       // SPLIT, EXACT: dimensions padded to whole matrix steps
@@ -169,7 +177,7 @@ struct fused_geometry
     // 16 matrix dimensions.
     static constexpr int CELLS = EXACT ? (DP <= 8 ? 3 : 2 * KS + 1) : 0;
     static constexpr int PT = SPLIT   ? (DK <= 16 ? 128 : (DK <= 32 ? 64 : 32))
-                              : EXACT ? (DP <= 16 ? 128 : (DP <= 32 ? 64 : 32))
+                              : EXACT ? (DP <= 16 ? 128 : (DP <= 32 ? 64 : 32)) * (BIG ? 2 : 1)
                               : WIDE  ? (DP <= 8 ? 128 : 64)
                                       : (DP <= 16 ? 256 : (DP <= 32 ? 128 : (DP <= 64 ? 64 : 32)));
     // threads per point when staging.  The small stages of the 64-slot geometry are staged by their
@@ -177,8 +185,8 @@ struct fused_geometry
     // initial accumulator as in the 32-slot geometry (same terms in the same order: both
     // geometries give the same bits).  EXACT: a thread carries 8 consecutive dimensions of a point
     // (4 in up to 8 dimensions), as with bf16x3 products.
-    static constexpr int TPP = EXACT ? FQ_THREADS / PT : (WIDE ? 1 : FQ_THREADS / PT);
-    static constexpr int STAGERS = SPLIT ? FQ_THREADS : TPP * PT; // threads that stage
+    static constexpr int TPP = EXACT ? THREADS / PT : (WIDE ? 1 : THREADS / PT);
+    static constexpr int STAGERS = SPLIT ? THREADS : TPP * PT; // threads that stage
     // point rows (zero beyond dim), then one row per staging thread of a point with its share of
     // ||p||^2 (at least two rows, so that the row count is even)
     // (one row where it is read as the initial accumulator and never multiplied)
@@ -192,7 +200,10 @@ struct fused_geometry
     static constexpr int ROWS = DP + NORM_ROWS;
     static constexpr int STEPS = ROWS / 2;    // MFMA steps of 2 rows
     static constexpr int VPT = SPLIT ? 8 : DP / TPP; // values a thread carries from global memory to LDS
-    static constexpr int MT = PT / 32;        // MFMA row tiles per stage
+    // MFMA row tiles per stage; the exact arithmetic takes the stages of 256 points in two passes
+    // of four tiles
+    static constexpr int MT = EXACT && PT > 128 ? 4 : PT / 32;
+    static constexpr int SUB = PT / 32 / MT;
     static constexpr int STAGE_FLOATS = SPLIT   ? 3 * KS * PT * 4 + PT
                                         : EXACT ? DP * PT + CELLS * PT * 4
                                                 : ROWS * PT;
@@ -223,26 +234,34 @@ struct fused_geometry
         !WIDE && (SPLIT ? K <= FQ_CAP
                         : (DP <= 8 && K <= 128) || (DP >= 16 && DP <= RING_MAX_DP && K <= FQ_CAP));
     static constexpr int NB = RING ? 3 : 2;
-    static constexpr int SLOTS = EXACT && K <= 16 ? 16 : RING && !SPLIT && DP >= 16 ? 24 : CAP; // slots a query buffer has in LDS
+    // slots a query buffer has in LDS (20 where the three stages of 256 points in 16 dimensions leave
+    // no more room next to the buffers of 256 queries)
+    static constexpr int SLOTS = EXACT && K <= 16 ? 16
+                                 : BIG && DP == 16 ? 20
+                                 : RING && !SPLIT && DP >= 16 ? 24
+                                                              : CAP;
     static_assert(!SPLIT || (DP <= 64 && TPP == KS), "one staging thread per point and cell");
-    static_assert(!EXACT || (DP <= 64 && VPT == (DP <= 8 ? 4 : 8) && PT <= 128),
-                  "the stages of the exact arithmetic serve up to 64 dimensions, in at most four tiles");
+    static_assert(!EXACT || (DP <= 64 && VPT == (DP <= 8 ? 4 : 8) && MT <= 4 && SUB <= 2),
+                  "the stages of the exact arithmetic serve up to 64 dimensions, in passes of at most four tiles");
     static constexpr size_t lds_bytes()
     {
         // the stages, the query buffers, exchange slots, merge flags and stage counters
         return NB * static_cast<size_t>(STAGE_FLOATS) * sizeof(float) +
-               static_cast<size_t>(FQ_WAVES) * FQ_QW * SLOTS * sizeof(u64) +
-               static_cast<size_t>(FQ_WAVES) * FQ_XCHG * sizeof(float) + 8 * sizeof(int);
+               static_cast<size_t>(WAVES) * FQ_QW * SLOTS * sizeof(u64) +
+               static_cast<size_t>(WAVES) * FQ_XCHG * sizeof(float) + 8 * sizeof(int);
     }
-    static_assert(!EXACT || lds_bytes() <= 80 * 1024, "two workgroups per compute unit");
+    static_assert(!EXACT || lds_bytes() <= (BIG ? 160 : 80) * 1024, "two workgroups per compute unit, or one of eight waves");
 };
 
 // K: list length.  DP: dimension padded to 8, 16, 32, 64, 128 or 256 (padding rows are zero on
 // both sides of the product).
-template <int K, int DP, int ARITH, bool WIDE_OK>
-__global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
+template <int K, int DP, int ARITH, bool WIDE_OK, bool BIG_OK = false>
+__global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>::THREADS)) fused_kernel(const fused_args a)
 {
-    using G = fused_geometry<DP, ARITH, K, WIDE_OK>;
+    using G = fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>;
+    constexpr int FQ_THREADS = G::THREADS; // (the workgroup's shape, which shadows the usual one)
+    constexpr int FQ_WAVES = G::WAVES;
+    constexpr int FQ_QB = G::QB;
     constexpr bool SPLIT = G::SPLIT;
     constexpr bool EXACT = G::EXACT;
     constexpr int PT = G::PT;
@@ -1082,28 +1101,21 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     u32 cut1[4] = {0, 0, 0, 0};
     u32 cut2[4] = {0, 0, 0, 0};
     u32 cut_norm = 0;
-    auto filter_values_and_cut = [&](const float* stage, vfloat16 (&w)[MT], int cut_base, auto mode_tag) __attribute__((always_inline)) {
-        constexpr int MODE = decltype(mode_tag)::value;
-        // (the cells are read in the order in which the matrix instructions take them, the norm
-        // cell last, so that the first instruction waits for the first read only)
+    constexpr int NCELL = DP <= 8 ? 2 : 2 * KB + 1; // cells of a point that a lane reads
+    // the tiles of a stage are multiplied in groups whose cells fit into 48 registers
+    constexpr int TG = MT * NCELL > 12 ? 2 : MT;
+    // (the cells are read in the order in which the matrix instructions take them, the norm cell
+    // last, so that the first instruction waits for the first read only)
+    auto read_cells = [&](const float* stage, vuint4 (&cell)[TG][NCELL], int first_tile) __attribute__((always_inline)) {
         const vuint4* const cells = reinterpret_cast<const vuint4*>(stage + DP * PT);
-        vfloat16 zero;
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-        {
-            zero[r] = 0.0F;
-        }
-        constexpr int TERMS = DP <= 8 ? 2 : 3 * KB + 1;
-        constexpr int NCELL = DP <= 8 ? 2 : 2 * KB + 1;
-        vuint4 cell[MT][NCELL];
-        const vuint4* const mine = cells + ql;
+        const vuint4* const mine = cells + 32 * first_tile + ql;
         if constexpr (DP <= 8)
         {
 #pragma unroll
             for (int c = 0; c < 2; ++c)
             {
 #pragma unroll
-                for (int t = 0; t < MT; ++t)
+                for (int t = 0; t < TG; ++t)
                 {
                     cell[t][c] = mine[32 * t + (half != 0 ? 1 + c : 0) * PT];
                 }
@@ -1115,23 +1127,34 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
             for (int kb = 0; kb < KB; ++kb)
             {
 #pragma unroll
-                for (int t = 0; t < MT; ++t)
+                for (int t = 0; t < TG; ++t)
                 {
                     cell[t][KB + kb] = mine[32 * t + (KS + 2 * kb + half) * PT];
                 }
 #pragma unroll
-                for (int t = 0; t < MT; ++t)
+                for (int t = 0; t < TG; ++t)
                 {
                     cell[t][kb] = mine[32 * t + (2 * kb + half) * PT];
                 }
             }
 #pragma unroll
-            for (int t = 0; t < MT; ++t)
+            for (int t = 0; t < TG; ++t)
             {
                 cell[t][2 * KB] = mine[32 * t + 2 * KS * PT];
             }
         }
-        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto filter_values_and_cut = [&](const float* stage, vfloat16 (&w)[MT], int cut_base, auto mode_tag, auto sub_tag) __attribute__((always_inline)) {
+        // (sub: which MT tiles of the stage; the cutting goes with the first ones)
+        constexpr int SUB_PASS = decltype(sub_tag)::value;
+        constexpr int MODE = SUB_PASS == 0 ? decltype(mode_tag)::value : 2;
+        vfloat16 zero;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+        {
+            zero[r] = 0.0F;
+        }
+        constexpr int TERMS = DP <= 8 ? 2 : 3 * KB + 1;
         constexpr int PAIRS_OF_VALUES = VPT / 2;
         constexpr int CHUNKS = MODE == 2 ? 0 : PAIRS_OF_VALUES + 1;
         static_assert(!EXACT || CHUNKS <= MT * TERMS, "a piece of the cutting per matrix instruction");
@@ -1164,25 +1187,32 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 cut_norm = cut_base + sp < n ? first | (second << 16U) : BF16_HUGE;
             }
         };
-        static_for<0, TERMS>([&](auto j_tag) {
-            constexpr int j = decltype(j_tag)::value;
-            constexpr bool norm_term = DP > 8 && j == 3 * KB;
-            constexpr int kb = DP <= 8 || norm_term ? 0 : j / 3;
-            constexpr int which = DP <= 8 ? j : j % 3;
-            constexpr int a_at = DP <= 8 ? j : (norm_term ? 2 * KB : (which == 0 ? KB + kb : kb));
-            constexpr int b_piece = DP <= 8 ? j : (norm_term ? 2 : (which == 1 ? 1 : 0));
-            constexpr int b_kb = kb;
-            static_for<0, MT>([&](auto t_tag) {
-                constexpr int t = decltype(t_tag)::value;
-                constexpr int m = j * MT + t; // number of this matrix instruction
-                w[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                    __builtin_bit_cast(vbf16x8, cell[t][a_at]), __builtin_bit_cast(vbf16x8, qs[b_piece][b_kb]),
-                    j == 0 ? zero : w[t], 0, 0, 0);
-                if constexpr (m < CHUNKS)
-                {
-                    chunk(std::integral_constant<int, m>{});
-                }
-                __builtin_amdgcn_sched_barrier(0);
+        static_for<0, MT / TG>([&](auto g_tag) {
+            constexpr int g = decltype(g_tag)::value;
+            vuint4 cell[TG][NCELL];
+            read_cells(stage, cell, SUB_PASS * MT + g * TG);
+            __builtin_amdgcn_sched_barrier(0);
+            static_for<0, TERMS>([&](auto j_tag) {
+                constexpr int j = decltype(j_tag)::value;
+                constexpr bool norm_term = DP > 8 && j == 3 * KB;
+                constexpr int kb = DP <= 8 || norm_term ? 0 : j / 3;
+                constexpr int which = DP <= 8 ? j : j % 3;
+                constexpr int a_at = DP <= 8 ? j : (norm_term ? 2 * KB : (which == 0 ? KB + kb : kb));
+                constexpr int b_piece = DP <= 8 ? j : (norm_term ? 2 : (which == 1 ? 1 : 0));
+                constexpr int b_kb = kb;
+                static_for<0, TG>([&](auto t_tag) {
+                    constexpr int tt = decltype(t_tag)::value;
+                    constexpr int t = g * TG + tt;
+                    constexpr int m = (g * TERMS + j) * TG + tt; // number of this matrix instruction
+                    w[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(vbf16x8, cell[tt][a_at]), __builtin_bit_cast(vbf16x8, qs[b_piece][b_kb]),
+                        j == 0 ? zero : w[t], 0, 0, 0);
+                    if constexpr (m < CHUNKS)
+                    {
+                        chunk(std::integral_constant<int, m>{});
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                });
             });
         });
     };
@@ -1667,11 +1697,14 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
                 {
                     BITSKNN_FT_LAP(0);
                     const float* const stage = stages + reads * STAGE_FLOATS;
-                    vfloat16 w[MT];
-                    __builtin_amdgcn_sched_barrier(0);
-                    filter_values_and_cut(stage, w, base + 2 * PT, mode_tag);
-                    BITSKNN_FT_LAP(2);
-                    filter_and_append(w, stage, base);
+                    static_for<0, G::SUB>([&](auto sub_tag) {
+                        constexpr int sub = decltype(sub_tag)::value;
+                        vfloat16 w[MT];
+                        __builtin_amdgcn_sched_barrier(0);
+                        filter_values_and_cut(stage, w, base + 2 * PT, mode_tag, sub_tag);
+                        BITSKNN_FT_LAP(2);
+                        filter_and_append(w, stage + 32 * MT * sub, base + 32 * MT * sub);
+                    });
                     wait_for(waits, uses);
                     BITSKNN_FT_LAP(1);
                     write_cut(stages + writes * STAGE_FLOATS, mode_tag);
@@ -1757,15 +1790,15 @@ __global__ void __launch_bounds__(FQ_THREADS) fused_kernel(const fused_args a)
     }
 }
 
-template <int K, int DP, int ARITH, bool WIDE_OK>
+template <int K, int DP, int ARITH, bool WIDE_OK, bool BIG_OK = false>
 hipError_t launch_fused_as(const fused_args& a, hipStream_t stream)
 {
-    using G = fused_geometry<DP, ARITH, K, WIDE_OK>;
+    using G = fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>;
     constexpr size_t lds_bytes = G::lds_bytes();
     if (lds_bytes > 48 * 1024)
     {
         const hipError_t status =
-            hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<K, DP, ARITH, WIDE_OK>),
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_kernel<K, DP, ARITH, WIDE_OK, BIG_OK>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
         if (status != hipSuccess)
         {
@@ -1781,9 +1814,9 @@ hipError_t launch_fused_as(const fused_args& a, hipStream_t stream)
         args.sample_offset = a.sample_scale / 2 * PT;
         args.split_points = (args.visit + 255) / 256 * 256;
     }
-    const unsigned grid = static_cast<unsigned>((a.q + FQ_QB - 1) / FQ_QB);
-    hipLaunchKernelGGL((fused_kernel<K, DP, ARITH, WIDE_OK>), dim3(grid, static_cast<unsigned>(a.splits)),
-                       dim3(FQ_THREADS), lds_bytes, stream, args);
+    const unsigned grid = static_cast<unsigned>((a.q + G::QB - 1) / G::QB);
+    hipLaunchKernelGGL((fused_kernel<K, DP, ARITH, WIDE_OK, BIG_OK>), dim3(grid, static_cast<unsigned>(a.splits)),
+                       dim3(G::THREADS), lds_bytes, stream, args);
     return hipGetLastError();
 }
 
@@ -1800,6 +1833,15 @@ hipError_t launch_fused(const fused_args& a, hipStream_t stream)
         if (a.splits > 1)
         {
             return launch_fused_as<K, DP, ARITH, true>(a, stream);
+        }
+    }
+    // Workgroups of 256 queries where the caller of the launch chose them and the geometry has them
+    // (no stage image: its stages are those of the workgroups of 128 queries)
+    if constexpr (fused_geometry<DP, ARITH, K, false, true>::BIG)
+    {
+        if (a.workgroup > 0 && a.image == nullptr)
+        {
+            return launch_fused_as<K, DP, ARITH, false, true>(a, stream);
         }
     }
     return launch_fused_as<K, DP, ARITH, false>(a, stream);

@@ -300,6 +300,11 @@ int bitsknn_fused_l2_topk_f32_ex(const float* queries_dim_major, const float* po
  *                 workspace behind the partial lists (bitsknn_fused_image_bytes), instead of by
  *                 every workgroup again: 1 = whenever the workspace has room, -1 = never, 0 = the
  *                 library's choice (from 4096 queries on, up to 16 dimensions)
+ *   workgroup     queries per workgroup where the kernel comes in two shapes (BITSKNN_FUSED_EXACT up
+ *                 to 32 dimensions, lists of up to 32 entries): 128 (four waves), 256 (eight waves
+ *                 sharing stages of twice the points; no stage image then) or 0 = the library's
+ *                 choice (256 where ceil(q / 256) * ranges >= 224, nearly one such workgroup for
+ *                 every compute unit)
  * tuning == NULL: the library's choices.  Results do not depend on the tuning (for
  * BITSKNN_FUSED_EXACT bit for bit; for the other arithmetics the distances of a point can differ in
  * the last bit between one range and several).  bitsknn/tuning.py sweeps these and records the
@@ -311,7 +316,8 @@ typedef struct bitsknn_fused_tuning
     int32_t ranges;
     int32_t first_radius;
     int32_t image;
-    int32_t reserved[5];
+    int32_t workgroup;
+    int32_t reserved[4];
 } bitsknn_fused_tuning;
 int bitsknn_fused_l2_topk_f32_tuned(const float* queries_dim_major, const float* points_dim_major,
                                     int dim, int32_t q, int32_t n, float* out_dist, int32_t* out_label,

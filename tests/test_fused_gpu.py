@@ -36,24 +36,31 @@ def _fused(bk, dev, points, queries, k, params=(8, 4, 2), bqd=1, dim_mult=1, wor
         od, ol = bk.fused_l2_topk(qd, pd, k, workspace="image", tuning=(0, 0, 1))
         bk.fused_status()
         return od.cpu().numpy(), ol.cpu().numpy()
+    if arithmetic == "big":
+        # the default arithmetic in workgroups of 256 queries (forced: the library itself takes them
+        # where they fill the chip), ranges as the library chooses
+        od, ol = bk.fused_l2_topk(qd, pd, k, workspace="auto", tuning=(0, 0, 0, 256))
+        bk.fused_status()
+        return od.cpu().numpy(), ol.cpu().numpy()
     od, ol = bk.fused_l2_topk(qd, pd, k, params, bqd, dim_mult, workspace=workspace, arithmetic=arithmetic)
     bk.fused_status()  # synchronises; raises if a wave gave up a wait for a stage
     return od.cpu().numpy(), ol.cpu().numpy()
 
 
 MODES = ["default", "mfma"]
-MODES_AND_IMAGE = ["default", "mfma", "image"]
+MODES_AND_IMAGE = ["default", "mfma", "image", "big"]
 
 
 def _arith(bk, mode):
     """C-ABI arithmetic of a test mode: None = the plain entry points; "image" = the default
-    arithmetic through bitsknn_fused_l2_topk_f32_tuned with the stage image (see _fused)"""
-    return {"default": None, "mfma": bk.FUSED_FP32, "bf16x3": bk.FUSED_BF16X3, "image": "image"}[mode]
+    arithmetic through bitsknn_fused_l2_topk_f32_tuned with the stage image, "big" = the same in
+    workgroups of 256 queries (see _fused)"""
+    return {"default": None, "mfma": bk.FUSED_FP32, "bf16x3": bk.FUSED_BF16X3, "image": "image", "big": "big"}[mode]
 
 
 def _bits(mode, dim):
     """whether the result of this mode must equal the oracle's bit for bit"""
-    return mode in ("default", "image") and dim <= 64
+    return mode in ("default", "image", "big") and dim <= 64
 
 
 def _check(oracle, points, queries, k, gd, gl, min_recall=0.999, bar_dim=None, bits=False):
@@ -142,7 +149,7 @@ def test_ragged_counts(bk, dev, oracle, n, q, mode):
 # points per stage by padded dimension.  fp32 matrix instructions: 256 up to 16 dimensions, 128 / 64
 # / 32 for 32 / 64 / 128; the exact arithmetic and bf16x3: 128 up to 16 dimensions, 64 / 32 for 32 / 64
 @pytest.mark.parametrize("d", [8, 16, 32, 64, 100])
-@pytest.mark.parametrize("mode", ["default", "mfma", "bf16x3", "image"])
+@pytest.mark.parametrize("mode", ["default", "mfma", "bf16x3", "image", "big"])
 def test_point_counts_around_whole_stages(bk, dev, oracle, d, mode):
     # one to five stages, each count one short of, at and one past a whole stage: the ring of three
     # stage buffers starts, wraps around and ends at every position
@@ -150,7 +157,11 @@ def test_point_counts_around_whole_stages(bk, dev, oracle, d, mode):
         pytest.skip("bf16x3 products serve 9 to 64 dimensions")
     if mode == "image" and d > 64:
         pytest.skip("the stage image serves up to 64 dimensions")
-    if mode == "mfma" or d > 64:
+    if mode == "big" and d > 32:
+        pytest.skip("workgroups of 256 queries serve up to 32 dimensions")
+    if mode == "big":
+        stage = {8: 256, 16: 256, 32: 128}[d]
+    elif mode == "mfma" or d > 64:
         stage = {8: 256, 16: 256, 32: 128, 64: 64, 100: 32}[d]
     else:
         stage = {8: 128, 16: 128, 32: 64, 64: 32}[d]
@@ -289,9 +300,11 @@ def test_the_filter_never_drops_a_neighbour(bk, dev, oracle, d, kind):
     if kind in ("signs", "near"):
         wd, wl = _fused(bk, dev, p, s, k, workspace="auto")
         assert np.array_equal(gd, wd) and np.array_equal(gl, wl)
-    # the same through the stage image (the launch that writes it cuts the points the same way)
-    wd, wl = _fused(bk, dev, p, s, k, arithmetic="image")
-    assert np.array_equal(gd.view(np.uint32), wd.view(np.uint32)) and np.array_equal(gl, wl)
+    # the same through the stage image (the launch that writes it cuts the points the same way) and in
+    # workgroups of 256 queries
+    for other in ("image", "big"):
+        wd, wl = _fused(bk, dev, p, s, k, arithmetic=other)
+        assert np.array_equal(gd.view(np.uint32), wd.view(np.uint32)) and np.array_equal(gl, wl), other
 
 
 # reference-held checksums of the fused runs (data/fused-*.err), query 0
@@ -595,7 +608,8 @@ def test_tuned_entry_point(bk, dev, oracle):
     bk.fused_status()
     assert np.array_equal(ol.cpu().numpy(), el)
     for bad, message in (((65, 0), "ranges must be"), ((-1, 0), "ranges must be"), ((0, 1), "first_radius must be"),
-                         ((0, -2), "first_radius must be"), ((0, 5000), "first_radius must be")):
+                         ((0, -2), "first_radius must be"), ((0, 5000), "first_radius must be"),
+                         ((0, 0, 0, 64), "workgroup must be")):
         with pytest.raises(bk.BitsKnnError, match=message):
             bk.fused_l2_topk(qd, pd, k, workspace=space, tuning=bad)
 
