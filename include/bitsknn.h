@@ -303,8 +303,9 @@ int bitsknn_fused_l2_topk_f32_ex(const float* queries_dim_major, const float* po
  *   workgroup     queries per workgroup where the kernel comes in two shapes (BITSKNN_FUSED_EXACT up
  *                 to 32 dimensions, lists of up to 32 entries): 128 (four waves), 256 (eight waves
  *                 sharing stages of twice the points; no stage image then) or 0 = the library's
- *                 choice (256 where ceil(q / 256) * ranges >= 224, nearly one such workgroup for
- *                 every compute unit)
+ *                 choice (256 where ceil(q / 256) * ranges workgroups, one at a time on each of
+ *                 the 256 compute units, leave at most an eighth of the units idle in their last
+ *                 round)
  * tuning == NULL: the library's choices.  Results do not depend on the tuning (for
  * BITSKNN_FUSED_EXACT bit for bit; for the other arithmetics the distances of a point can differ in
  * the last bit between one range and several).  bitsknn/tuning.py sweeps these and records the
