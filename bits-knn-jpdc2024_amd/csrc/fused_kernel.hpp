@@ -161,7 +161,8 @@ struct fused_geometry
     // workgroup per compute unit -- the same two waves per SIMD, but half the staging, LDS writes
     // and hand-overs per pair.  The exact arithmetic in 32 dimensions on the ring of stages; worth
     // it where the queries alone give every compute unit such a workgroup (launch_fused).
-    static constexpr bool BIG = BIG_OK && ARITH == FUSED_ARITH_EXACT && DP <= 32 && K <= FQ_CAP;
+    static constexpr bool BIG =
+        BIG_OK && ARITH == FUSED_ARITH_EXACT && DP <= 32 && (K <= FQ_CAP || (DP <= 8 && K <= 128));
     static constexpr int WAVES = BIG ? 2 * FQ_WAVES : FQ_WAVES;
     static constexpr int THREADS = WAVES * WAVE;
     static constexpr int QB = FQ_QW * WAVES; // queries per workgroup
