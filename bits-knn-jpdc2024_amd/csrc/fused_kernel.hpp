@@ -162,7 +162,7 @@ struct fused_geometry
     // and hand-overs per pair.  The exact arithmetic in 32 dimensions on the ring of stages; worth
     // it where the queries alone give every compute unit such a workgroup (launch_fused).
     static constexpr bool BIG =
-        BIG_OK && ARITH == FUSED_ARITH_EXACT && DP <= 32 && (K <= FQ_CAP || (DP <= 8 && K <= 128));
+        BIG_OK && ARITH == FUSED_ARITH_EXACT && DP <= 64 && (K <= FQ_CAP || (DP <= 8 && K <= 128));
     static constexpr int WAVES = BIG ? 2 * FQ_WAVES : FQ_WAVES;
     static constexpr int THREADS = WAVES * WAVE;
     static constexpr int QB = FQ_QW * WAVES; // queries per workgroup
@@ -176,7 +176,10 @@ struct fused_geometry
     // instructions): two pieces per value and a cell with two pieces of the lowered norm.  Up to 8
     // dimensions a point is three cells, (piece 1 | piece 2 | norm), used as the two halves of the
     // 16 matrix dimensions.
-    static constexpr int CELLS = EXACT ? (DP <= 8 ? 3 : 2 * KS + 1) : 0;
+    // (one norm cell holds the shares of four groups of 8 dimensions: a second one where eight
+    // groups are staged by eight waves)
+    static constexpr int NORM_CELLS = DP == 64 && BIG_OK && ARITH == FUSED_ARITH_EXACT && K <= FQ_CAP ? 2 : 1;
+    static constexpr int CELLS = EXACT ? (DP <= 8 ? 3 : 2 * KS + NORM_CELLS) : 0;
     static constexpr int PT = SPLIT   ? (DK <= 16 ? 128 : (DK <= 32 ? 64 : 32))
                               : EXACT ? (DP <= 16 ? 128 : (DP <= 32 ? 64 : 32)) * (BIG ? 2 : 1)
                               : WIDE  ? (DP <= 8 ? 128 : 64)
@@ -741,7 +744,9 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
     const int sp = EXACT ? t % PT : (SPLIT || G::PAIRED ? t / TPP : t % PT);
     const int sd0 = EXACT ? VPT * (t / PT) : (SPLIT ? VPT * (t % TPP) : (G::PAIRED ? t % TPP : t / PT));
     // EXACT: the word of a point's norm cell that takes this thread's share of the norm
-    const int norm_slot = DP == 64 ? wave : t / PT;
+    // (64 dimensions in workgroups of four waves: the two groups of a wave share a word)
+    constexpr bool PAIRED_SHARES = DP == 64 && !G::BIG;
+    const int norm_slot = PAIRED_SHARES ? wave : t / PT;
     auto dim_of = [&](int i) -> int { return SPLIT || EXACT ? sd0 + i : sd0 + TPP * i; };
     float pre[VPT];
     // Point values are read with buffer loads: a constant byte offset per value and lane (beyond
@@ -886,7 +891,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
                 halves[2 * sp + h] = vuint2{piece[0][0], piece[0][1]};
                 halves[2 * (PIECE2 * PT + sp) + h] = vuint2{piece[1][0], piece[1][1]};
             }
-            if constexpr (DP == 64)
+            if constexpr (PAIRED_SHARES)
             {
                 // two groups of dimensions per wave: one share
                 share += __builtin_bit_cast(float, lane_xor32<32>(__builtin_bit_cast(u32, share)));
@@ -901,8 +906,9 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
                 const vfloat2 rest{lowered - __builtin_bit_cast(float, first << 16U), 0.0F};
                 const u32 second = __builtin_bit_cast(u32, __builtin_convertvector(rest, vbf16x2)) & 0xFFFFU;
                 u32* const norm_cell =
-                    reinterpret_cast<u32*>(reinterpret_cast<vuint4*>(stage + DP * PT) + (G::CELLS - 1) * PT + sp);
-                norm_cell[norm_slot] = base + sp < n ? first | (second << 16U) : BF16_HUGE;
+                    reinterpret_cast<u32*>(reinterpret_cast<vuint4*>(stage + DP * PT) +
+                                           (G::CELLS - G::NORM_CELLS + norm_slot / 4) * PT + sp);
+                norm_cell[norm_slot % 4] = base + sp < n ? first | (second << 16U) : BF16_HUGE;
             }
         }
         else if constexpr (SPLIT)
@@ -1106,9 +1112,9 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
     u32 cut1[4] = {0, 0, 0, 0};
     u32 cut2[4] = {0, 0, 0, 0};
     u32 cut_norm = 0;
-    constexpr int NCELL = DP <= 8 ? 2 : 2 * KB + 1; // cells of a point that a lane reads
+    constexpr int NCELL = DP <= 8 ? 2 : 2 * KB + G::NORM_CELLS; // cells of a point that a lane reads
     // the tiles of a stage are multiplied in groups whose cells fit into 48 registers
-    constexpr int TG = MT * NCELL > 12 ? 2 : MT;
+    constexpr int TG = MT * NCELL <= 12 ? MT : (2 * NCELL <= 12 ? 2 : 1);
     // (the cells are read in the order in which the matrix instructions take them, the norm cell
     // last, so that the first instruction waits for the first read only)
     auto read_cells = [&](const float* stage, vuint4 (&cell)[TG][NCELL], int first_tile) __attribute__((always_inline)) {
@@ -1143,9 +1149,13 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
                 }
             }
 #pragma unroll
-            for (int t = 0; t < TG; ++t)
+            for (int c = 0; c < G::NORM_CELLS; ++c)
             {
-                cell[t][2 * KB] = mine[32 * t + 2 * KS * PT];
+#pragma unroll
+                for (int t = 0; t < TG; ++t)
+                {
+                    cell[t][2 * KB + c] = mine[32 * t + (2 * KS + c) * PT];
+                }
             }
         }
     };
@@ -1159,7 +1169,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
         {
             zero[r] = 0.0F;
         }
-        constexpr int TERMS = DP <= 8 ? 2 : 3 * KB + 1;
+        constexpr int TERMS = DP <= 8 ? 2 : 3 * KB + G::NORM_CELLS;
         constexpr int PAIRS_OF_VALUES = VPT / 2;
         constexpr int CHUNKS = MODE == 2 ? 0 : PAIRS_OF_VALUES + 1;
         static_assert(!EXACT || CHUNKS <= MT * TERMS, "a piece of the cutting per matrix instruction");
@@ -1180,7 +1190,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
             }
             else
             {
-                if constexpr (DP == 64)
+                if constexpr (PAIRED_SHARES)
                 {
                     share += __builtin_bit_cast(float, lane_xor32<32>(__builtin_bit_cast(u32, share)));
                 }
@@ -1199,10 +1209,10 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
             __builtin_amdgcn_sched_barrier(0);
             static_for<0, TERMS>([&](auto j_tag) {
                 constexpr int j = decltype(j_tag)::value;
-                constexpr bool norm_term = DP > 8 && j == 3 * KB;
+                constexpr bool norm_term = DP > 8 && j >= 3 * KB;
                 constexpr int kb = DP <= 8 || norm_term ? 0 : j / 3;
                 constexpr int which = DP <= 8 ? j : j % 3;
-                constexpr int a_at = DP <= 8 ? j : (norm_term ? 2 * KB : (which == 0 ? KB + kb : kb));
+                constexpr int a_at = DP <= 8 ? j : (norm_term ? 2 * KB + (j - 3 * KB) : (which == 0 ? KB + kb : kb));
                 constexpr int b_piece = DP <= 8 ? j : (norm_term ? 2 : (which == 1 ? 1 : 0));
                 constexpr int b_kb = kb;
                 static_for<0, TG>([&](auto t_tag) {
@@ -1252,7 +1262,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
                 halves[2 * sp + h] = vuint2{cut1[0], cut1[1]};
                 halves[2 * (PIECE2 * PT + sp) + h] = vuint2{cut2[0], cut2[1]};
             }
-            reinterpret_cast<u32*>(into_cells + (G::CELLS - 1) * PT + sp)[norm_slot] = cut_norm;
+            reinterpret_cast<u32*>(into_cells + (G::CELLS - G::NORM_CELLS + norm_slot / 4) * PT + sp)[norm_slot % 4] = cut_norm;
         }
     };
     // EXACT, second half of a stage.  First every tile is filtered without a branch: the smallest

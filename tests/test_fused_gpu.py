@@ -157,10 +157,10 @@ def test_point_counts_around_whole_stages(bk, dev, oracle, d, mode):
         pytest.skip("bf16x3 products serve 9 to 64 dimensions")
     if mode == "image" and d > 64:
         pytest.skip("the stage image serves up to 64 dimensions")
-    if mode == "big" and d > 32:
-        pytest.skip("workgroups of 256 queries serve up to 32 dimensions")
+    if mode == "big" and d > 64:
+        pytest.skip("workgroups of 256 queries serve up to 64 dimensions")
     if mode == "big":
-        stage = {8: 256, 16: 256, 32: 128}[d]
+        stage = {8: 256, 16: 256, 32: 128, 64: 64}[d]
     elif mode == "mfma" or d > 64:
         stage = {8: 256, 16: 256, 32: 128, 64: 64, 100: 32}[d]
     else:
