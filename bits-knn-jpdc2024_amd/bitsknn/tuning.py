@@ -236,7 +236,7 @@ def sweep_fused(repeats=3, shapes=FUSED_SHAPES, dims=FUSED_DIMS, k_values=FUSED_
 
 # ---- launch parameters of the fused kernels (bitsknn_fused_tuning) -------------------------------
 FUSED_TUNING_COLUMNS = ("hostname", "GPU", "point_count", "query_count", "dim", "k", "arithmetic", "ranges",
-                        "first_radius", "image", "time", "time_with_the_librarys_choice")
+                        "first_radius", "image", "workgroup", "time", "time_with_the_librarys_choice")
 DEFAULT_FUSED_TUNING = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fused_tuning.csv")
 FUSED_TUNING_SHAPES = ((1024, 1 << 20), (8192, 1 << 17), (65536, 1 << 20))
 FUSED_RANGES = (1, 2, 4, 8, 16, 32, 64)
@@ -249,9 +249,9 @@ def sweep_fused_tuning(repeats=3, shapes=FUSED_TUNING_SHAPES, dims=FUSED_DIMS, k
     """Time bits-fused on cuda:0 over what bitsknn_fused_l2_topk_f32_tuned lets a caller choose: the
     number of ranges the points are cut into, whether (and how densely) a sample of the points
     gives the first radii, and (exact arithmetic) whether the points are cut into stages once per
-    call, per arithmetic.  The counterpart of the reference's sweep over the register tiling of its
+    call and whether a workgroup has 128 or 256 queries, per arithmetic.  The counterpart of the reference's sweep over the register tiling of its
     fused kernel (scripts/run-fused-cache-params.sh).  Yields one dict per measurement; `ranges` 0,
-    `first_radius` 0 and `image` 0 are the library's own choice."""
+    `first_radius` 0, `image` 0 and `workgroup` 0 are the library's own choice."""
     import torch
     import bitsknn
 
@@ -268,19 +268,22 @@ def sweep_fused_tuning(repeats=3, shapes=FUSED_TUNING_SHAPES, dims=FUSED_DIMS, k
                 lists = (8 * q * 64 * k + 255) // 256 * 256
                 workspace = torch.empty(lists + bitsknn.fused_image_bytes(dim, n), dtype=torch.uint8, device=dev)
                 for arithmetic in arithmetics:
-                    choices = [(0, 0, 0)]
+                    choices = [(0, 0, 0, 0)]
                     for ranges in FUSED_RANGES:
                         # more workgroups than eight per compute unit gain nothing
                         if ranges > 1 and (q // 128) * ranges > 2048:
                             continue
                         for first_radius in FUSED_FIRST_RADII:
                             for image in ((-1, 1) if arithmetic == 2 else (-1,)):
-                                choices.append((ranges, first_radius, image))
-                    for ranges, first_radius, image in choices:
+                                choices.append((ranges, first_radius, image, 128))
+                            # (workgroups of 256 queries take no stage image)
+                            if arithmetic == 2 and dim <= 64 and (k <= 32 or (dim <= 8 and k <= 128)):
+                                choices.append((ranges, first_radius, -1, 256))
+                    for ranges, first_radius, image, workgroup in choices:
                         def run():
                             bitsknn.fused_l2_topk(queries, points, k, out_dist=out_d, out_label=out_l,
                                                   workspace=workspace, arithmetic=arithmetic,
-                                                  tuning=(ranges, first_radius, image))
+                                                  tuning=(ranges, first_radius, image, workgroup))
                         run()
                         start = torch.cuda.Event(enable_timing=True)
                         end = torch.cuda.Event(enable_timing=True)
@@ -291,7 +294,7 @@ def sweep_fused_tuning(repeats=3, shapes=FUSED_TUNING_SHAPES, dims=FUSED_DIMS, k
                         end.synchronize()
                         yield {"point_count": n, "query_count": q, "dim": dim, "k": k,
                                "arithmetic": ARITHMETIC_NAMES[arithmetic], "ranges": ranges,
-                               "first_radius": first_radius, "image": image,
+                               "first_radius": first_radius, "image": image, "workgroup": workgroup,
                                "time": start.elapsed_time(end) / 1e3 / repeats}
             if progress is not None:
                 progress(q, dim)
@@ -299,13 +302,13 @@ def sweep_fused_tuning(repeats=3, shapes=FUSED_TUNING_SHAPES, dims=FUSED_DIMS, k
 
 
 def fused_optima(rows):
-    """The fastest (ranges, first_radius, image) per problem and arithmetic, with the time of the
-    library's own choice beside it."""
+    """The fastest (ranges, first_radius, image, workgroup) per problem and arithmetic, with the time
+    of the library's own choice beside it."""
     best = {}
     own = {}
     for row in rows:
         key = (row["point_count"], row["query_count"], row["dim"], row["k"], row["arithmetic"])
-        if row["ranges"] == 0 and row["first_radius"] == 0 and row.get("image", 0) == 0:
+        if row["ranges"] == 0 and row["first_radius"] == 0 and row.get("image", 0) == 0 and row.get("workgroup", 0) == 0:
             own[key] = row["time"]
         elif key not in best or row["time"] < best[key]["time"]:
             best[key] = row
@@ -325,12 +328,12 @@ def write_fused_tuning(rows, path, hostname="mi355x", gpu="MI355X"):
 
 
 def config_fused(query_count, point_count, dim, k, arithmetic="exact", tuning_file=DEFAULT_FUSED_TUNING):
-    """(ranges, first_radius, image) for bitsknn_fused_l2_topk_f32_tuned from the shipped
+    """(ranges, first_radius, image, workgroup) for bitsknn_fused_l2_topk_f32_tuned from the shipped
     measurements: the row of the arithmetic whose problem is nearest to the request (sum of the
-    absolute log ratios of queries, points, dimension and list length); (0, 0, 0), the library's
+    absolute log ratios of queries, points, dimension and list length); (0, 0, 0, 0), the library's
     choice, without a file."""
     import math
-    best, best_cost = (0, 0, 0), None
+    best, best_cost = (0, 0, 0, 0), None
     try:
         with open(tuning_file, newline="") as handle:
             for row in csv.DictReader(handle):
@@ -340,7 +343,8 @@ def config_fused(query_count, point_count, dim, k, arithmetic="exact", tuning_fi
                            for name, want in (("query_count", query_count), ("point_count", point_count),
                                               ("dim", dim), ("k", k)))
                 if best_cost is None or cost < best_cost:
-                    best, best_cost = (int(row["ranges"]), int(row["first_radius"]), int(row.get("image") or 0)), cost
+                    best, best_cost = (int(row["ranges"]), int(row["first_radius"]), int(row.get("image") or 0),
+                                       int(row.get("workgroup") or 0)), cost
     except OSError:
         pass
     return best

@@ -355,7 +355,10 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     // compute unit, ranges of points included.  65536 queries x 2^20 points, k = 32: d = 8 7.65 ->
     // 6.40 ms, d = 16 10.1 -> 8.86 ms, d = 32 16.8 -> 14.3 ms (the stage image, which only the
     // workgroups of 128 queries take, gives 7.10 / 9.82 / 17.2 ms).
+    // (lists of 128 entries in up to 8 dimensions have the shape too, but gain nothing from it:
+    // 11.0 ms against 10.6 ms with the stage image)
     const bool has_big = arithmetic == BITSKNN_FUSED_EXACT && dim <= 64 && (k <= 32 || (dim <= 8 && k <= 128));
+    const bool big_pays = k <= 32 || (dim <= 8 && k <= 64);
     const long long big_workgroups = (static_cast<long long>(q) + 255) / 256 * splits;
     // (every compute unit runs one of them at a time: they are taken where their last round leaves
     // at most an eighth of the units idle -- 224 .. 256, 448 .. 512, ... -- since workgroups of
@@ -363,7 +366,8 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     // two ranges, d = 16: 9.6 ms against 10.2 ms)
     const long long big_rounds = (big_workgroups + 255) / 256;
     const bool big_fills = 8 * big_workgroups >= 7 * 256 * big_rounds;
-    const bool big = has_big && (tuning != nullptr && tuning->workgroup != 0 ? tuning->workgroup == 256 : big_fills);
+    const bool big =
+        has_big && (tuning != nullptr && tuning->workgroup != 0 ? tuning->workgroup == 256 : big_fills && big_pays);
     a.workgroup = big ? 1 : 0;
 
     auto* hip_stream = static_cast<hipStream_t>(stream);
