@@ -355,10 +355,16 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     // compute unit, ranges of points included.  65536 queries x 2^20 points, k = 32: d = 8 7.65 ->
     // 6.40 ms, d = 16 10.1 -> 8.86 ms, d = 32 16.8 -> 14.3 ms (the stage image, which only the
     // workgroups of 128 queries take, gives 7.10 / 9.82 / 17.2 ms).
-    // (lists of 128 entries in up to 8 dimensions have the shape too, but gain nothing from it:
-    // 11.0 ms against 10.6 ms with the stage image)
-    const bool has_big = arithmetic == BITSKNN_FUSED_EXACT && dim <= 64 && (k <= 32 || (dim <= 8 && k <= 128));
-    const bool big_pays = k <= 32 || (dim <= 8 && k <= 64);
+    // Every list length has the shape (its LDS holds the ring of stages for all of them), but long
+    // lists gain from it only where merges are not what the time goes into -- one range of points,
+    // and the longer the list the more dimensions (65536 queries x 2^20 points, 128 -> 256 queries per
+    // workgroup: k = 64 d = 16 / 32 / 64 13.4 -> 10.8, 23.0 -> 17.1, 46.1 -> 30.9 ms; k = 128 d = 16 14.5 ->
+    // 15.4 but d = 32 / 64 25.0 -> 20.7, 51.4 -> 35.2 ms; k = 256 d = 32 28.4 -> 33.7 but d = 64 58.8 ->
+    // 48.5 ms; over ranges 8192 x 2^17, d = 32, k = 128: 1.23 -> 1.83 ms): the waves of the smaller
+    // workgroups merge long lists together at a barrier, these each on its own.
+    const bool has_big = arithmetic == BITSKNN_FUSED_EXACT && dim <= 64;
+    const bool big_pays = k <= 32 || (dim <= 8 && k <= 64) ||
+                          (splits == 1 && (k == 64 || (k == 128 && dim > 16) || (k == 256 && dim > 32)));
     const long long big_workgroups = (static_cast<long long>(q) + 255) / 256 * splits;
     // (every compute unit runs one of them at a time: they are taken where their last round leaves
     // at most an eighth of the units idle -- 224 .. 256, 448 .. 512, ... -- since workgroups of

@@ -69,8 +69,8 @@ struct fused_args
     // below 2^31
     const void* image;
     int image_bytes;
-    // queries per workgroup where the kernel has two shapes (FUSED_ARITH_EXACT up to 32 dimensions,
-    // lists of up to 32 entries): 1 = 256, else 128
+    // queries per workgroup where the kernel has two shapes (FUSED_ARITH_EXACT up to 64 dimensions):
+    // 1 = 256, else 128
     int workgroup;
 #ifdef BITSKNN_FUSED_TIMING
     // instrumented build: cycles of all waves per phase of the stage loop, added up here

@@ -161,8 +161,7 @@ struct fused_geometry
     // workgroup per compute unit -- the same two waves per SIMD, but half the staging, LDS writes
     // and hand-overs per pair.  The exact arithmetic in 32 dimensions on the ring of stages; worth
     // it where the queries alone give every compute unit such a workgroup (launch_fused).
-    static constexpr bool BIG =
-        BIG_OK && ARITH == FUSED_ARITH_EXACT && DP <= 64 && (K <= FQ_CAP || (DP <= 8 && K <= 128));
+    static constexpr bool BIG = BIG_OK && ARITH == FUSED_ARITH_EXACT && DP <= 64;
     static constexpr int WAVES = BIG ? 2 * FQ_WAVES : FQ_WAVES;
     static constexpr int THREADS = WAVES * WAVE;
     static constexpr int QB = FQ_QW * WAVES; // queries per workgroup
@@ -178,7 +177,7 @@ struct fused_geometry
     // 16 matrix dimensions.
     // (one norm cell holds the shares of four groups of 8 dimensions: a second one where eight
     // groups are staged by eight waves)
-    static constexpr int NORM_CELLS = DP == 64 && BIG_OK && ARITH == FUSED_ARITH_EXACT && K <= FQ_CAP ? 2 : 1;
+    static constexpr int NORM_CELLS = DP == 64 && BIG ? 2 : 1;
     static constexpr int CELLS = EXACT ? (DP <= 8 ? 3 : 2 * KS + NORM_CELLS) : 0;
     static constexpr int PT = SPLIT   ? (DK <= 16 ? 128 : (DK <= 32 ? 64 : 32))
                               : EXACT ? (DP <= 16 ? 128 : (DP <= 32 ? 64 : 32)) * (BIG ? 2 : 1)
@@ -234,9 +233,11 @@ struct fused_geometry
     // (The geometry with 64-slot buffers would have room for three of its small stages, but its
     // long lists over ranges want the waves merging together: 8192 queries x 2^17 points, d = 8,
     // k = 128 1.10 -> 1.46 ms on the ring.)
+    // (The workgroups of 256 queries have the LDS of a whole compute unit: the ring for every list
+    // length, with buffers of 20 to 32 slots.)
     static constexpr bool RING =
         !WIDE && (SPLIT ? K <= FQ_CAP
-                        : (DP <= 8 && K <= 128) || (DP >= 16 && DP <= RING_MAX_DP && K <= FQ_CAP));
+                        : BIG || (DP <= 8 && K <= 128) || (DP >= 16 && DP <= RING_MAX_DP && K <= FQ_CAP));
     static constexpr int NB = RING ? 3 : 2;
     // slots a query buffer has in LDS (20 where the three stages of 256 points in 16 dimensions leave
     // no more room next to the buffers of 256 queries)
@@ -244,6 +245,9 @@ struct fused_geometry
                                  : BIG && DP == 16 ? 20
                                  : RING && !SPLIT && DP >= 16 ? 24
                                                               : CAP;
+    // (lists longer than a buffer sort their buffers as CAP keys; a buffer of fewer slots keeps the
+    // last SLOTS of them, since the first CAP - SLOTS of the descending order are padding)
+    static constexpr int DROP = CAP - SLOTS;
     static_assert(!SPLIT || (DP <= 64 && TPP == KS), "one staging thread per point and cell");
     static_assert(!EXACT || (DP <= 64 && VPT == (DP <= 8 ? 4 : 8) && MT <= 4 && SUB <= 2),
                   "the stages of the exact arithmetic serve up to 64 dimensions, in passes of at most four tiles");
@@ -271,7 +275,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
     constexpr int PT = G::PT;
     constexpr int CAP = G::CAP;
     constexpr int SLOTS = G::SLOTS;
-    static_assert(K <= CAP || SLOTS == CAP, "lists longer than a buffer sort all CAP slots of it in place");
+    constexpr int DROP = K > CAP ? G::DROP : 0;
     // Norms in the accumulator: where ||p||^2 is one row after the point rows -- one staging thread
     // carries a whole point (DP <= 16), or the 2 or 4 staging threads of a point are neighbouring
     // lanes that add up their shares (DP = 32, 64) -- it is read as the initial value of the
@@ -502,7 +506,12 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
 #pragma unroll
                 for (int r = 0; r < BR; ++r)
                 {
-                    wbuf[qm * SLOTS + sub * BR + r] = buf[r];
+                    // (descending, padding first: at least the first DROP keys are padding)
+                    const int i = sub * BR + r;
+                    if (DROP == 0 || i >= DROP)
+                    {
+                        wbuf[qm * SLOTS + i - DROP] = buf[r];
+                    }
                 }
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -547,7 +556,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
                 {
                     // the sorted buffer (descending, padding first) is the tail of a descending
                     // sequence of K keys
-                    buf[r] = i >= K - CAP ? wbuf[qm * SLOTS + i - (K - CAP)] : PAD_KEY;
+                    buf[r] = i >= K - CAP + DROP ? wbuf[qm * SLOTS + i - (K - CAP) - DROP] : PAD_KEY;
                 }
                 else
                 {

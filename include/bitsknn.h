@@ -301,11 +301,11 @@ int bitsknn_fused_l2_topk_f32_ex(const float* queries_dim_major, const float* po
  *                 every workgroup again: 1 = whenever the workspace has room, -1 = never, 0 = the
  *                 library's choice (from 4096 queries on, up to 16 dimensions)
  *   workgroup     queries per workgroup where the kernel comes in two shapes (BITSKNN_FUSED_EXACT up
- *                 to 32 dimensions, lists of up to 32 entries): 128 (four waves), 256 (eight waves
- *                 sharing stages of twice the points; no stage image then) or 0 = the library's
- *                 choice (256 where ceil(q / 256) * ranges workgroups, one at a time on each of
- *                 the 256 compute units, leave at most an eighth of the units idle in their last
- *                 round)
+ *                 to 64 dimensions): 128 (four waves), 256 (eight waves sharing stages of twice
+ *                 the points; no stage image then) or 0 = the library's choice (256 where
+ *                 ceil(q / 256) * ranges workgroups, one at a time on each of the 256 compute
+ *                 units, leave at most an eighth of the units idle in their last round; lists of
+ *                 64 and more only over one range of points, the longer ones in more dimensions)
  * tuning == NULL: the library's choices.  Results do not depend on the tuning (for
  * BITSKNN_FUSED_EXACT bit for bit; for the other arithmetics the distances of a point can differ in
  * the last bit between one range and several).  bitsknn/tuning.py sweeps these and records the
