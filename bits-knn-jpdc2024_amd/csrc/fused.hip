@@ -363,8 +363,12 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     // 48.5 ms; over ranges 8192 x 2^17, d = 32, k = 128: 1.23 -> 1.83 ms): the waves of the smaller
     // workgroups merge long lists together at a barrier, these each on its own.
     const bool has_big = arithmetic == BITSKNN_FUSED_EXACT && dim <= 64;
-    const bool big_pays = k <= 32 || (dim <= 8 && k <= 64) ||
-                          (splits == 1 && (k == 64 || (k == 128 && dim > 16) || (k == 256 && dim > 32)));
+    // (Over ranges, lists of 64 gain above 32 dimensions -- 4096 x 2^20, d = 64: 4.7 -> 3.4 ms,
+    // 8192 x 2^17: 1.78 -> 1.60 ms -- and lists of 128 where a range has at least 2^18 points: 16384 x
+    // 2^20, d = 64: 16.1 -> 13.1 ms, but 8192 x 2^17: 2.05 -> 2.53 ms.)
+    const bool long_ranges = splits == 1 || n / splits >= (1 << 18);
+    const bool big_pays = k <= 32 || (dim <= 8 && k <= 64) || (k == 64 && (splits == 1 || dim > 32)) ||
+                          (k == 128 && dim > 16 && long_ranges) || (k == 256 && dim > 32 && splits == 1);
     const long long big_workgroups = (static_cast<long long>(q) + 255) / 256 * splits;
     // (every compute unit runs one of them at a time: they are taken where their last round leaves
     // at most an eighth of the units idle -- 224 .. 256, 448 .. 512, ... -- since workgroups of
