@@ -38,8 +38,9 @@ def _fused(bk, dev, points, queries, k, params=(8, 4, 2), bqd=1, dim_mult=1, wor
         return od.cpu().numpy(), ol.cpu().numpy()
     if arithmetic == "big":
         # the default arithmetic in workgroups of 256 queries (forced: the library itself takes them
-        # where they fill the chip), ranges as the library chooses
-        od, ol = bk.fused_l2_topk(qd, pd, k, workspace="auto", tuning=(0, 0, 0, 256))
+        # where they fill the chip), ranges as the library chooses ("one-range": a single one)
+        od, ol = bk.fused_l2_topk(qd, pd, k, workspace=None if workspace == "one-range" else "auto",
+                                  tuning=(0, 0, 0, 256))
         bk.fused_status()
         return od.cpu().numpy(), ol.cpu().numpy()
     od, ol = bk.fused_l2_topk(qd, pd, k, params, bqd, dim_mult, workspace=workspace, arithmetic=arithmetic)
@@ -403,7 +404,10 @@ def _sampled_points(n, d, small_stages, scale):
                                              (16, 128, "mfma", True), (32, 64, "mfma", True),
                                              (8, 64, "default", True), (8, 256, "default", True),
                                              (16, 128, "default", True), (32, 64, "default", True),
-                                             (24, 128, "bf16x3", True)])
+                                             (24, 128, "bf16x3", True),
+                                             (8, 64, "big", False), (16, 128, "big", False), (32, 256, "big", False),
+                                             (64, 128, "big", False), (8, 256, "big", True), (32, 64, "big", True),
+                                             (64, 64, "big", True)])
 def test_first_radius_from_a_sample(bk, dev, oracle, d, k, mode, ranges):
     """Lists on many points start from radii that a launch over a sample of the points
     estimates, and workgroups with a query whose estimate proved too low repeat their pass; the
@@ -417,13 +421,17 @@ def test_first_radius_from_a_sample(bk, dev, oracle, d, k, mode, ranges):
     arithmetic = _arith(bk, mode)
     bits = _bits(mode, d)
     workspace = "auto" if ranges else None
+    if mode == "big" and not ranges:
+        workspace = "one-range"
     if ranges:
         assert bk.fused_workspace_bytes(q, n, k) > 0
     gd, gl = _fused(bk, dev, points, queries, k, arithmetic=arithmetic, workspace=workspace)
     _check(oracle, points, queries, k, gd, gl, bits=bits)
     assert not np.isnan(gd).any()
     # (over ranges the sample has about 2048 points: one stage in every 64 .. 256)
-    sample = _sampled_points(n, d, mode == "bf16x3" or bits, max(64, min(256, n // 2048)) if ranges else 64)
+    # (the workgroups of 256 queries have the stage sizes of the fp32 matrix instructions)
+    sample = _sampled_points(n, d, mode == "bf16x3" or (bits and mode != "big"),
+                             max(64, min(256, n // 2048)) if ranges else 64)
     assert sample.size >= 2 * 32
     points = rng.random((n, d), dtype=np.float32)
     points[:, :4] += 1.0                    # all points a step away in four dimensions ...
