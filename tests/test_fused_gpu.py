@@ -442,7 +442,7 @@ def test_first_radius_from_a_sample(bk, dev, oracle, d, k, mode, ranges):
     assert not np.isnan(gd).any()
 
 
-@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("mode", MODES + ["big"])
 def test_random_shapes_against_the_oracle(bk, dev, oracle, mode):
     """40 random problems over dimensions on both sides of every padded size, all list lengths,
     ragged point and query counts, with the plain entry point, the workspace the library asks for
@@ -464,8 +464,8 @@ def test_random_shapes_against_the_oracle(bk, dev, oracle, mode):
             workspace = torch.empty(max(8, 8 * q * 64 * k), dtype=torch.uint8, device=dev)
         p, s = oracle.generate(3000 + case, n, q, d)
         arithmetic = _arith(bk, mode)
-        if arithmetic is not None and workspace is None:
-            workspace = None  # (bitsknn_fused_l2_topk_f32_ex takes no workspace as well)
+        if mode == "big":
+            workspace = "one-range" if kind == 0 else "auto"
         gd, gl = _fused(bk, dev, p, s, k, (2, 4, 1), 1, 1, workspace=workspace, arithmetic=arithmetic)
         try:
             _check(oracle, p, s, k, gd, gl, bits=_bits(mode, d))
