@@ -362,7 +362,9 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     // 15.4 but d = 32 / 64 25.0 -> 20.7, 51.4 -> 35.2 ms; k = 256 d = 32 28.4 -> 33.7 but d = 64 58.8 ->
     // 48.5 ms; over ranges 8192 x 2^17, d = 32, k = 128: 1.23 -> 1.83 ms): the waves of the smaller
     // workgroups merge long lists together at a barrier, these each on its own.
-    const bool has_big = arithmetic == BITSKNN_FUSED_EXACT && dim <= 64;
+    // (65 .. 128 dimensions have the exact arithmetic in this shape only)
+    const bool has_big = arithmetic == BITSKNN_FUSED_EXACT && dim <= 128;
+    const bool only_big = has_big && dim > 64;
     // (Over ranges, lists of 64 gain above 32 dimensions -- 4096 x 2^20, d = 64: 4.7 -> 3.4 ms,
     // 8192 x 2^17: 1.78 -> 1.60 ms -- and lists of 128 where a range has at least 2^18 points: 16384 x
     // 2^20, d = 64: 16.1 -> 13.1 ms, but 8192 x 2^17: 2.05 -> 2.53 ms.)
@@ -377,7 +379,8 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     const long long big_rounds = (big_workgroups + 255) / 256;
     const bool big_fills = 8 * big_workgroups >= 7 * 256 * big_rounds;
     const bool big =
-        has_big && (tuning != nullptr && tuning->workgroup != 0 ? tuning->workgroup == 256 : big_fills && big_pays);
+        has_big && (only_big || (tuning != nullptr && tuning->workgroup != 0 ? tuning->workgroup == 256
+                                                                             : big_fills && big_pays));
     a.workgroup = big ? 1 : 0;
 
     auto* hip_stream = static_cast<hipStream_t>(stream);

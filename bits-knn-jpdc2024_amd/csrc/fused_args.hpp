@@ -22,7 +22,7 @@ constexpr int FQ_CAP = 32;                    // buffer slots per query (= point
 //  FUSED_ARITH_EXACT     a lower bound of every distance from three bf16 matrix products of two
 //                        pieces per operand filters the tile; what passes is computed with
 //                        sequential fused multiply-adds in dimension order (the reference's
-//                        arithmetic), filtered again and appended (dimensions up to 64)
+//                        arithmetic), filtered again and appended (dimensions up to 128)
 constexpr int FUSED_ARITH_MFMA_F32 = 0;
 constexpr int FUSED_ARITH_BF16X3 = 1;
 constexpr int FUSED_ARITH_EXACT = 2;
@@ -70,7 +70,7 @@ struct fused_args
     const void* image;
     int image_bytes;
     // queries per workgroup where the kernel has two shapes (FUSED_ARITH_EXACT up to 64 dimensions):
-    // 1 = 256, else 128
+    // 1 = 256, else 128 (65 .. 128 dimensions: always 256)
     int workgroup;
 #ifdef BITSKNN_FUSED_TIMING
     // instrumented build: cycles of all waves per phase of the stage loop, added up here

@@ -14,8 +14,9 @@ namespace bitsknn
 #define BITSKNN_CAT_EXPANDED(a, b) BITSKNN_CAT2(a, b)
 
 // FUSED_ARITH_BF16X3: dimensions 9 .. 64 (below 9 the fp32 matrix instructions are as fast);
-// FUSED_ARITH_EXACT: dimensions up to 64 (a stage holds the points twice, as fp32 rows and as bf16
-// pieces); everything else takes the fp32 matrix instructions
+// FUSED_ARITH_EXACT: dimensions up to 128 (a stage holds the points twice, as fp32 rows and as bf16
+// pieces; 65 .. 128 dimensions only in workgroups of 256 queries, whatever fused_args::workgroup
+// says); everything else takes the fp32 matrix instructions
 hipError_t BITSKNN_CAT_EXPANDED(launch_fused_k_, BITSKNN_FUSED_K)(const fused_args& a, int arith,
                                                                   hipStream_t stream)
 {
@@ -32,6 +33,10 @@ hipError_t BITSKNN_CAT_EXPANDED(launch_fused_k_, BITSKNN_FUSED_K)(const fused_ar
                : a.dim <= 16 ? launch_fused<K, 16, FUSED_ARITH_EXACT>(a, stream)
                : a.dim <= 32 ? launch_fused<K, 32, FUSED_ARITH_EXACT>(a, stream)
                              : launch_fused<K, 64, FUSED_ARITH_EXACT>(a, stream);
+    }
+    if (arith == FUSED_ARITH_EXACT && a.dim <= 128)
+    {
+        return launch_fused_as<K, 128, FUSED_ARITH_EXACT, false, true>(a, stream);
     }
     if (a.dim <= 8)
     {

@@ -123,8 +123,13 @@ __device__ __forceinline__ void cut_bf16x2(const float (&x)[8], vuint4& p1, vuin
 //   W <= V + FILTER_REL * Q        whenever V is finite,
 // and a pair can only have V < radius if W < radius + FILTER_REL * Q.  The compare is written so
 // that a NaN in W passes; FILTER_ABS covers products of pieces that underflow.
+// In 65 .. 128 dimensions (28 matrix instructions per tile, d + 2 <= 130 roundings in V) the three
+// terms are 7.8e-6, 4.7e-5 and 5.7e-5 of S: FILTER_REL_WIDE = 1.5 * 2^-13 (1.83e-4) leaves a factor
+// of 1.6, with NORM_LOWER_WIDE = 1.75 * 2^-12 >= 2 FILTER_REL_WIDE + 2^-15.3.
 constexpr float FILTER_REL = 0x1.0p-13F;
 constexpr float NORM_LOWER = 0x1.4p-12F;
+constexpr float FILTER_REL_WIDE = 0x1.8p-13F;
+constexpr float NORM_LOWER_WIDE = 0x1.cp-12F;
 constexpr float FILTER_ABS = 0x1.0p-100F;
 // norm of the points beyond the end of a range: the largest finite bf16, so that they only pass the
 // filter while a radius is still infinite (what passes is checked against the range again)
@@ -161,7 +166,8 @@ struct fused_geometry
     // workgroup per compute unit -- the same two waves per SIMD, but half the staging, LDS writes
     // and hand-overs per pair.  The exact arithmetic in 32 dimensions on the ring of stages; worth
     // it where the queries alone give every compute unit such a workgroup (launch_fused).
-    static constexpr bool BIG = BIG_OK && ARITH == FUSED_ARITH_EXACT && DP <= 64;
+    // (65 .. 128 dimensions exist in this shape only: a stage of 32 points has 34 KB there)
+    static constexpr bool BIG = BIG_OK && ARITH == FUSED_ARITH_EXACT && DP <= 128;
     static constexpr int WAVES = BIG ? 2 * FQ_WAVES : FQ_WAVES;
     static constexpr int THREADS = WAVES * WAVE;
     static constexpr int QB = FQ_QW * WAVES; // queries per workgroup
@@ -177,10 +183,10 @@ struct fused_geometry
     // 16 matrix dimensions.
     // (one norm cell holds the shares of four groups of 8 dimensions: a second one where eight
     // groups are staged by eight waves)
-    static constexpr int NORM_CELLS = DP == 64 && BIG ? 2 : 1;
+    static constexpr int NORM_CELLS = DP == 128 && BIG ? 4 : (DP == 64 && BIG ? 2 : 1);
     static constexpr int CELLS = EXACT ? (DP <= 8 ? 3 : 2 * KS + NORM_CELLS) : 0;
     static constexpr int PT = SPLIT   ? (DK <= 16 ? 128 : (DK <= 32 ? 64 : 32))
-                              : EXACT ? (DP <= 16 ? 128 : (DP <= 32 ? 64 : 32)) * (BIG ? 2 : 1)
+                              : EXACT ? (DP <= 16 ? 128 : (DP <= 32 ? 64 : (DP <= 64 ? 32 : 16))) * (BIG ? 2 : 1)
                               : WIDE  ? (DP <= 8 ? 128 : 64)
                                       : (DP <= 16 ? 256 : (DP <= 32 ? 128 : (DP <= 64 ? 64 : 32)));
     // threads per point when staging.  The small stages of the 64-slot geometry are staged by their
@@ -249,8 +255,9 @@ struct fused_geometry
     // last SLOTS of them, since the first CAP - SLOTS of the descending order are padding)
     static constexpr int DROP = CAP - SLOTS;
     static_assert(!SPLIT || (DP <= 64 && TPP == KS), "one staging thread per point and cell");
-    static_assert(!EXACT || (DP <= 64 && VPT == (DP <= 8 ? 4 : 8) && MT <= 4 && SUB <= 2),
-                  "the stages of the exact arithmetic serve up to 64 dimensions, in passes of at most four tiles");
+    static_assert(!EXACT || ((DP <= 64 || (DP == 128 && BIG)) && VPT == (DP <= 8 ? 4 : 8) && MT <= 4 && SUB <= 2),
+                  "the stages of the exact arithmetic serve up to 64 dimensions (128 in workgroups of 256 "
+                  "queries), in passes of at most four tiles");
     static constexpr size_t lds_bytes()
     {
         // the stages, the query buffers, exchange slots, merge flags and stage counters
@@ -338,7 +345,11 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
     vuint4 qs[SPLIT || EXACT ? 3 : 1][SPLIT || EXACT ? KB : 1];
     // EXACT: the query itself, every dimension, for the sequential arithmetic; the slack of its
     // filter threshold above the radius
-    float qx[EXACT ? DP : 1];
+    // (beyond 64 dimensions the query is read again where a candidate needs it)
+    constexpr bool QUERY_IN_REGISTERS = EXACT && DP <= 64;
+    constexpr float FILTER_REL_DP = DP > 64 ? FILTER_REL_WIDE : FILTER_REL;
+    constexpr float NORM_LOWER_DP = DP > 64 ? NORM_LOWER_WIDE : NORM_LOWER;
+    float qx[QUERY_IN_REGISTERS ? DP : 1];
     float filter_slack = 0.0F;
     float thr = __builtin_inff();    // EXACT: what a filter value must not exceed to be looked at
     int radius_label = 0x7FFFFFFF;   // EXACT: label of the list entry the radius comes from
@@ -349,39 +360,74 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
         // (every load from a valid address, so that they are all in flight together)
         const bool live = my_q < a.q;
         const float* const mine = a.queries + (live ? my_q : 0);
-#pragma unroll
-        for (int dd = 0; dd < DP; ++dd)
-        {
-            const float x = mine[static_cast<size_t>(dd < dim ? dd : 0) * a.q];
-            qx[dd] = dd < dim && live ? x : 0.0F;
-        }
-#pragma unroll
-        for (int dd = 0; dd < DP; ++dd)
-        {
-            qq = __builtin_fmaf(qx[dd], qx[dd], qq);
-        }
-        filter_slack = FILTER_REL * qq * (1.0F + 0x1.0p-20F) + FILTER_ABS * (1.0F + qq);
         // (the norm cell holds two pieces per share of the norm, at most four shares)
         const vuint4 ones{0x3F803F80U, 0x3F803F80U, 0x3F803F80U, 0x3F803F80U};
         const vuint4 zeros{0, 0, 0, 0};
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb)
+        if constexpr (QUERY_IN_REGISTERS)
         {
-            float val[8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
+            for (int dd = 0; dd < DP; ++dd)
             {
-                // (a select between registers: the query is not indexed by the lane)
-                const int first = DP <= 8 ? j : 16 * kb + j;
-                const int second = DP <= 8 ? j : 16 * kb + 8 + j;
-                float lower = qx[first];
-                float upper = qx[second < DP ? second : 0];
-                asm volatile("" : "+v"(lower), "+v"(upper));
-                val[j] = -2.0F * (half != 0 ? upper : lower);
+                const float x = mine[static_cast<size_t>(dd < dim ? dd : 0) * a.q];
+                qx[dd] = dd < dim && live ? x : 0.0F;
             }
-            cut_bf16x2(val, qs[0][kb], qs[1][kb]);
-            qs[2][kb] = half == 0 ? ones : zeros;
+#pragma unroll
+            for (int dd = 0; dd < DP; ++dd)
+            {
+                qq = __builtin_fmaf(qx[dd], qx[dd], qq);
+            }
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+            {
+                float val[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                {
+                    // (a select between registers: the query is not indexed by the lane)
+                    const int first = DP <= 8 ? j : 16 * kb + j;
+                    const int second = DP <= 8 ? j : 16 * kb + 8 + j;
+                    float lower = qx[first];
+                    float upper = qx[second < DP ? second : 0];
+                    asm volatile("" : "+v"(lower), "+v"(upper));
+                    val[j] = -2.0F * (half != 0 ? upper : lower);
+                }
+                cut_bf16x2(val, qs[0][kb], qs[1][kb]);
+                qs[2][kb] = half == 0 ? ones : zeros;
+            }
         }
+        else
+        {
+            // 16 dimensions at a time: the lane keeps the pieces of its half of them
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+            {
+                float both[16];
+#pragma unroll
+                for (int j = 0; j < 16; ++j)
+                {
+                    const int dd = 16 * kb + j;
+                    const float x = mine[static_cast<size_t>(dd < dim ? dd : 0) * a.q];
+                    both[j] = dd < dim && live ? x : 0.0F;
+                }
+                float val[8];
+#pragma unroll
+                for (int j = 0; j < 16; ++j)
+                {
+                    qq = __builtin_fmaf(both[j], both[j], qq);
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                {
+                    float lower = both[j];
+                    float upper = both[8 + j];
+                    asm volatile("" : "+v"(lower), "+v"(upper));
+                    val[j] = -2.0F * (half != 0 ? upper : lower);
+                }
+                cut_bf16x2(val, qs[0][kb], qs[1][kb]);
+                qs[2][kb] = half == 0 ? ones : zeros;
+            }
+        }
+        filter_slack = FILTER_REL_DP * qq * (1.0F + 0x1.0p-20F) + FILTER_ABS * (1.0F + qq);
         if constexpr (DP <= 8)
         {
             qs[1][0] = half == 0 ? qs[1][0] : ones;
@@ -909,7 +955,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
                 // the lowered share of the norm in two pieces, one word of the point's norm cell per
                 // share (the matrix instruction adds them up); points beyond the end only pass an
                 // infinite radius
-                const float lowered = __builtin_fmaf(-NORM_LOWER, share, share);
+                const float lowered = __builtin_fmaf(-NORM_LOWER_DP, share, share);
                 const vfloat2 whole{lowered, 0.0F};
                 const u32 first = __builtin_bit_cast(u32, __builtin_convertvector(whole, vbf16x2)) & 0xFFFFU;
                 const vfloat2 rest{lowered - __builtin_bit_cast(float, first << 16U), 0.0F};
@@ -1004,12 +1050,51 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
             const float* const column = stage + local;
             float norm = 0.0F;
             float dot = 0.0F;
-#pragma unroll
-            for (int dd = 0; dd < DP; ++dd)
+            if constexpr (QUERY_IN_REGISTERS)
             {
-                const float x = column[dd * PT];
-                norm = __builtin_fmaf(x, x, norm);
-                dot = __builtin_fmaf(qx[dd], x, dot);
+#pragma unroll
+                for (int dd = 0; dd < DP; ++dd)
+                {
+                    const float x = column[dd * PT];
+                    norm = __builtin_fmaf(x, x, norm);
+                    dot = __builtin_fmaf(qx[dd], x, dot);
+                }
+            }
+            else
+            {
+                // the query comes from memory again, QC dimensions at a time, whose loads are all
+                // issued ahead of their arithmetic (zero beyond dim, as the point's rows are)
+                constexpr int QC = 16;
+                const float* const mine = a.queries + (my_q < a.q ? my_q : 0);
+#pragma unroll 1
+                for (int d0 = 0; d0 < DP; d0 += QC)
+                {
+                    float y[QC];
+                    if (d0 + QC <= dim)
+                    {
+#pragma unroll
+                        for (int j = 0; j < QC; ++j)
+                        {
+                            y[j] = mine[static_cast<size_t>(d0 + j) * a.q];
+                        }
+                    }
+                    else
+                    {
+#pragma unroll
+                        for (int j = 0; j < QC; ++j)
+                        {
+                            const float there = mine[static_cast<size_t>(d0 + j < dim ? d0 + j : 0) * a.q];
+                            y[j] = d0 + j < dim ? there : 0.0F;
+                        }
+                    }
+#pragma unroll
+                    for (int j = 0; j < QC; ++j)
+                    {
+                        const float x = column[(d0 + j) * PT];
+                        norm = __builtin_fmaf(x, x, norm);
+                        dot = __builtin_fmaf(y[j], x, dot);
+                    }
+                }
             }
             const float value = __builtin_fmaf(-2.0F, dot, norm);
             const int label = base + local;
@@ -1203,7 +1288,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
                 {
                     share += __builtin_bit_cast(float, lane_xor32<32>(__builtin_bit_cast(u32, share)));
                 }
-                const float lowered = __builtin_fmaf(-NORM_LOWER, share, share);
+                const float lowered = __builtin_fmaf(-NORM_LOWER_DP, share, share);
                 const vfloat2 whole{lowered, 0.0F};
                 const u32 first = __builtin_bit_cast(u32, __builtin_convertvector(whole, vbf16x2)) & 0xFFFFU;
                 const vfloat2 rest{lowered - __builtin_bit_cast(float, first << 16U), 0.0F};
@@ -1211,6 +1296,61 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
                 cut_norm = cut_base + sp < n ? first | (second << 16U) : BF16_HUGE;
             }
         };
+        if constexpr (NCELL > 12)
+        {
+            // (one tile whose cells do not fit the registers at once: they are read in pairs -- the
+            // two cells of 16 dimensions that three matrix instructions take, then the norm cells --
+            // AHEAD pairs ahead of the instructions that take them)
+            static_assert(MT == 1 && G::SUB == 1 && G::NORM_CELLS == 4);
+            constexpr int AHEAD = 2;
+            constexpr int PAIRS = KB + 2;
+            const vuint4* const mine = reinterpret_cast<const vuint4*>(stage + DP * PT) + ql;
+            vuint4 pair[AHEAD + 1][2];
+            auto read_pair = [&](auto s_tag) __attribute__((always_inline)) {
+                constexpr int at = decltype(s_tag)::value;
+                if constexpr (at < KB)
+                {
+                    // piece 2, then piece 1, of dimensions 16 at ..
+                    pair[at % (AHEAD + 1)][0] = mine[(KS + 2 * at + half) * PT];
+                    pair[at % (AHEAD + 1)][1] = mine[(2 * at + half) * PT];
+                }
+                else if constexpr (at < PAIRS)
+                {
+                    pair[at % (AHEAD + 1)][0] = mine[(2 * KS + 2 * (at - KB)) * PT];
+                    pair[at % (AHEAD + 1)][1] = mine[(2 * KS + 2 * (at - KB) + 1) * PT];
+                }
+            };
+            static_for<0, AHEAD>([&](auto s_tag) { read_pair(s_tag); });
+            static_for<0, PAIRS>([&](auto s_tag) {
+                constexpr int at = decltype(s_tag)::value;
+                read_pair(std::integral_constant<int, at + AHEAD>{});
+                constexpr int slot = at % (AHEAD + 1);
+                if constexpr (at < KB)
+                {
+                    static_for<0, 3>([&](auto which_tag) {
+                        constexpr int which = decltype(which_tag)::value;
+                        constexpr int m = 3 * at + which;
+                        w[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(vbf16x8, pair[slot][which == 0 ? 0 : 1]),
+                            __builtin_bit_cast(vbf16x8, qs[which == 1 ? 1 : 0][at]), m == 0 ? zero : w[0], 0, 0, 0);
+                        if constexpr (m < CHUNKS)
+                        {
+                            chunk(std::integral_constant<int, m>{});
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    });
+                }
+                else
+                {
+                    w[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(vbf16x8, pair[slot][0]),
+                                                                   __builtin_bit_cast(vbf16x8, qs[2][0]), w[0], 0, 0, 0);
+                    w[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(vbf16x8, pair[slot][1]),
+                                                                   __builtin_bit_cast(vbf16x8, qs[2][0]), w[0], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            });
+        }
+        else
         static_for<0, MT / TG>([&](auto g_tag) {
             constexpr int g = decltype(g_tag)::value;
             vuint4 cell[TG][NCELL];

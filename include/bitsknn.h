@@ -202,7 +202,7 @@ int bitsknn_dist_layout_f32(int op, int dim, size_t q, size_t n, const float* qu
  *                             over them measures the same kernel every time (what a sweep can
  *                             vary here: bitsknn_fused_l2_topk_f32_tuned)
  * The distances are computed in the reference's arithmetic (BITSKNN_FUSED_EXACT below) for
- * dim <= 64 and on the fp32 matrix instructions beyond.
+ * dim <= 128 and on the fp32 matrix instructions beyond.
  * A call enqueues one to three kernels on `stream` (long lists over many points are preceded by a
  * pass over a sample of the points, which gives every query a first radius, and followed by one
  * that repeats the queries whose first radius proved too low); until the last of them has run,
@@ -229,7 +229,7 @@ int bitsknn_fused_l2_topk_f32(const float* queries_dim_major, const float* point
  * ranges; 0 when the queries fill the GPU by themselves.  A smaller workspace (4-byte aligned) is
  * not an error: the call uses as many ranges as fit, down to the single kernel without any.
  *
- * The stage image.  In the exact arithmetic (dim <= 64) every workgroup cuts every point into bf16
+ * The stage image.  In the exact arithmetic every workgroup cuts every point into bf16
  * pieces again.  With bitsknn_fused_image_bytes(dim, n) more bytes in the workspace, behind the
  * partial lists rounded up to a multiple of 256 bytes (and the workspace 16-byte aligned), a launch
  * of its own writes the stages of the whole point matrix there once per call and the fused kernel
@@ -250,7 +250,7 @@ int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major, const float* po
  * bits-fused with the arithmetic of the products q.p chosen per call (nothing process-wide is
  * read); workspace may be NULL (then as bitsknn_fused_l2_topk_f32) or as for
  * bitsknn_fused_l2_topk_f32_ws.
- *   BITSKNN_FUSED_EXACT   what the entry points above use.  For dim <= 64 every reported distance
+ *   BITSKNN_FUSED_EXACT   what the entry points above use.  For dim <= 128 every reported distance
  *                         is computed as the reference's kernel computes it -- norm and dot
  *                         product by sequential fused multiply-adds over the dimensions in order,
  *                         then norm - 2 dot (include/bits/topk/singlepass/
@@ -259,8 +259,9 @@ int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major, const float* po
  *                         Which pairs to compute is decided by a filter on the bf16 matrix
  *                         instructions (v_mfma_f32_32x32x16_bf16, two bf16 pieces per operand, three
  *                         products) whose value is a guaranteed lower bound of the distance less a
- *                         slack of 2^-13 ||q||^2: no pair below a query's current k-th distance is
- *                         ever dropped.  Larger dimensions use BITSKNN_FUSED_FP32.
+ *                         slack of 2^-13 ||q||^2 (1.5 * 2^-13 above 64 dimensions): no pair below a
+ *                         query's current k-th distance is ever dropped.  Larger dimensions use
+ *                         BITSKNN_FUSED_FP32.
  *   BITSKNN_FUSED_FP32    every distance from fp32 matrix instructions (v_mfma_f32_32x32x2_f32):
  *                         within 1e-5 of the reference arithmetic, not bit-identical to it.
  *   BITSKNN_FUSED_BF16X3  for 9 <= dim <= 64: every fp32 operand is cut exactly into three bf16
@@ -301,7 +302,8 @@ int bitsknn_fused_l2_topk_f32_ex(const float* queries_dim_major, const float* po
  *                 every workgroup again: 1 = whenever the workspace has room, -1 = never, 0 = the
  *                 library's choice (from 4096 queries on, up to 16 dimensions)
  *   workgroup     queries per workgroup where the kernel comes in two shapes (BITSKNN_FUSED_EXACT up
- *                 to 64 dimensions): 128 (four waves), 256 (eight waves sharing stages of twice
+ *                 to 64 dimensions; 65 .. 128 dimensions have the one of 256 queries only and
+ *                 ignore the field): 128 (four waves), 256 (eight waves sharing stages of twice
  *                 the points; no stage image then) or 0 = the library's choice (256 where
  *                 ceil(q / 256) * ranges workgroups, one at a time on each of the 256 compute
  *                 units, leave at most an eighth of the units idle in their last round; lists of
