@@ -371,7 +371,10 @@ def leg_gemm(bitsknn, torch, timer, oracle, dev, steps, check, q=4096, n=1 << 20
 def filter_flops_per_pair(d):
     """bf16 matrix flops the default fused kernel executes per (query, point) pair: matrix
     instructions of 32 x 32 x 16, two per tile up to 8 dimensions, else three per 16 dimensions
-    (two pieces per operand, the smallest product left out) and one for the norm"""
+    (two pieces per operand, the smallest product left out) and one for the norm; 65 .. 128
+    dimensions are padded to 128 and take two for the norm (sixteen shares of it)"""
+    if d > 64:
+        return (3 * 8 + 2) * 32.0
     terms = 2 if d <= 8 else 3 * ((d + 15) // 16) + 1
     return terms * 32.0
 
@@ -439,7 +442,7 @@ def leg_fused(bitsknn, torch, timer, oracle, dev, steps, check, dims, ks, q=6553
                 ok, detail = verify_neighbours(np, points_h, queries_h, exp_d, exp_l, out_d[sample].cpu().numpy(),
                                                out_l[sample].cpu().numpy(), k)
                 # the default arithmetic is the reference's: nothing but bit for bit counts
-                entry["verified"] = bool(ok and (detail["bit_exact_values_and_labels"] or d > 64))
+                entry["verified"] = bool(ok and (detail["bit_exact_values_and_labels"] or d > 128))
                 entry["verification"] = detail
             (grid if k in ks else long_lists).append(entry)
             if d == 32 and k == 32 and not workspace:

@@ -123,9 +123,9 @@ __device__ __forceinline__ void cut_bf16x2(const float (&x)[8], vuint4& p1, vuin
 //   W <= V + FILTER_REL * Q        whenever V is finite,
 // and a pair can only have V < radius if W < radius + FILTER_REL * Q.  The compare is written so
 // that a NaN in W passes; FILTER_ABS covers products of pieces that underflow.
-// In 65 .. 128 dimensions (28 matrix instructions per tile, d + 2 <= 130 roundings in V) the three
-// terms are 7.8e-6, 4.7e-5 and 5.7e-5 of S: FILTER_REL_WIDE = 1.5 * 2^-13 (1.83e-4) leaves a factor
-// of 1.6, with NORM_LOWER_WIDE = 1.75 * 2^-12 >= 2 FILTER_REL_WIDE + 2^-15.3.
+// In 65 .. 128 dimensions (26 matrix instructions per tile, d + 2 <= 130 roundings in V) the three
+// terms are 7.8e-6, 4.7e-5 and 5.3e-5 of S: FILTER_REL_WIDE = 1.5 * 2^-13 (1.83e-4) leaves a factor
+// of 1.7, with NORM_LOWER_WIDE = 1.75 * 2^-12 >= 2 FILTER_REL_WIDE + 2^-15.3.
 constexpr float FILTER_REL = 0x1.0p-13F;
 constexpr float NORM_LOWER = 0x1.4p-12F;
 constexpr float FILTER_REL_WIDE = 0x1.8p-13F;
@@ -185,6 +185,10 @@ struct fused_geometry
     // groups are staged by eight waves)
     static constexpr int NORM_CELLS = DP == 128 && BIG ? 4 : (DP == 64 && BIG ? 2 : 1);
     static constexpr int CELLS = EXACT ? (DP <= 8 ? 3 : 2 * KS + NORM_CELLS) : 0;
+    // matrix instructions that add up the norm cells: one takes a cell in the first half of its 16
+    // inner dimensions (against ones there and zeros in the second half), or two cells, one in
+    // either half (against ones throughout)
+    static constexpr int NORM_TERMS = NORM_CELLS >= 2 ? NORM_CELLS / 2 : 1;
     static constexpr int PT = SPLIT   ? (DK <= 16 ? 128 : (DK <= 32 ? 64 : 32))
                               : EXACT ? (DP <= 16 ? 128 : (DP <= 32 ? 64 : (DP <= 64 ? 32 : 16))) * (BIG ? 2 : 1)
                               : WIDE  ? (DP <= 8 ? 128 : 64)
@@ -392,7 +396,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
                     val[j] = -2.0F * (half != 0 ? upper : lower);
                 }
                 cut_bf16x2(val, qs[0][kb], qs[1][kb]);
-                qs[2][kb] = half == 0 ? ones : zeros;
+                qs[2][kb] = half == 0 || G::NORM_CELLS >= 2 ? ones : zeros;
             }
         }
         else
@@ -424,7 +428,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
                     val[j] = -2.0F * (half != 0 ? upper : lower);
                 }
                 cut_bf16x2(val, qs[0][kb], qs[1][kb]);
-                qs[2][kb] = half == 0 ? ones : zeros;
+                qs[2][kb] = half == 0 || G::NORM_CELLS >= 2 ? ones : zeros;
             }
         }
         filter_slack = FILTER_REL_DP * qq * (1.0F + 0x1.0p-20F) + FILTER_ABS * (1.0F + qq);
@@ -1063,29 +1067,48 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
             else
             {
                 // the query comes from memory again, QC dimensions at a time, whose loads are all
-                // issued ahead of their arithmetic (zero beyond dim, as the point's rows are)
-                constexpr int QC = 16;
-                const float* const mine = a.queries + (my_q < a.q ? my_q : 0);
+                // issued ahead of their arithmetic (zero beyond dim, as the point's rows are; the
+                // dimensions from dim on add nothing to either sum and are left out).  The two
+                // halves of the wave have the same queries: of every 16 dimensions each half loads
+                // 8 and a swap of the halves hands them to the other.
+                constexpr int QC = 32;
+                const float* const mine =
+                    a.queries + (my_q < a.q ? my_q : 0) + static_cast<size_t>(8 * half) * static_cast<size_t>(a.q);
 #pragma unroll 1
-                for (int d0 = 0; d0 < DP; d0 += QC)
+                for (int d0 = 0; d0 < dim; d0 += QC)
                 {
                     float y[QC];
+                    float mine_of[QC / 2];
                     if (d0 + QC <= dim)
                     {
 #pragma unroll
-                        for (int j = 0; j < QC; ++j)
+                        for (int j = 0; j < QC / 2; ++j)
                         {
-                            y[j] = mine[static_cast<size_t>(d0 + j) * a.q];
+                            mine_of[j] = mine[static_cast<size_t>(d0 + 16 * (j / 8) + j % 8) * a.q];
                         }
                     }
                     else
                     {
 #pragma unroll
-                        for (int j = 0; j < QC; ++j)
+                        for (int j = 0; j < QC / 2; ++j)
                         {
-                            const float there = mine[static_cast<size_t>(d0 + j < dim ? d0 + j : 0) * a.q];
-                            y[j] = d0 + j < dim ? there : 0.0F;
+                            const int at = d0 + 16 * (j / 8) + j % 8; // (this lane's dimension: 8 * half more)
+                            const bool inside = at + 8 * half < dim;
+                            const float there = mine[static_cast<size_t>(inside ? at : 0) * a.q];
+                            mine_of[j] = inside ? there : 0.0F;
                         }
+                    }
+#pragma unroll
+                    for (int j = 0; j < QC / 2; ++j)
+                    {
+                        const u32 bits = __builtin_bit_cast(u32, mine_of[j]);
+                        const auto both = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+                        // (copied out before the cast: a cast of an element of a vector reads the
+                        // vector's first element with this compiler)
+                        const u32 of_first_half = both[0];
+                        const u32 of_second_half = both[1];
+                        y[16 * (j / 8) + j % 8] = __builtin_bit_cast(float, of_first_half);
+                        y[16 * (j / 8) + 8 + j % 8] = __builtin_bit_cast(float, of_second_half);
                     }
 #pragma unroll
                     for (int j = 0; j < QC; ++j)
@@ -1206,7 +1229,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
     u32 cut1[4] = {0, 0, 0, 0};
     u32 cut2[4] = {0, 0, 0, 0};
     u32 cut_norm = 0;
-    constexpr int NCELL = DP <= 8 ? 2 : 2 * KB + G::NORM_CELLS; // cells of a point that a lane reads
+    constexpr int NCELL = DP <= 8 ? 2 : 2 * KB + G::NORM_TERMS; // cells of a point that a lane reads
     // the tiles of a stage are multiplied in groups whose cells fit into 48 registers
     constexpr int TG = MT * NCELL <= 12 ? MT : (2 * NCELL <= 12 ? 2 : 1);
     // (the cells are read in the order in which the matrix instructions take them, the norm cell
@@ -1243,12 +1266,12 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
                 }
             }
 #pragma unroll
-            for (int c = 0; c < G::NORM_CELLS; ++c)
+            for (int c = 0; c < G::NORM_TERMS; ++c)
             {
 #pragma unroll
                 for (int t = 0; t < TG; ++t)
                 {
-                    cell[t][2 * KB + c] = mine[32 * t + (2 * KS + c) * PT];
+                    cell[t][2 * KB + c] = mine[32 * t + (2 * KS + (G::NORM_CELLS >= 2 ? 2 * c + half : c)) * PT];
                 }
             }
         }
@@ -1263,7 +1286,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
         {
             zero[r] = 0.0F;
         }
-        constexpr int TERMS = DP <= 8 ? 2 : 3 * KB + G::NORM_CELLS;
+        constexpr int TERMS = DP <= 8 ? 2 : 3 * KB + G::NORM_TERMS;
         constexpr int PAIRS_OF_VALUES = VPT / 2;
         constexpr int CHUNKS = MODE == 2 ? 0 : PAIRS_OF_VALUES + 1;
         static_assert(!EXACT || CHUNKS <= MT * TERMS, "a piece of the cutting per matrix instruction");
@@ -1299,11 +1322,11 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
         if constexpr (NCELL > 12)
         {
             // (one tile whose cells do not fit the registers at once: they are read in pairs -- the
-            // two cells of 16 dimensions that three matrix instructions take, then the norm cells --
-            // AHEAD pairs ahead of the instructions that take them)
+            // two cells of 16 dimensions that three matrix instructions take, then the two norm cells
+            // of this half of the wave -- AHEAD pairs ahead of the instructions that take them)
             static_assert(MT == 1 && G::SUB == 1 && G::NORM_CELLS == 4);
             constexpr int AHEAD = 2;
-            constexpr int PAIRS = KB + 2;
+            constexpr int PAIRS = KB + 1;
             const vuint4* const mine = reinterpret_cast<const vuint4*>(stage + DP * PT) + ql;
             vuint4 pair[AHEAD + 1][2];
             auto read_pair = [&](auto s_tag) __attribute__((always_inline)) {
@@ -1316,8 +1339,8 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
                 }
                 else if constexpr (at < PAIRS)
                 {
-                    pair[at % (AHEAD + 1)][0] = mine[(2 * KS + 2 * (at - KB)) * PT];
-                    pair[at % (AHEAD + 1)][1] = mine[(2 * KS + 2 * (at - KB) + 1) * PT];
+                    pair[at % (AHEAD + 1)][0] = mine[(2 * KS + half) * PT];
+                    pair[at % (AHEAD + 1)][1] = mine[(2 * KS + 2 + half) * PT];
                 }
             };
             static_for<0, AHEAD>([&](auto s_tag) { read_pair(s_tag); });
