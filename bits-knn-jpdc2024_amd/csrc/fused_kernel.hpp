@@ -1072,8 +1072,8 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
                 // halves of the wave have the same queries: of every 16 dimensions each half loads
                 // 8 and a swap of the halves hands them to the other.
                 constexpr int QC = 32;
-                const float* const mine =
-                    a.queries + (my_q < a.q ? my_q : 0) + static_cast<size_t>(8 * half) * static_cast<size_t>(a.q);
+                const float* const mine_first = a.queries + (my_q < a.q ? my_q : 0);
+                const float* const mine = mine_first + static_cast<size_t>(8 * half) * static_cast<size_t>(a.q);
 #pragma unroll 1
                 for (int d0 = 0; d0 < dim; d0 += QC)
                 {
@@ -1092,10 +1092,14 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
 #pragma unroll
                         for (int j = 0; j < QC / 2; ++j)
                         {
-                            const int at = d0 + 16 * (j / 8) + j % 8; // (this lane's dimension: 8 * half more)
-                            const bool inside = at + 8 * half < dim;
-                            const float there = mine[static_cast<size_t>(inside ? at : 0) * a.q];
-                            mine_of[j] = inside ? there : 0.0F;
+                            // (the first half's dimension `at`, the second half's at + 8: every
+                            // lane loads from a row that exists, by an index the wave shares)
+                            const int at = d0 + 16 * (j / 8) + j % 8;
+                            const bool first_inside = at < dim;
+                            const bool second_inside = at + 8 < dim;
+                            const float* const from = second_inside ? mine : mine_first;
+                            const float there = from[static_cast<size_t>(first_inside ? at : 0) * a.q];
+                            mine_of[j] = (half == 0 ? first_inside : second_inside) ? there : 0.0F;
                         }
                     }
 #pragma unroll
