@@ -182,7 +182,7 @@ struct fused_geometry
     // dimensions a point is three cells, (piece 1 | piece 2 | norm), used as the two halves of the
     // 16 matrix dimensions.
     // (one norm cell holds the shares of four groups of 8 dimensions: a second one where eight
-    // groups are staged by eight waves)
+    // groups are staged by eight waves, four for the sixteen groups of 128 dimensions)
     static constexpr int NORM_CELLS = DP == 128 && BIG ? 4 : (DP == 64 && BIG ? 2 : 1);
     static constexpr int CELLS = EXACT ? (DP <= 8 ? 3 : 2 * KS + NORM_CELLS) : 0;
     // matrix instructions that add up the norm cells: one takes a cell in the first half of its 16
@@ -346,6 +346,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
     // EXACT: two pieces; up to 8 dimensions qs[0][0] is piece 1 of dimensions 0 .. 7 in both halves
     // of the wave and qs[1][0] piece 2 in the first half, (1, 1, 0, ...) for the norm cell in the
     // second; from 16 dimensions on qs[2][0] is the norm cell's (1, 1, 0, ...) in the first half
+    // (ones in both halves where a point has two or four norm cells, which the halves take in pairs)
     vuint4 qs[SPLIT || EXACT ? 3 : 1][SPLIT || EXACT ? KB : 1];
     // EXACT: the query itself, every dimension, for the sequential arithmetic; the slack of its
     // filter threshold above the radius
