@@ -358,9 +358,9 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
     // Every list length has the shape (its LDS holds the ring of stages for all of them), but long
     // lists gain from it only where merges are not what the time goes into -- one range of points,
     // and the longer the list the more dimensions (65536 queries x 2^20 points, 128 -> 256 queries per
-    // workgroup: k = 64 d = 16 / 32 / 64 13.4 -> 10.8, 23.0 -> 17.1, 46.1 -> 30.9 ms; k = 128 d = 16 14.5 ->
-    // 15.4 but d = 32 / 64 25.0 -> 20.7, 51.4 -> 35.2 ms; k = 256 d = 32 28.4 -> 33.7 but d = 64 58.8 ->
-    // 48.5 ms; over ranges 8192 x 2^17, d = 32, k = 128: 1.23 -> 1.83 ms): the waves of the smaller
+    // workgroup: k = 64 d = 16 / 32 / 64 13.4 -> 10.8, 23.0 -> 17.1, 46.1 -> 28.6 ms; k = 128 d = 16 14.5 ->
+    // 15.4 but d = 32 / 64 25.0 -> 20.7, 51.4 -> 33.1 ms; k = 256 d = 32 28.4 -> 33.7 but d = 64 58.8 ->
+    // 47.4 ms; over ranges 8192 x 2^17, d = 32, k = 128: 1.23 -> 1.83 ms): the waves of the smaller
     // workgroups merge long lists together at a barrier, these each on its own.
     // (65 .. 128 dimensions have the exact arithmetic in this shape only)
     const bool has_big = arithmetic == BITSKNN_FUSED_EXACT && dim <= 128;
