@@ -258,7 +258,7 @@ def test_exact_arithmetic_is_bit_exact(bk, dev, oracle):
         assert np.array_equal(gd, ed) and np.array_equal(gl, el)
 
 
-@pytest.mark.parametrize("d", [5, 8, 16, 24, 32, 64])
+@pytest.mark.parametrize("d", [5, 8, 16, 24, 32, 64, 72, 100, 128])
 @pytest.mark.parametrize("kind", ["tiny", "huge", "signs", "near", "ranges-of-magnitude", "subnormal", "constant"])
 def test_the_filter_never_drops_a_neighbour(bk, dev, oracle, d, kind):
     """The filter of the default arithmetic promises a lower bound of every distance (bf16 pieces,
