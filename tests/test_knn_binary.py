@@ -200,6 +200,20 @@ def test_algorithms_agree_and_verify_is_silent():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("d", [72, 128])
+def test_fused_cache_in_wide_dimensions_agrees_with_the_cpu_path(d):
+    """65 to 128 dimensions take the reference's arithmetic in the fused kernel too: the driver's
+    run verifies against the CPU path and gives the same checksum of labels."""
+    base = ("-n", "32k", "-q", "300", "-d", str(d), "-k", "16", "--seed", "11")
+    cpu = run("-a", "parallel", *base)
+    assert cpu.returncode == 0, cpu.stderr
+    gpu = run("-a", "fused-cache", *base, "--items-per-thread", "8,4,2", "--block-size", "1", "-v", "parallel")
+    assert gpu.returncode == 0, gpu.stderr
+    assert "Difference" not in gpu.stderr, gpu.stderr[:2000]
+    assert checksums(gpu)[0] == checksums(cpu)[0]
+
+
+@pytest.mark.gpu
 def test_layouts_and_distance_runners():
     for alg in ("magma-dist", "magma-part-dist", "cublas-dist"):
         p = run("-a", alg, "-n", "8k", "-q", "128", "-d", "16", "-k", "4", "--seed", "5",
