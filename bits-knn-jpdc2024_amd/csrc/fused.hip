@@ -286,10 +286,6 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
         return fail(BITSKNN_ERR_UNSUPPORTED, "Dimension of vectors must not be lower than %d, but is %d",
                     dim_mult * dim_reg, dim);
     }
-    if (dim > 256)
-    {
-        return fail(BITSKNN_ERR_UNSUPPORTED, "Unsupported dimension: %d (at most 256)", dim);
-    }
     if (arithmetic != BITSKNN_FUSED_FP32 && arithmetic != BITSKNN_FUSED_BF16X3 && arithmetic != BITSKNN_FUSED_EXACT)
     {
         return fail(BITSKNN_ERR_INVALID, "bitsknn_fused_l2_topk_f32: unknown arithmetic %d", arithmetic);
@@ -423,6 +419,9 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
         scale = scale < SAMPLE_SCALE_RANGES_MIN ? SAMPLE_SCALE_RANGES_MIN
                                                 : (scale > SAMPLE_SCALE_RANGES_MAX ? SAMPLE_SCALE_RANGES_MAX : scale);
     }
+    // (more than 256 dimensions: the plain kernel of any_dim.hip, whatever the arithmetic asked for;
+    // it takes the ranges of points but neither first radii nor the other launch parameters)
+    const bool any_dim = dim > 256;
     bool sample = n >= SAMPLE_MIN_POINTS && k >= (splits == 1 ? SAMPLE_MIN_K : SAMPLE_MIN_K_RANGES);
     if (tuning != nullptr && tuning->first_radius != 0)
     {
@@ -430,6 +429,7 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
         sample = tuning->first_radius > 0 && n / tuning->first_radius >= 512;
         scale = sample ? tuning->first_radius : scale;
     }
+    sample = sample && !any_dim;
     const int rank = sample ? first_radius_rank(k, scale) : 0;
     if (rank > 0)
     {
@@ -445,7 +445,7 @@ int fused_impl(const float* queries_dim_major, const float* points_dim_major, in
         BITSKNN_HIP_CHECK(status);
         a.first_radius = FUSED_FIRST_RADIUS_FROM + rank - 1;
     }
-    status = launch_for_k(k, a, split, hip_stream);
+    status = any_dim ? launch_fused_any_dim(a, k, hip_stream) : launch_for_k(k, a, split, hip_stream);
     BITSKNN_HIP_CHECK(status);
     if (splits > 1)
     {

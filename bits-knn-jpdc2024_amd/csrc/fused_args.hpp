@@ -83,6 +83,9 @@ struct fused_args
 // the stage image of FUSED_ARITH_EXACT (stage_image.hip): its size for a point matrix of up to 64
 // dimensions (0 otherwise), and the launch that writes it
 size_t fused_image_bytes(int dim, int n);
+// more than 256 dimensions (any_dim.hip): a plain kernel in the reference's arithmetic, one query per
+// thread; takes the ranges of points of `a` (splits, split_points, list_stride), lists of k entries
+hipError_t launch_fused_any_dim(const fused_args& a, int k, hipStream_t stream);
 hipError_t launch_fused_image(const float* points, int dim, int n, void* image, hipStream_t stream);
 hipError_t launch_fused_k_4(const fused_args& a, int arith, hipStream_t stream);
 hipError_t launch_fused_k_8(const fused_args& a, int arith, hipStream_t stream);

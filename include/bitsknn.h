@@ -202,7 +202,10 @@ int bitsknn_dist_layout_f32(int op, int dim, size_t q, size_t n, const float* qu
  *                             over them measures the same kernel every time (what a sweep can
  *                             vary here: bitsknn_fused_l2_topk_f32_tuned)
  * The distances are computed in the reference's arithmetic (BITSKNN_FUSED_EXACT below) for
- * dim <= 128 and on the fp32 matrix instructions beyond.
+ * dim <= 128 and on the fp32 matrix instructions up to 256 dimensions.  More than 256 dimensions
+ * (the reference's kernel has only a lower bound on the dimension, fused_cache_knn.cu:63-67) are
+ * served by a plain kernel on the vector unit, one query per thread, again in the reference's
+ * arithmetic: correct and bit-identical, not tuned.
  * A call enqueues one to three kernels on `stream` (long lists over many points are preceded by a
  * pass over a sample of the points, which gives every query a first radius, and followed by one
  * that repeats the queries whose first radius proved too low); until the last of them has run,
@@ -260,14 +263,15 @@ int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major, const float* po
  *                         instructions (v_mfma_f32_32x32x16_bf16, two bf16 pieces per operand, three
  *                         products) whose value is a guaranteed lower bound of the distance less a
  *                         slack of 2^-13 ||q||^2 (1.5 * 2^-13 above 64 dimensions): no pair below a
- *                         query's current k-th distance is ever dropped.  Larger dimensions use
- *                         BITSKNN_FUSED_FP32.
+ *                         query's current k-th distance is ever dropped.  129 to 256 dimensions
+ *                         use BITSKNN_FUSED_FP32.
  *   BITSKNN_FUSED_FP32    every distance from fp32 matrix instructions (v_mfma_f32_32x32x2_f32):
  *                         within 1e-5 of the reference arithmetic, not bit-identical to it.
  *   BITSKNN_FUSED_BF16X3  for 9 <= dim <= 64: every fp32 operand is cut exactly into three bf16
  *                         pieces and a product is the fp32 sum of six bf16 products on the bf16
  *                         matrix path; what is left out is below 2^-23 of a product, the size of
  *                         one fp32 rounding.  Other dimensions use BITSKNN_FUSED_FP32.
+ *   (More than 256 dimensions: whatever the value, the plain kernel in the reference's arithmetic.)
  * The reference's fused kernel multiplies on the fp32 vector unit
  * (fused_cache_kernel_structs.cuh:457-522); the last two have no counterpart there.
  * BITSKNN_ERR_INVALID for another value of `arithmetic`.

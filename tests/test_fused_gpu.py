@@ -1,11 +1,11 @@
 """Parity of bits-fused (distance + top-k in one kernel, through the C ABI) with the CPU oracle.
 
-Up to 128 dimensions the plain entry points report distances computed with the reference's own
+Up to 128 dimensions, and above 256, the plain entry points report distances computed with the reference's own
 arithmetic (sequential fused multiply-adds over the dimensions in order, norm - 2 dot), found
 through a filter on the bf16 matrix instructions that is guaranteed never to drop a candidate:
 there the result must equal the oracle's BIT FOR BIT, values and labels, equal distances by lower
 index ("default" below).  With the distances taken from the fp32 matrix instructions ("mfma": every
-dimension above 128, and BITSKNN_FUSED_FP32 on request) or from bf16x3 products they are not
+dimension from 129 to 256, and BITSKNN_FUSED_FP32 on request up to 256 dimensions) or from bf16x3 products they are not
 bit-identical to the reference's; the bar there (the stated tolerance of this path) is the k-th
 neighbour distance within 1e-5 relative of the oracle's -- of the completed distance
 (value + ||q||^2) for dim >= 16, of the reported partial distance below that, see tests/parity.py --
@@ -61,7 +61,7 @@ def _arith(bk, mode):
 
 def _bits(mode, dim):
     """whether the result of this mode must equal the oracle's bit for bit"""
-    return mode in ("default", "image", "big") and dim <= 128
+    return (mode in ("default", "image", "big") and dim <= 128) or dim > 256
 
 
 def _check(oracle, points, queries, k, gd, gl, min_recall=0.999, bar_dim=None, bits=False):
@@ -130,7 +130,7 @@ def test_all_k_values(bk, dev, oracle, k, d, mode):
 
 
 @pytest.mark.parametrize("mode", MODES_AND_IMAGE)
-@pytest.mark.parametrize("d", [1, 2, 3, 5, 7, 9, 15, 17, 31, 33, 48, 49, 63, 64, 65, 100, 113, 200, 256])
+@pytest.mark.parametrize("d", [1, 2, 3, 5, 7, 9, 15, 17, 31, 33, 48, 49, 63, 64, 65, 100, 113, 200, 256, 257, 300, 520])
 def test_dimensions(bk, dev, oracle, d, mode):
     p, s = oracle.generate(d, 3000, 70, d)
     gd, gl = _fused(bk, dev, p, s, 16, (2, 4, 1), 1, 1, arithmetic=_arith(bk, mode))
@@ -377,6 +377,20 @@ def test_point_matrix_of_2_gib_takes_the_plain_loads(bk, dev, oracle, k, d):
         assert np.array_equal(fl[:first].cpu().numpy(), el)
 
 
+@pytest.mark.parametrize("n,q,d,k,workspace,mode", [(5000, 130, 300, 32, None, "default"), (20000, 300, 512, 16, None, "default"),
+                                                    (3000, 70, 1000, 4, None, "default"), (25, 7, 260, 16, None, "default"),
+                                                    (10, 300, 290, 128, None, "default"), (9000, 150, 384, 256, None, "default"),
+                                                    (5000, 130, 300, 64, None, "mfma"), (5000, 130, 300, 8, None, "bf16x3"),
+                                                    (70001, 300, 300, 16, "auto", "default"),
+                                                    (131072, 100, 257, 128, "auto", "default")])
+def test_more_than_256_dimensions(bk, dev, oracle, n, q, d, k, workspace, mode):
+    """Above 256 dimensions every arithmetic takes the plain kernel with one query per thread, in the
+    reference's arithmetic: bit for bit against the oracle, with and without ranges of points."""
+    p, s = oracle.generate(n + d + k, n, q, d)
+    gd, gl = _fused(bk, dev, p, s, k, arithmetic=_arith(bk, mode), workspace=workspace)
+    _check(oracle, p, s, k, gd, gl, bits=True)
+
+
 @pytest.mark.parametrize("k", [128, 256])
 def test_long_lists_stay_in_the_fused_kernel(bk, dev, oracle, k):
     """k >= 128: the workspace the library asks for holds partial lists only (never the q x n
@@ -460,7 +474,7 @@ def test_random_shapes_against_the_oracle(bk, dev, oracle, mode):
     and a workspace that only holds partial lists."""
     import torch
     rng = np.random.default_rng(77)
-    dims = [1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 24, 31, 32, 33, 40, 63, 64, 65, 100, 128, 129, 200, 256]
+    dims = [1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 24, 31, 32, 33, 40, 63, 64, 65, 100, 128, 129, 200, 256, 257, 300, 511]
     for case in range(40):
         d = int(rng.choice(dims))
         k = int(rng.choice([4, 8, 16, 32, 64, 128, 256]))

@@ -200,10 +200,11 @@ def test_algorithms_agree_and_verify_is_silent():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("d", [72, 128])
+@pytest.mark.parametrize("d", [72, 128, 300])
 def test_fused_cache_in_wide_dimensions_agrees_with_the_cpu_path(d):
-    """65 to 128 dimensions take the reference's arithmetic in the fused kernel too: the driver's
-    run verifies against the CPU path and gives the same checksum of labels."""
+    """65 to 128 dimensions take the reference's arithmetic in the fused kernel too, and so does the
+    plain kernel of more than 256: the driver's run verifies against the CPU path and gives the same
+    checksum of labels."""
     base = ("-n", "32k", "-q", "300", "-d", str(d), "-k", "16", "--seed", "11")
     cpu = run("-a", "parallel", *base)
     assert cpu.returncode == 0, cpu.stderr
