@@ -13,9 +13,10 @@
 // in the matrix kernels) in tiles of 16 points, 32 dimensions at a time: the tile's values go
 // through LDS, where every thread reads them as broadcasts, its own query's 32 values come from
 // global memory into registers.  The list of a query lives in the caller's output arrays
-// (fused_args::out_dist / out_label, k entries): unordered while the points are visited, with the
-// position of its largest entry kept in a register -- a point that is nearer replaces that entry
-// and the list is scanned for its new largest one -- and sorted by its thread at the end.
+// (fused_args::out_dist / out_label, k entries): unordered while the points are visited, with its
+// AD_TOP largest entries (keys, labels, positions) kept in registers.  A point that is nearer than
+// the largest one replaces it and either joins those registers or leaves one entry fewer in them;
+// only when they are used up is the list scanned again.  Its thread sorts the list at the end.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -32,6 +33,7 @@ namespace
 constexpr int AD_THREADS = 256; // queries per workgroup
 constexpr int AD_POINTS = 16;   // points per tile
 constexpr int AD_DIMS = 32;     // dimensions per step
+constexpr int AD_TOP = 8;       // largest entries of a list that its thread keeps track of
 constexpr std::int32_t AD_NO_LABEL = 0x7FFFFFFF;
 
 typedef float vfloat4 __attribute__((ext_vector_type(4)));
@@ -64,9 +66,44 @@ __global__ void __launch_bounds__(AD_THREADS) fused_any_dim_kernel(const fused_a
             list_l[i] = AD_NO_LABEL;
         }
     }
-    int fill = 0;                           // entries of the list that hold a point
-    int largest = 0;                        // where the largest entry is, once the list is full
-    float radius = __builtin_inff();        // its key
+    int fill = 0;                    // entries of the list that hold a point
+    // the `tracked` largest entries of the full list, largest first (by key, then label); the
+    // others are not above the last of them
+    float top_key[AD_TOP];
+    std::int32_t top_label[AD_TOP];
+    int top_at[AD_TOP];
+    int tracked = 0;
+#pragma unroll
+    for (int j = 0; j < AD_TOP; ++j)
+    {
+        top_key[j] = -__builtin_inff();
+        top_label[j] = -1;
+        top_at[j] = 0;
+    }
+    // (key, label) of an entry above that of another
+    auto above = [](float key, std::int32_t label, float other, std::int32_t other_label) -> bool {
+        return key > other || (key == other && label > other_label);
+    };
+    // puts an entry into the tracked ones where it belongs (the last one falls out if all are in use)
+    auto track = [&](float key, std::int32_t label, int at) {
+#pragma unroll
+        for (int j = 0; j < AD_TOP; ++j)
+        {
+            const bool here = j < tracked ? above(key, label, top_key[j], top_label[j]) : true;
+            if (here)
+            {
+                const float was_key = top_key[j];
+                const std::int32_t was_label = top_label[j];
+                const int was_at = top_at[j];
+                top_key[j] = key;
+                top_label[j] = label;
+                top_at[j] = at;
+                key = was_key;
+                label = was_label;
+                at = was_at;
+            }
+        }
+    };
     // the staging of a tile: thread t carries point t % 16 in dimensions t / 16 and t / 16 + 16 of a step
     const int sp = t % AD_POINTS;
     const int sc = t / AD_POINTS;
@@ -142,29 +179,59 @@ __global__ void __launch_bounds__(AD_THREADS) fused_any_dim_kernel(const fused_a
                     continue;
                 }
             }
-            else if (key < radius)
+            else if (key < top_key[0])
             {
                 // (labels come in ascending order: of equal distances the earlier point stays)
-                list_d[largest] = value;
-                list_l[largest] = label;
+                const int at = top_at[0];
+                list_d[at] = value;
+                list_l[at] = label;
+                // the largest entry is gone: the others move up
+#pragma unroll
+                for (int j = 0; j + 1 < AD_TOP; ++j)
+                {
+                    top_key[j] = top_key[j + 1];
+                    top_label[j] = top_label[j + 1];
+                    top_at[j] = top_at[j + 1];
+                }
+                --tracked;
+                // the new entry is one of the tracked ones if it is above the last of them (everything
+                // that is not tracked is not above that one)
+                if (tracked > 0)
+                {
+                    bool joins = false;
+#pragma unroll
+                    for (int j = 0; j < AD_TOP; ++j)
+                    {
+                        joins = joins || (j == tracked - 1 && above(key, label, top_key[j], top_label[j]));
+                    }
+                    if (joins)
+                    {
+                        track(key, label, at);
+                        ++tracked;
+                    }
+                    continue;
+                }
             }
             else
             {
                 continue;
             }
-            // the largest entry of the full list, of equal ones the one with the highest label
-            radius = order_key(list_d[0]);
-            largest = 0;
-            std::int32_t largest_label = list_l[0];
-            for (int i = 1; i < k; ++i)
+            // the list is full and nothing is tracked: its AD_TOP largest entries (all of a shorter list)
+            tracked = 0;
+            for (int i = 0; i < k; ++i)
             {
                 const float there = order_key(list_d[i]);
                 const std::int32_t its_label = list_l[i];
-                if (there > radius || (there == radius && its_label > largest_label))
+                bool in = tracked < AD_TOP;
+#pragma unroll
+                for (int jj = 0; jj < AD_TOP; ++jj)
                 {
-                    radius = there;
-                    largest = i;
-                    largest_label = its_label;
+                    in = in || (jj == AD_TOP - 1 && above(there, its_label, top_key[jj], top_label[jj]));
+                }
+                if (in)
+                {
+                    track(there, its_label, i);
+                    tracked = tracked < AD_TOP ? tracked + 1 : AD_TOP;
                 }
             }
         }

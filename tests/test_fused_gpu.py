@@ -391,6 +391,21 @@ def test_more_than_256_dimensions(bk, dev, oracle, n, q, d, k, workspace, mode):
     _check(oracle, p, s, k, gd, gl, bits=True)
 
 
+@pytest.mark.parametrize("k", [4, 32, 128])
+def test_more_than_256_dimensions_with_equal_distances(bk, dev, oracle, k):
+    """Many copies of few points: equal distances are reported by lower index, and lists whose largest
+    entries tie are kept right (the plain kernel tracks the largest entries of a list in registers)."""
+    rng = np.random.default_rng(k)
+    n, q, d = 4000, 90, 270
+    few = rng.random((12, d), dtype=np.float32)
+    p = np.ascontiguousarray(few[rng.integers(0, 12, size=n)])
+    p[::7] = rng.random((len(p[::7]), d), dtype=np.float32)
+    s = rng.random((q, d), dtype=np.float32)
+    for workspace in (None, "auto"):
+        gd, gl = _fused(bk, dev, p, s, k, workspace=workspace)
+        _check(oracle, p, s, k, gd, gl, bits=True)
+
+
 @pytest.mark.parametrize("k", [128, 256])
 def test_long_lists_stay_in_the_fused_kernel(bk, dev, oracle, k):
     """k >= 128: the workspace the library asks for holds partial lists only (never the q x n
