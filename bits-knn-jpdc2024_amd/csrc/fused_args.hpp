@@ -26,6 +26,9 @@ constexpr int FQ_CAP = 32;                    // buffer slots per query (= point
 constexpr int FUSED_ARITH_MFMA_F32 = 0;
 constexpr int FUSED_ARITH_BF16X3 = 1;
 constexpr int FUSED_ARITH_EXACT = 2;
+// (kernel-internal, 129 .. 256 dimensions of FUSED_ARITH_EXACT: the fp32 matrix instructions, on norms
+// lowered by the error budget, are the filter; what passes is computed and appended as above)
+constexpr int FUSED_ARITH_EXACT_F32 = 3;
 
 constexpr int FUSED_PLAIN = -1;
 constexpr int FUSED_REPEAT_MARKED = -2;

@@ -16,7 +16,8 @@ namespace bitsknn
 // FUSED_ARITH_BF16X3: dimensions 9 .. 64 (below 9 the fp32 matrix instructions are as fast);
 // FUSED_ARITH_EXACT: dimensions up to 128 (a stage holds the points twice, as fp32 rows and as bf16
 // pieces; 65 .. 128 dimensions only in workgroups of 256 queries, whatever fused_args::workgroup
-// says); everything else takes the fp32 matrix instructions
+// says; 129 .. 256 with the fp32 matrix instructions as the filter); everything else takes the fp32
+// matrix instructions
 hipError_t BITSKNN_CAT_EXPANDED(launch_fused_k_, BITSKNN_FUSED_K)(const fused_args& a, int arith,
                                                                   hipStream_t stream)
 {
@@ -37,6 +38,11 @@ hipError_t BITSKNN_CAT_EXPANDED(launch_fused_k_, BITSKNN_FUSED_K)(const fused_ar
     if (arith == FUSED_ARITH_EXACT && a.dim <= 128)
     {
         return launch_fused_as<K, 128, FUSED_ARITH_EXACT, false, true>(a, stream);
+    }
+    if (arith == FUSED_ARITH_EXACT)
+    {
+        // 129 .. 256 dimensions: the fp32 matrix instructions as the filter
+        return launch_fused<K, 256, FUSED_ARITH_EXACT_F32>(a, stream);
     }
     if (a.dim <= 8)
     {

@@ -126,6 +126,10 @@ __device__ __forceinline__ void cut_bf16x2(const float (&x)[8], vuint4& p1, vuin
 // In 65 .. 128 dimensions (26 matrix instructions per tile, d + 2 <= 130 roundings in V) the three
 // terms are 7.8e-6, 4.7e-5 and 5.3e-5 of S: FILTER_REL_WIDE = 1.5 * 2^-13 (1.83e-4) leaves a factor
 // of 1.7, with NORM_LOWER_WIDE = 1.75 * 2^-12 >= 2 FILTER_REL_WIDE + 2^-15.3.
+// In 129 .. 256 dimensions (FUSED_ARITH_EXACT_F32) W comes from v_mfma_f32_32x32x2_f32 on the plain
+// values and on norm shares lowered by NORM_LOWER: at most 258 accumulations of 2^-23 each (3.1e-5 S),
+// the shares' own sums (64 * 2^-24 N) and the d + 2 <= 258 roundings of V (1.5e-5 S), 5e-5 S together
+// against FILTER_REL = 2^-13 (1.22e-4).
 constexpr float FILTER_REL = 0x1.0p-13F;
 constexpr float NORM_LOWER = 0x1.4p-12F;
 constexpr float FILTER_REL_WIDE = 0x1.8p-13F;
@@ -283,6 +287,11 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
     constexpr int FQ_QB = G::QB;
     constexpr bool SPLIT = G::SPLIT;
     constexpr bool EXACT = G::EXACT;
+    // 129 .. 256 dimensions of the default arithmetic: stages, matrix instructions and loops of the
+    // fp32 kernel, whose values (on lowered norms) only filter; lists as with EXACT
+    constexpr bool VIA_F32 = ARITH == FUSED_ARITH_EXACT_F32;
+    constexpr bool EXACT_LISTS = EXACT || VIA_F32;
+    static_assert(!VIA_F32 || (G::MT == 1 && !G::RING && !G::PAIRED), "one tile per stage, two stages, a norm row per staging thread");
     constexpr int PT = G::PT;
     constexpr int CAP = G::CAP;
     constexpr int SLOTS = G::SLOTS;
@@ -473,6 +482,19 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
             }
             qf[s] = val;
         }
+        if constexpr (VIA_F32)
+        {
+            // ||q||^2 from the fragments (-2 q; a lane has every other dimension)
+            float qq = 0.0F;
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+            {
+                const float half_of = 2 * s + half < DP ? -0.5F * qf[s] : 0.0F;
+                qq = __builtin_fmaf(half_of, half_of, qq);
+            }
+            qq += __builtin_bit_cast(float, lane_xor32<32>(__builtin_bit_cast(u32, qq)));
+            filter_slack = FILTER_REL * qq * (1.0F + 0x1.0p-20F) + FILTER_ABS * (1.0F + qq);
+        }
     }
 
     // rows that never change in any stage: padding dimensions, unused norm rows
@@ -513,7 +535,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
     // tile (40000 queries x 2^20 points: 560 ms instead of 9).
     const bool live_query = my_q < a.q;
     float radius = live_query ? first_radius : -__builtin_inff(); // k-th smallest distance of my query so far
-    if constexpr (EXACT)
+    if constexpr (EXACT_LISTS)
     {
         // (a first radius from a sample gives the filter its threshold from the first tile on)
         thr = live_query ? radius + (filter_slack + 0x1.0p-22F * __builtin_fabsf(radius)) : -__builtin_inff();
@@ -643,7 +665,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
                 if (i == K - 1)
                 {
                     wx[qm] = key_value(list[r]);
-                    if constexpr (EXACT)
+                    if constexpr (EXACT_LISTS)
                     {
                         reinterpret_cast<int*>(wx)[64 + qm] = key_label(list[r]);
                     }
@@ -655,7 +677,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         // (a first radius from a sample stays until the list has a smaller one)
         radius = live_query ? fminf(wx[ql], first_radius) : -__builtin_inff();
-        if constexpr (EXACT)
+        if constexpr (EXACT_LISTS)
         {
             // (the slack also covers the rounding of this sum)
             thr = live_query ? radius + (filter_slack + 0x1.0p-22F * __builtin_fabsf(radius)) : -__builtin_inff();
@@ -1023,6 +1045,11 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
             }
             else
             {
+                if constexpr (VIA_F32)
+                {
+                    // (the filter's norm: lowered by the error budget, as the bf16 filter's is)
+                    share = __builtin_fmaf(-NORM_LOWER, share, share);
+                }
                 stage[(DP + sd0) * PT + sp] = base + sp < n ? share : __builtin_inff();
             }
         }
@@ -1064,6 +1091,36 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
                     norm = __builtin_fmaf(x, x, norm);
                     dot = __builtin_fmaf(qx[dd], x, dot);
                 }
+            }
+            else if constexpr (VIA_F32)
+            {
+                // the query from the fragments of the matrix instructions (-2 q, halved exactly): a
+                // lane has every other dimension, the lane of the other half of the wave, which
+                // has the same query, the ones in between
+                static_for<0, DP / 32>([&](auto c_tag) {
+                    constexpr int c = decltype(c_tag)::value;
+                    if (32 * c < dim)
+                    {
+#pragma unroll
+                        for (int s = 16 * c; s < 16 * c + 16; ++s)
+                        {
+                            const u32 bits = __builtin_bit_cast(u32, qf[s]);
+                            const auto both = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+                            // (copied out before the cast: a cast of an element of a vector reads
+                            // the vector's first element with this compiler)
+                            const u32 of_first_half = both[0];
+                            const u32 of_second_half = both[1];
+                            const float even = -0.5F * __builtin_bit_cast(float, of_first_half);
+                            const float odd = -0.5F * __builtin_bit_cast(float, of_second_half);
+                            const float x0 = column[(2 * s) * PT];
+                            const float x1 = column[(2 * s + 1) * PT];
+                            norm = __builtin_fmaf(x0, x0, norm);
+                            dot = __builtin_fmaf(even, x0, dot);
+                            norm = __builtin_fmaf(x1, x1, norm);
+                            dot = __builtin_fmaf(odd, x1, dot);
+                        }
+                    }
+                });
             }
             else
             {
@@ -1701,7 +1758,19 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
             {
                 acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(arow[2 * s * PT], qf[s], acc0, 0, 0, 0);
             }
-            filter_tile(acc0, base);
+            if constexpr (VIA_F32)
+            {
+                // the tile's values are lower bounds (less the slack in thr): what is not above the
+                // threshold is computed in the reference's arithmetic
+                if (__builtin_amdgcn_ballot_w64(!(smallest_of(acc0) > thr)) != 0)
+                {
+                    exact_candidates(static_cast<u64>(bits_of(acc0)), stage, base);
+                }
+            }
+            else
+            {
+                filter_tile(acc0, base);
+            }
         }
     };
 

@@ -201,11 +201,10 @@ int bitsknn_dist_layout_f32(int op, int dim, size_t q, size_t n, const float* qu
  *                             vector unit and do not change the matrix-core kernel, so a sweep
  *                             over them measures the same kernel every time (what a sweep can
  *                             vary here: bitsknn_fused_l2_topk_f32_tuned)
- * The distances are computed in the reference's arithmetic (BITSKNN_FUSED_EXACT below) for
- * dim <= 128 and on the fp32 matrix instructions up to 256 dimensions.  More than 256 dimensions
- * (the reference's kernel has only a lower bound on the dimension, fused_cache_knn.cu:63-67) are
- * served by a plain kernel on the vector unit, one query per thread, again in the reference's
- * arithmetic: correct and bit-identical, not tuned.
+ * The distances are computed in the reference's arithmetic (BITSKNN_FUSED_EXACT below) in every
+ * dimension.  More than 256 dimensions (the reference's kernel has only a lower bound on the
+ * dimension, fused_cache_knn.cu:63-67) are served by a plain kernel on the vector unit, one query
+ * per thread: correct and bit-identical, not tuned.
  * A call enqueues one to three kernels on `stream` (long lists over many points are preceded by a
  * pass over a sample of the points, which gives every query a first radius, and followed by one
  * that repeats the queries whose first radius proved too low); until the last of them has run,
@@ -253,7 +252,7 @@ int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major, const float* po
  * bits-fused with the arithmetic of the products q.p chosen per call (nothing process-wide is
  * read); workspace may be NULL (then as bitsknn_fused_l2_topk_f32) or as for
  * bitsknn_fused_l2_topk_f32_ws.
- *   BITSKNN_FUSED_EXACT   what the entry points above use.  For dim <= 128 every reported distance
+ *   BITSKNN_FUSED_EXACT   what the entry points above use.  Every reported distance
  *                         is computed as the reference's kernel computes it -- norm and dot
  *                         product by sequential fused multiply-adds over the dimensions in order,
  *                         then norm - 2 dot (include/bits/topk/singlepass/
@@ -263,8 +262,10 @@ int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major, const float* po
  *                         instructions (v_mfma_f32_32x32x16_bf16, two bf16 pieces per operand, three
  *                         products) whose value is a guaranteed lower bound of the distance less a
  *                         slack of 2^-13 ||q||^2 (1.5 * 2^-13 above 64 dimensions): no pair below a
- *                         query's current k-th distance is ever dropped.  129 to 256 dimensions
- *                         use BITSKNN_FUSED_FP32.
+ *                         query's current k-th distance is ever dropped.  In 129 to 256
+ *                         dimensions the fp32 matrix instructions (on norms lowered by the same
+ *                         budget) are that filter: 1.2 to 3 times the time of BITSKNN_FUSED_FP32
+ *                         there, which callers who do not need the reference's bits can ask for.
  *   BITSKNN_FUSED_FP32    every distance from fp32 matrix instructions (v_mfma_f32_32x32x2_f32):
  *                         within 1e-5 of the reference arithmetic, not bit-identical to it.
  *   BITSKNN_FUSED_BF16X3  for 9 <= dim <= 64: every fp32 operand is cut exactly into three bf16

@@ -210,7 +210,7 @@ def _check_neighbours(oracle, points_dm, queries_dm, sample, got_d, got_l, k, wh
 # fp32 matrix instructions to the tolerance.
 @pytest.mark.parametrize("d,k,mode", [(8, 4, "default"), (16, 16, "default"), (32, 32, "default"),
                                       (8, 32, "default"), (32, 4, "default"), (32, 32, "mfma"), (8, 4, "mfma"),
-                                      (64, 32, "default"), (100, 16, "default"), (128, 32, "default")])
+                                      (64, 32, "default"), (100, 16, "default"), (128, 32, "default"), (192, 16, "default")])
 def test_fused_at_full_size(bk, dev, oracle, d, k, mode):
     import torch
     q, n = 65536, 1 << 20
