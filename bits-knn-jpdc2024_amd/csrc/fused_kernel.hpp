@@ -248,10 +248,13 @@ struct fused_geometry
     // long lists over ranges want the waves merging together: 8192 queries x 2^17 points, d = 8,
     // k = 128 1.10 -> 1.46 ms on the ring.)
     // (The workgroups of 256 queries have the LDS of a whole compute unit: the ring for every list
-    // length, with buffers of 20 to 32 slots.)
+    // length, with buffers of 20 to 32 slots.  So has the exact arithmetic of 129 .. 256 dimensions,
+    // one workgroup of four waves per compute unit, whose candidates differ most from wave to wave:
+    // 65536 queries x 2^20 points, d = 256, k = 32: 452 -> 376 ms against the two stages with a barrier.)
     static constexpr bool RING =
         !WIDE && (SPLIT ? K <= FQ_CAP
-                        : BIG || (DP <= 8 && K <= 128) || (DP >= 16 && DP <= RING_MAX_DP && K <= FQ_CAP));
+                        : BIG || ARITH == FUSED_ARITH_EXACT_F32 || (DP <= 8 && K <= 128) ||
+                              (DP >= 16 && DP <= RING_MAX_DP && K <= FQ_CAP));
     static constexpr int NB = RING ? 3 : 2;
     // slots a query buffer has in LDS (20 where the three stages of 256 points in 16 dimensions leave
     // no more room next to the buffers of 256 queries)
@@ -291,7 +294,7 @@ __global__ void __launch_bounds__((fused_geometry<DP, ARITH, K, WIDE_OK, BIG_OK>
     // fp32 kernel, whose values (on lowered norms) only filter; lists as with EXACT
     constexpr bool VIA_F32 = ARITH == FUSED_ARITH_EXACT_F32;
     constexpr bool EXACT_LISTS = EXACT || VIA_F32;
-    static_assert(!VIA_F32 || (G::MT == 1 && !G::RING && !G::PAIRED), "one tile per stage, two stages, a norm row per staging thread");
+    static_assert(!VIA_F32 || (G::MT == 1 && !G::PAIRED), "one tile per stage, a norm row per staging thread");
     constexpr int PT = G::PT;
     constexpr int CAP = G::CAP;
     constexpr int SLOTS = G::SLOTS;

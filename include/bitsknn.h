@@ -264,7 +264,7 @@ int bitsknn_fused_l2_topk_f32_ws(const float* queries_dim_major, const float* po
  *                         slack of 2^-13 ||q||^2 (1.5 * 2^-13 above 64 dimensions): no pair below a
  *                         query's current k-th distance is ever dropped.  In 129 to 256
  *                         dimensions the fp32 matrix instructions (on norms lowered by the same
- *                         budget) are that filter: 1.2 to 3 times the time of BITSKNN_FUSED_FP32
+ *                         budget) are that filter: 1 to 3 times the time of BITSKNN_FUSED_FP32
  *                         there, which callers who do not need the reference's bits can ask for.
  *   BITSKNN_FUSED_FP32    every distance from fp32 matrix instructions (v_mfma_f32_32x32x2_f32):
  *                         within 1e-5 of the reference arithmetic, not bit-identical to it.
