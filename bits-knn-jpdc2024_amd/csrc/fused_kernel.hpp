@@ -158,7 +158,7 @@ constexpr u32 BF16_HUGE = 0x7F7FU;
 // n = 2^17, d = 8: 4.4 -> 2.7 ms at k = 256 and 1.7 -> 1.3 ms at k = 128 before the first radii from
 // a sample; at k = 64 the smaller stages cost more than the merges save).  WIDE_OK is set for
 // launches over ranges only (see launch_fused).
-constexpr int RING_MAX_DP = 128; // largest padded dimension that takes the ring of stages
+constexpr int RING_MAX_DP = 256; // largest padded dimension that takes the ring of stages
 constexpr int FQ_XCHG = 96;      // words a wave has for the exchange at a merge: 32 radii, fills, labels
 
 template <int DP, int ARITH, int K, bool WIDE_OK = false, bool BIG_OK = false>
@@ -238,7 +238,9 @@ struct fused_geometry
     //    gain 2-3 % at k = 64 on many queries but lose 4-8 % (k = 64) and 26 % (k = 128) over
     //    ranges of points, where merges of long lists are what the time goes into.  (65536 queries x 2^20
     //    points, k = 32: d = 16 20.4 -> 19.9 ms, d = 32 38.5 -> 37.5 ms, d = 64 75.4 -> 73.0 ms,
-    //    d = 128 138.7 -> 137.9 ms.)
+    //    d = 128 138.7 -> 137.9 ms.)  In 256 dimensions, where a compute unit holds one workgroup
+    //    anyway (registers), three stages of 33 KB: d = 256, k = 32 304 -> 283 ms; with longer lists
+    //    it gains 4 % on many queries but loses a third over ranges (k = 256, 8192 x 2^17: 7.2 -> 9.9 ms).
     //  * the stages of the bf16 pieces have 12.5 KB in every dimension: three fit as they are.
     //    Lists of up to 32 entries (65536 queries x 2^20 points, k = 32: d = 16 14.0 -> 13.8 ms,
     //    d = 64 51.2 -> 47.0 ms; 8192 queries x 2^17 points over ranges: d = 16 0.78 -> 0.68 ms,
