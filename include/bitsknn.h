@@ -296,7 +296,8 @@ int bitsknn_fused_l2_topk_f32_ex(const float* queries_dim_major, const float* po
  *                 BITSKNN_FUSED_EXACT)
  *   ranges        how many ranges the points are cut into (separate workgroups per range, partial
  *                 lists of 8*q*ranges*k bytes in the workspace, one bits pass at the end); 0 = the
- *                 library's choice (enough workgroups for two per compute unit, at most 64); fewer
+ *                 library's choice (enough workgroups for two per compute unit -- one in 129 to
+ *                 256 dimensions of BITSKNN_FUSED_EXACT, where a unit holds one --, at most 64); fewer
  *                 are used when the workspace is smaller or the ranges would fall below 256 points
  *   first_radius  whether the lists start from radii taken from a launch over a sample of the points
  *                 (one stage in every first_radius, 2 .. 4096; -1: never; 0: the library's choice,
