@@ -384,8 +384,18 @@ def fused_roofline(q, n, d, seconds):
     its filter (executed flops, padding included) against the bf16 peak; next to it the
     algorithmic 2*q*n*d flops of the distance over the time, and what fraction of the fp32 matrix
     peak that is (above 1: the contraction does not run on the fp32 unit)."""
-    executed = filter_flops_per_pair(d) * q * n / seconds / 1e12
     algorithmic = 2.0 * q * n * d / seconds / 1e12
+    if d > 128:
+        # 129 .. 256 dimensions: the filter runs on the fp32 matrix instructions (256 dimensions and
+        # four norm rows per pair); above 256 a vector-unit kernel, priced by its algorithmic flops
+        flops = 2.0 * (256 + 4) if d <= 256 else 2.0 * d
+        executed = flops * q * n / seconds / 1e12
+        return {"bound": "mfma", "achieved": executed, "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": executed / MFMA_F32_PEAK_TFLOPS,
+                "matrix_instructions": ("v_mfma_f32_32x32x2_f32, %d flops per pair executed" % flops) if d <= 256
+                else "none (vector unit), priced against the fp32 matrix peak",
+                "algorithmic_tflops": algorithmic, "algorithmic_over_fp32_matrix_peak": algorithmic / MFMA_F32_PEAK_TFLOPS}
+    executed = filter_flops_per_pair(d) * q * n / seconds / 1e12
     return {"bound": "mfma", "achieved": executed, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": executed / MFMA_BF16_PEAK_TFLOPS,
             "matrix_instructions": "v_mfma_f32_32x32x16_bf16, %d flops per pair executed" % filter_flops_per_pair(d),
