@@ -141,7 +141,7 @@ def test_dimensions(bk, dev, oracle, d, mode):
 @pytest.mark.parametrize("mode", MODES_AND_IMAGE)
 @pytest.mark.parametrize("n,q", [(1, 1), (31, 5), (32, 33), (33, 127), (255, 128), (257, 129), (1000, 300), (5001, 1)])
 def test_ragged_counts(bk, dev, oracle, n, q, mode):
-    for d in (8, 24, 72):
+    for d in (8, 24, 72, 200):
         p, s = oracle.generate(n + q + d, n, q, d)
         for k in (4, 32):
             gd, gl = _fused(bk, dev, p, s, k, arithmetic=_arith(bk, mode))
@@ -152,7 +152,7 @@ def test_ragged_counts(bk, dev, oracle, n, q, mode):
 # / 32 for 32 / 64 / 128; the exact arithmetic and bf16x3: 128 up to 16 dimensions, 64 / 32 for 32 / 64
 # (the exact arithmetic in workgroups of 256 queries: twice that, and 32 in 65 .. 128 dimensions,
 # which have this shape only)
-@pytest.mark.parametrize("d", [8, 16, 32, 64, 100])
+@pytest.mark.parametrize("d", [8, 16, 32, 64, 100, 200])
 @pytest.mark.parametrize("mode", ["default", "mfma", "bf16x3", "image", "big"])
 def test_point_counts_around_whole_stages(bk, dev, oracle, d, mode):
     # one to five stages, each count one short of, at and one past a whole stage: the ring of three
@@ -162,9 +162,9 @@ def test_point_counts_around_whole_stages(bk, dev, oracle, d, mode):
     if mode == "image" and d > 64:
         pytest.skip("the stage image serves up to 64 dimensions")
     if mode == "big":
-        stage = {8: 256, 16: 256, 32: 128, 64: 64, 100: 32}[d]
+        stage = {8: 256, 16: 256, 32: 128, 64: 64, 100: 32, 200: 32}[d]
     elif mode == "mfma" or d > 64:
-        stage = {8: 256, 16: 256, 32: 128, 64: 64, 100: 32}[d]
+        stage = {8: 256, 16: 256, 32: 128, 64: 64, 100: 32, 200: 32}[d]
     else:
         stage = {8: 128, 16: 128, 32: 64, 64: 32}[d]
     q = 130
